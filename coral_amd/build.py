@@ -1,0 +1,61 @@
+"""Build recipe for libcoral_search.so (HIP kernels + C ABI + host-side C++).
+
+Everything is compiled for gfx950 only.  `python -m coral_amd.build` rebuilds
+in-tree; the shared library lands in coral_amd/lib/ and is what the Python
+binding, the tests, the CLI and the benchmark load.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIBDIR, "libcoral_search.so")
+CLI = os.path.join(LIBDIR, "test_search_pipeline")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+          "-Wall", "-Wno-unused-result"]
+# packed fp32 code generation is switched off for all device code
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+LIB_SOURCES = ["beam_search.hip", "coral_search.cpp", "formats.cpp", "index_gpu.cpp"]
+CLI_SOURCES = ["test_search_pipeline.cpp"]
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if out.strip():
+        print(out, flush=True)
+    if r.returncode != 0:
+        raise RuntimeError("build step failed: " + " ".join(cmd))
+
+
+def build(verbose=True):
+    os.makedirs(LIBDIR, exist_ok=True)
+    objs = []
+    for src in LIB_SOURCES:
+        path = os.path.join(CSRC, src)
+        if not os.path.exists(path):
+            continue
+        obj = os.path.join(LIBDIR, src + ".o")
+        cmd = [HIPCC] + COMMON + ["-fopenmp", "-fvisibility=hidden", "-DCORAL_BUILD"]
+        cmd += DEVICE if src.endswith(".hip") else ["-x", "hip"] + DEVICE
+        _run(cmd + ["-c", path, "-o", obj])
+        objs.append(obj)
+    _run([HIPCC, "-shared", "-fopenmp", "-o", LIB] + objs)
+    for src in CLI_SOURCES:
+        path = os.path.join(CSRC, src)
+        if os.path.exists(path):
+            _run([HIPCC] + COMMON + ["-x", "hip"] + DEVICE + [path, "-o", CLI, "-L" + LIBDIR, "-lcoral_search",
+                  "-Wl,-rpath,$ORIGIN"])
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    print("built", LIB)

@@ -1,0 +1,162 @@
+"""ctypes binding of libcoral_search.so (include/coral_search.h).
+
+Loading fails loudly when the library has not been built: there is no Python or
+CPU fallback for the search path.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libcoral_search.so")
+
+L2, IP = 0, 1
+POLICY_ROUNDS, POLICY_BEST_FIRST = 0, 1
+
+OK, ERR_ARG, ERR_GRAPH, ERR_DEVICE, ERR_MEMORY, ERR_IO, ERR_STATE = range(7)
+
+
+class CoralError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("coral status %d: %s" % (code, msg))
+        self.code = code
+
+
+class IndexDesc(C.Structure):
+    _fields_ = [("base", C.c_void_p), ("nbrs", C.c_void_p), ("n", C.c_int64), ("dim", C.c_int32),
+                ("R", C.c_int32), ("start_ids", C.c_void_p), ("n_start", C.c_int32),
+                ("metric", C.c_int32), ("device", C.c_int32)]
+
+
+class Stats(C.Structure):
+    _fields_ = [("time_s", C.c_double), ("hops", C.c_int64), ("expansions", C.c_int64),
+                ("dist_evals", C.c_int64), ("rounds", C.c_int64), ("spills", C.c_int64)]
+
+    def as_dict(self):
+        return {f: getattr(self, f) for f, _ in self._fields_}
+
+
+class Tuning(C.Structure):
+    _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
+                ("reserved", C.c_int32 * 5)]
+
+
+_lib = None
+
+# name -> (restype, argtypes); also the list of symbols the header declares
+SIGNATURES = {
+    "coral_last_error": (C.c_char_p, []),
+    "coral_index_create": (C.c_int, [C.POINTER(IndexDesc), C.POINTER(C.c_void_p)]),
+    "coral_index_destroy": (None, [C.c_void_p]),
+    "coral_index_set_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
+    "coral_index_set_deleted": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "coral_index_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32),
+                                   C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "coral_search_prepare": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(Tuning)]),
+    "coral_search_gpu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                   C.c_int32, C.c_int32, C.c_void_p, C.POINTER(Stats)]),
+    "coral_search_query_counters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
+    "coral_search": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                               C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(Stats)]),
+    "coral_search_verify": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                      C.POINTER(C.c_int64)]),
+}
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("%s is missing: build it with `python -m coral_amd.build`" % LIB_PATH)
+        _lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(_lib, name)
+            fn.restype, fn.argtypes = res, args
+        from . import formats  # registers the format entry points on the same handle
+        formats.register(_lib)
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise CoralError(rc, lib().coral_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+class Index:
+    """An HBM-resident index (vectors + compact graph rows + start ids)."""
+
+    def __init__(self, base, nbrs, start_ids, metric=L2, device=0):
+        base = np.ascontiguousarray(base, dtype=np.float32)
+        nbrs = np.ascontiguousarray(nbrs, dtype=np.int32)
+        start_ids = np.ascontiguousarray(start_ids, dtype=np.int32)
+        if base.ndim != 2 or nbrs.ndim != 2 or nbrs.shape[0] != base.shape[0]:
+            raise ValueError("base must be [n,dim] and nbrs [n,R]")
+        d = IndexDesc(_ptr(base), _ptr(nbrs), base.shape[0], base.shape[1], nbrs.shape[1], _ptr(start_ids),
+                      start_ids.size, metric, device)
+        h = C.c_void_p()
+        _check(lib().coral_index_create(C.byref(d), C.byref(h)))
+        self._h = h
+        self.n, self.dim, self.R, self.metric = base.shape[0], base.shape[1], nbrs.shape[1], metric
+        self.n_start = int(start_ids.size)
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().coral_index_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def set_graph(self, nbrs, start_ids):
+        nbrs = np.ascontiguousarray(nbrs, dtype=np.int32)
+        start_ids = np.ascontiguousarray(start_ids, dtype=np.int32)
+        if nbrs.shape != (self.n, self.R):
+            raise ValueError("nbrs must be [n,R]")
+        _check(lib().coral_index_set_graph(self._h, _ptr(nbrs), _ptr(start_ids), start_ids.size))
+        self.n_start = int(start_ids.size)
+
+    def set_deleted(self, mask_words):
+        if mask_words is None:
+            _check(lib().coral_index_set_deleted(self._h, None))
+            return
+        m = np.ascontiguousarray(mask_words, dtype=np.uint32)
+        if m.size != (self.n + 31) // 32:
+            raise ValueError("mask must hold ceil(n/32) words")
+        _check(lib().coral_index_set_deleted(self._h, _ptr(m)))
+
+    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0):
+        t = Tuning(visited_slots_log2, workgroups, threads)
+        _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
+
+    def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):
+        """Host buffers in and out (the IndexGPU::Search shape)."""
+        q = np.ascontiguousarray(queries, dtype=np.float32)
+        Q = q.shape[0]
+        ids = np.empty((Q, k), dtype=np.int32)
+        dists = np.empty((Q, k), dtype=np.float32) if want_dists else None
+        st = Stats()
+        _check(lib().coral_search(self._h, _ptr(q), Q, k, L, policy, int(have_delete), _ptr(ids), _ptr(dists),
+                                  C.byref(st)))
+        return ids, dists, st
+
+    def search_device(self, d_queries, d_ids, d_dists, Q, k, policy=POLICY_ROUNDS, have_delete=False,
+                      stream=None):
+        """Device pointers (ints) in and out (the GPUFuncs::search_gpu shape)."""
+        st = Stats()
+        _check(lib().coral_search_gpu(self._h, d_queries, d_ids, d_dists, Q, k, policy, int(have_delete),
+                                      stream, C.byref(st)))
+        return st
+
+    def query_counters(self, Q):
+        out = np.empty((Q, 4), dtype=np.int32)
+        _check(lib().coral_search_query_counters(self._h, _ptr(out), Q))
+        return out
+
+    def verify(self, d_ids_res, d_ids_gt, Q, k):
+        hits = C.c_int64()
+        _check(lib().coral_search_verify(self._h, d_ids_res, d_ids_gt, Q, k, C.byref(hits)))
+        return hits.value

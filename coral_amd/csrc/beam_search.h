@@ -1,0 +1,42 @@
+// beam_search.h -- kernel argument block and host-side launchers shared by
+// beam_search.hip (device code) and coral_search.cpp (the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace coral {
+
+// Everything the search kernel reads, passed by value like the reference passes
+// its BP block (include/uni.h:323-354).
+struct SearchArgs {
+    const float* vec;          // [n][dim]
+    const int32_t* nbrs;       // [n][R], -1 padded
+    const int32_t* start_ids;  // [M]
+    const uint32_t* deleted;   // tombstone mask or nullptr
+    const float* queries;      // [Q][dim]
+    int32_t* ids_out;          // [Q][k]
+    float* dists_out;          // [Q][k] or nullptr
+    int32_t* counters;         // [Q][4]: hops, expansions, dist_evals, rounds
+    uint32_t* spill;           // [workgroups][spill_words] zeroed bitmaps
+    int* next_qid;             // work counter, zero at launch
+    int* spill_count;          // queries that left LDS, zero at launch
+    size_t spill_words;        // ceil(n/32)
+    int64_t n;
+    int32_t dim, R, M, Q, k, L;
+    int32_t metric;            // 0 = L2, 1 = IP
+    int32_t policy;            // 0 = rounds, 1 = best first
+    int32_t slots_log2;        // LDS visited table size
+    int32_t vis_limit;         // inserts after which the table is frozen
+    int32_t tcap, ccap;        // LDS todo / candidate capacities (multiples of 4, ccap >= tcap)
+};
+
+size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap);
+hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu);
+hipError_t launch_search(const SearchArgs& a, int workgroups, int threads, size_t lds_bytes,
+                         hipStream_t stream);
+hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,
+                         hipStream_t stream);
+hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t stream);
+
+}  // namespace coral

@@ -1,0 +1,522 @@
+// beam_search.hip -- batched graph beam search for gfx950 (MI355X), one
+// workgroup per in-flight query, persistent workgroups pulling query ids from a
+// device counter.
+//
+// What it computes is the search of the reference's CUDA kernel
+// (src/search_gpu.cu:347-580, tombstone variant :582-833) and, with
+// policy == CORAL_POLICY_BEST_FIRST, of its CPU path (src/search_in_cpu.cpp:63-108).
+// How it computes it is specific to this GPU:
+//   * per query the sorted beam (64-bit keys), the exact visited set (open
+//     addressing, 32-bit ids), the candidate buffer and the query live in LDS;
+//     the reference keeps beam scratch and an N-bit visited bitmap per block in
+//     global memory and clears the bitmap for every query (:388);
+//   * a graph row is 32 int32 = one 128-byte line, read by half a wavefront;
+//   * a vector row is read as float4 by a group of 16/32/64 lanes, eight rows in
+//     flight per wave, and reduced across lanes (the reference lets one thread
+//     walk a whole row, include/utils.cuh:254-275);
+//   * candidates are bitonic-sorted and merged into the beam by rank; the
+//     reference replaces the current worst entry one candidate at a time (:530-570).
+//
+// Distance summation order (mirrored bit for bit by the test oracle): lane l of a
+// group of G lanes accumulates float4 chunks l, l+G, ... with four fused
+// multiply-adds per chunk in x,y,z,w order; partials are combined by a butterfly
+// p[l] += p[l^off], off = G/2..1.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "beam_search.h"
+
+namespace coral {
+
+constexpr uint32_t kEmpty = 0xFFFFFFFFu;
+constexpr uint64_t kKeyMax = ~0ull;
+
+// float -> uint32 whose unsigned order is the float order
+__device__ __forceinline__ uint32_t ord32(float s) {
+    const uint32_t u = __float_as_uint(s);
+    return u ^ ((uint32_t)((int32_t)u >> 31) | 0x80000000u);
+}
+__device__ __forceinline__ float unord32(uint32_t o) {
+    const uint32_t u = (o & 0x80000000u) ? (o ^ 0x80000000u) : ~o;
+    return __uint_as_float(u);
+}
+// key order = (signed distance, id, expanded flag)
+__device__ __forceinline__ uint64_t make_key(float s, int32_t id, uint32_t flag) {
+    return ((uint64_t)ord32(s) << 32) | ((uint64_t)((uint32_t)id << 1)) | flag;
+}
+__device__ __forceinline__ int32_t key_id(uint64_t k) { return (int32_t)((uint32_t)k >> 1); }
+__device__ __forceinline__ float key_s(uint64_t k) { return unord32((uint32_t)(k >> 32)); }
+
+__device__ __forceinline__ uint32_t hash_slot(uint32_t id, int shift) {
+    return (id * 0x9E3779B1u) >> shift;
+}
+
+// 1 if id was not in the table (and is now), 0 if it was there
+__device__ __forceinline__ int visit_lds(uint32_t* table, uint32_t mask, int shift, uint32_t id) {
+    uint32_t h = hash_slot(id, shift);
+    for (;;) {
+        const uint32_t x = table[h];
+        if (x == id) return 0;
+        if (x == kEmpty) {
+            const uint32_t old = atomicCAS(&table[h], kEmpty, id);
+            if (old == kEmpty) return 1;
+            if (old == id) return 0;
+        }
+        h = (h + 1) & mask;
+    }
+}
+
+// after the LDS table stopped taking inserts: look it up, then test-and-set the
+// workgroup's bitmap in global memory
+__device__ __forceinline__ int visit_spill(const uint32_t* table, uint32_t mask, int shift,
+                                           uint32_t* bitmap, uint32_t id) {
+    uint32_t h = hash_slot(id, shift);
+    for (;;) {
+        const uint32_t x = table[h];
+        if (x == id) return 0;
+        if (x == kEmpty) break;
+        h = (h + 1) & mask;
+    }
+    const uint32_t bit = 1u << (id & 31);
+    const uint32_t old = atomicOr(&bitmap[id >> 5], bit);
+    return (old & bit) == 0;
+}
+
+// number of set bits of m below the calling lane
+__device__ __forceinline__ int prefix_popc(uint64_t m) {
+    const uint32_t lane = threadIdx.x & 63;
+    return __popcll(m & ((1ull << lane) - 1ull));
+}
+
+__device__ __forceinline__ int lower_bound_u64(const uint64_t* a, int n, uint64_t key) {
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (a[mid] < key)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+struct WgState {
+    int nb;           // beam entries
+    int cur;          // which LDS beam buffer is current
+    uint64_t live;    // key of the worst entry of a full beam, else kKeyMax
+};
+
+template <int G, int CPL>
+__global__ __launch_bounds__(512) void beam_search_kernel(const SearchArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, NT = blockDim.x;
+    const int lane = tid & 63, wave = tid >> 6, NW = NT >> 6;
+    const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2;
+    const int Lp = (L + 3) & ~3;
+    const int slots = 1 << a.slots_log2;
+    const uint32_t hmask = (uint32_t)slots - 1u;
+    const int hshift = 32 - a.slots_log2;
+    const int TCAP = a.tcap, CCAP = a.ccap;
+
+    uint64_t* beam0 = (uint64_t*)smem;
+    uint64_t* beam1 = beam0 + Lp;
+    uint64_t* cand = beam1 + Lp;
+    uint32_t* table = (uint32_t*)(cand + CCAP);
+    uint32_t* todo = table + slots;
+    uint32_t* elist = todo + TCAP;
+    float* qs = (float*)(elist + Lp);
+
+    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_ne, s_first, s_outpos;
+
+    uint32_t* bitmap = a.spill + (size_t)blockIdx.x * a.spill_words;
+
+    constexpr int GPW = 64 / G;                    // row groups per wave
+    constexpr int U = (CPL >= 8) ? 1 : (8 / CPL);  // rows in flight per group
+    constexpr int RPI = GPW * U;                   // rows per wave iteration
+    const int gl = lane & (G - 1), grp = lane / G;
+
+    for (;;) {
+        __syncthreads();
+        if (tid == 0) s_qid = atomicAdd(a.next_qid, 1);
+        __syncthreads();
+        const int qid = s_qid;
+        if (qid >= a.Q) break;
+
+        for (int i = tid; i < slots; i += NT) table[i] = kEmpty;
+        for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
+        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_ne = 0;
+        __syncthreads();
+
+        float4 qreg[CPL];
+#pragma unroll
+        for (int t = 0; t < CPL; ++t) {
+            const int c = gl + G * t;
+            qreg[t] = c < chunks ? reinterpret_cast<const float4*>(qs)[c] : make_float4(0, 0, 0, 0);
+        }
+
+        WgState st;
+        st.nb = 0, st.cur = 0, st.live = kKeyMax;
+        float thr = 3.402823466e+38f;  // signed form of the farthest sentinel
+        int hops = 0, nd = 0, rounds = 0;
+        bool spill = false;
+
+        // ---- distance phase: todo[0..T) -> cand[], counting passes of the frozen threshold
+        auto distance_phase = [&](int T) {
+            int cntf = 0;
+            for (int base = wave * RPI; base < T; base += NW * RPI) {
+                int vid[U];
+                float4 v[U][CPL];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int r = base + grp * U + u;
+                    vid[u] = r < T ? (int)todo[r] : -1;
+                    const float4* row =
+                        reinterpret_cast<const float4*>(a.vec + (size_t)(vid[u] < 0 ? 0 : vid[u]) * dim);
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        const int c = gl + G * t;
+                        v[u][t] = (vid[u] >= 0 && c < chunks) ? row[c] : make_float4(0, 0, 0, 0);
+                    }
+                }
+                float acc[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    float s = 0.0f;
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        if (a.metric == 0) {
+                            float d;
+                            d = qreg[t].x - v[u][t].x, s = __fmaf_rn(d, d, s);
+                            d = qreg[t].y - v[u][t].y, s = __fmaf_rn(d, d, s);
+                            d = qreg[t].z - v[u][t].z, s = __fmaf_rn(d, d, s);
+                            d = qreg[t].w - v[u][t].w, s = __fmaf_rn(d, d, s);
+                        } else {
+                            s = __fmaf_rn(qreg[t].x, v[u][t].x, s);
+                            s = __fmaf_rn(qreg[t].y, v[u][t].y, s);
+                            s = __fmaf_rn(qreg[t].z, v[u][t].z, s);
+                            s = __fmaf_rn(qreg[t].w, v[u][t].w, s);
+                        }
+                    }
+                    acc[u] = s;
+                }
+#pragma unroll
+                for (int off = G / 2; off > 0; off >>= 1) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) acc[u] = acc[u] + __shfl_xor(acc[u], off, 64);
+                }
+                float mine = acc[0];
+                int myid = vid[0];
+#pragma unroll
+                for (int u = 1; u < U; ++u)
+                    if (gl == u) mine = acc[u], myid = vid[u];
+                const bool valid = gl < U && myid >= 0;
+                const float s = a.metric == 0 ? mine : 0.0f - mine;
+                const bool pf = valid && (s < thr);
+                const uint64_t key = make_key(s, myid, 0u);
+                const bool app = pf && key < st.live;
+                cntf += __popcll(__ballot(pf));
+                const uint64_t m = __ballot(app);
+                if (m) {
+                    int pos = 0;
+                    if (lane == 0) pos = atomicAdd(&s_ncand, __popcll(m));
+                    pos = __shfl(pos, 0, 64);
+                    if (app) cand[pos + prefix_popc(m)] = key;
+                }
+            }
+            if (lane == 0 && cntf) atomicAdd(&s_cntf, cntf);
+        };
+
+        // ---- merge cand[0..s_ncand) into the beam (all threads; barriers inside)
+        auto merge = [&]() {
+            __syncthreads();
+            const int nc = s_ncand;
+            if (nc == 0) return;
+            int P = 2;
+            while (P < nc) P <<= 1;
+            for (int i = nc + tid; i < P; i += NT) cand[i] = kKeyMax;
+            __syncthreads();
+            for (int k2 = 2; k2 <= P; k2 <<= 1) {
+                for (int j = k2 >> 1; j > 0; j >>= 1) {
+                    for (int t = tid; t < (P >> 1); t += NT) {
+                        const int i = 2 * t - (t & (j - 1));
+                        const int x = i + j;
+                        const bool asc = (i & k2) == 0;
+                        const uint64_t ka = cand[i], kb = cand[x];
+                        if ((ka > kb) == asc) cand[i] = kb, cand[x] = ka;
+                    }
+                    __syncthreads();
+                }
+            }
+            const uint64_t* src = st.cur ? beam1 : beam0;
+            uint64_t* dst = st.cur ? beam0 : beam1;
+            const int nb = st.nb;
+            for (int i = tid; i < nb; i += NT) {
+                const uint64_t key = src[i];
+                const int pos = i + lower_bound_u64(cand, nc, key);
+                if (pos < L) dst[pos] = key;
+            }
+            for (int j = tid; j < nc; j += NT) {
+                const uint64_t key = cand[j];
+                const int pos = j + lower_bound_u64(src, nb, key);
+                if (pos < L) dst[pos] = key;
+            }
+            __syncthreads();
+            st.nb = min(L, nb + nc);
+            st.cur ^= 1;
+            st.live = st.nb == L ? dst[L - 1] : kKeyMax;
+            if (tid == 0) s_ncand = 0;
+            __syncthreads();
+        };
+
+        // ---- seeds: every start id is visited and measured, none counts as a hop
+        const int M = a.M;
+        for (int i = tid; i < M; i += NT) {
+            const uint32_t id = (uint32_t)a.start_ids[i];
+            visit_lds(table, hmask, hshift, id);
+            todo[i] = id;
+        }
+        __syncthreads();
+        distance_phase(M);
+        merge();
+        if (tid == 0) s_nvis = M, s_cntf = 0;
+        nd = M;
+        if (a.policy == 1) hops = M;
+
+        // ---- rounds
+        for (;;) {
+            uint64_t* beam = st.cur ? beam1 : beam0;
+            const int nb0 = st.nb;
+            if (tid == 0) s_nexp = 0, s_first = 0x7fffffff;
+            __syncthreads();
+            if (a.policy == 0) {
+                for (int i0 = 0; i0 < nb0; i0 += NT) {
+                    const int i = i0 + tid;
+                    uint64_t key = 0;
+                    bool un = false;
+                    if (i < nb0) key = beam[i], un = (key & 1ull) == 0;
+                    const uint64_t m = __ballot(un);
+                    if (m) {
+                        int pos = 0;
+                        if (lane == 0) pos = atomicAdd(&s_nexp, __popcll(m));
+                        pos = __shfl(pos, 0, 64);
+                        if (un) {
+                            elist[pos + prefix_popc(m)] = (uint32_t)key_id(key);
+                            beam[i] = key | 1ull;
+                        }
+                    }
+                }
+            } else {
+                for (int i0 = 0; i0 < nb0; i0 += NT) {
+                    const int i = i0 + tid;
+                    const bool un = i < nb0 && (beam[i] & 1ull) == 0;
+                    const uint64_t m = __ballot(un);
+                    if (m && lane == 0) atomicMin(&s_first, i0 + wave * 64 + (__ffsll((long long)m) - 1));
+                }
+                __syncthreads();
+                if (tid == 0 && s_first < nb0) {
+                    const uint64_t key = beam[s_first];
+                    elist[0] = (uint32_t)key_id(key);
+                    beam[s_first] = key | 1ull;
+                    s_nexp = 1;
+                }
+            }
+            __syncthreads();
+            const int nexp = s_nexp;
+            if (nexp == 0) break;
+
+            const int ech = TCAP / R;  // beam entries whose rows fit the todo list
+            for (int e0 = 0; e0 < nexp; e0 += ech) {
+                const int ecount = min(ech, nexp - e0);
+                if (!spill && s_nvis > a.vis_limit) spill = true;
+                if (tid == 0) s_ntodo = 0;
+                __syncthreads();
+                const int total = ecount * R;
+                for (int f0 = 0; f0 < total; f0 += NT) {
+                    const int f = f0 + tid;
+                    int v = -1;
+                    bool head = false;
+                    if (f < total) {
+                        const int e = f / R, j = f - e * R;
+                        v = a.nbrs[(size_t)elist[e0 + e] * R + j];
+                        head = j == 0;
+                    }
+                    bool isnew = false;
+                    if (v >= 0)
+                        isnew = spill ? visit_spill(table, hmask, hshift, bitmap, (uint32_t)v)
+                                      : visit_lds(table, hmask, hshift, (uint32_t)v);
+                    const uint64_t mh = __ballot(head);
+                    const uint64_t m = __ballot(isnew);
+                    if (lane == 0 && mh) atomicAdd(&s_ne, __popcll(mh));
+                    if (m) {
+                        int pos = 0;
+                        if (lane == 0) pos = atomicAdd(&s_ntodo, __popcll(m));
+                        pos = __shfl(pos, 0, 64);
+                        if (isnew) todo[pos + prefix_popc(m)] = (uint32_t)v;
+                    }
+                }
+                __syncthreads();
+                const int T = s_ntodo;
+                nd += T;
+                if (s_ncand + T > CCAP) merge();  // merge() starts and ends with a barrier
+                if (tid == 0) s_nvis += T;
+                distance_phase(T);
+                __syncthreads();
+            }
+            ++rounds;
+            const int cntf = s_cntf;
+            if (a.policy == 0) {
+                if (cntf == 0) break;
+                hops += cntf;
+            } else {
+                hops += 1;
+            }
+            merge();
+            if (tid == 0) s_cntf = 0;
+            if (a.policy == 0 && nb0 + cntf > L) thr = key_s((st.cur ? beam1 : beam0)[L - 1]);
+        }
+
+        // ---- output: the k closest live entries, closest first
+        {
+            __syncthreads();
+            const uint64_t* beam = st.cur ? beam1 : beam0;
+            int32_t* ids_out = a.ids_out + (size_t)qid * a.k;
+            float* dists_out = a.dists_out ? a.dists_out + (size_t)qid * a.k : nullptr;
+            if (tid == 0) s_outpos = 0;
+            __syncthreads();
+            for (int i0 = 0; i0 < st.nb; i0 += NT) {
+                const int i = i0 + tid;
+                uint64_t key = 0;
+                bool livee = false;
+                if (i < st.nb) {
+                    key = beam[i];
+                    livee = true;
+                    if (a.deleted) {
+                        const int32_t id = key_id(key);
+                        livee = ((a.deleted[id >> 5] >> (id & 31)) & 1u) == 0;
+                    }
+                }
+                // ordered compaction: waves take their turn through s_outpos
+                const uint64_t m = __ballot(livee);
+                for (int w = 0; w < NW; ++w) {
+                    if (w == wave) {
+                        const int basepos = s_outpos;
+                        const int pos = basepos + prefix_popc(m);
+                        if (livee && pos < a.k) {
+                            ids_out[pos] = key_id(key);
+                            if (dists_out) {
+                                const float s = key_s(key);
+                                dists_out[pos] = a.metric == 0 ? s : 0.0f - s;
+                            }
+                        }
+                        if (lane == 0) s_outpos = basepos + __popcll(m);
+                    }
+                    __syncthreads();
+                }
+                if (s_outpos >= a.k) break;
+            }
+            __syncthreads();
+            for (int i = s_outpos + tid; i < a.k; i += NT) {
+                ids_out[i] = -1;
+                if (dists_out) dists_out[i] = a.metric == 0 ? 3.402823466e+38f : -3.402823466e+38f;
+            }
+            if (tid == 0) {
+                int32_t* c = a.counters + (size_t)qid * 4;
+                c[0] = hops, c[1] = s_ne, c[2] = nd, c[3] = rounds;
+                if (spill) atomicAdd(a.spill_count, 1);
+            }
+            if (spill) {
+                for (size_t i = tid; i < a.spill_words; i += NT) bitmap[i] = 0u;
+            }
+        }
+    }
+}
+
+// hits = sum_q |res[q][0..k) n gt[q][0..k)| (src/search_gpu.cu:888-907)
+__global__ void ids_verify_kernel(const int32_t* __restrict__ res, const int32_t* __restrict__ gt,
+                                  unsigned long long* hit, int Q, int k) {
+    __shared__ int s_hit;
+    for (int q = blockIdx.x; q < Q; q += gridDim.x) {
+        if (threadIdx.x == 0) s_hit = 0;
+        __syncthreads();
+        const int32_t* g = gt + (size_t)q * k;
+        int mine = 0;
+        for (int i = threadIdx.x; i < k; i += blockDim.x) {
+            const int32_t id = res[(size_t)q * k + i];
+            for (int j = 0; j < k; ++j)
+                if (g[j] == id) {
+                    ++mine;
+                    break;
+                }
+        }
+        if (mine) atomicAdd(&s_hit, mine);
+        __syncthreads();
+        if (threadIdx.x == 0 && s_hit) atomicAdd(hit, (unsigned long long)s_hit);
+        __syncthreads();
+    }
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, size_t n, uint32_t v) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * blockDim.x)
+        p[i] = v;
+}
+
+// ------------------------------------------------------------------ launchers
+
+typedef void (*kernel_fn)(const SearchArgs);
+
+static kernel_fn pick_kernel(int dim) {
+    const int chunks = dim / 4;
+    if (chunks <= 16) return beam_search_kernel<16, 1>;
+    if (chunks <= 32) return beam_search_kernel<32, 1>;
+    if (chunks <= 64) return beam_search_kernel<64, 1>;
+    if (chunks <= 128) return beam_search_kernel<64, 2>;
+    if (chunks <= 256) return beam_search_kernel<64, 4>;
+    if (chunks <= 512) return beam_search_kernel<64, 8>;
+    return nullptr;
+}
+
+size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap) {
+    const size_t Lp = (size_t)((L + 3) & ~3);
+    return Lp * 8 * 2 + (size_t)ccap * 8 + ((size_t)4 << slots_log2) + (size_t)tcap * 4 + Lp * 4 +
+           (size_t)((dim + 3) & ~3) * 4;
+}
+
+hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu) {
+    kernel_fn fn = pick_kernel(dim);
+    if (!fn) return hipErrorInvalidValue;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    int nb = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, reinterpret_cast<const void*>(fn), threads,
+                                                     lds_bytes);
+    if (e != hipSuccess) return e;
+    *max_wg_per_cu = nb;
+    return hipSuccess;
+}
+
+hipError_t launch_search(const SearchArgs& a, int workgroups, int threads, size_t lds_bytes,
+                         hipStream_t stream) {
+    kernel_fn fn = pick_kernel(a.dim);
+    if (!fn) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fn, dim3(workgroups), dim3(threads), lds_bytes, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,
+                         hipStream_t stream) {
+    hipLaunchKernelGGL(ids_verify_kernel, dim3(Q < 1024 ? Q : 1024), dim3(64), 0, stream, res, gt, hit,
+                       Q, k);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, n, v);
+    return hipGetLastError();
+}
+
+}  // namespace coral

@@ -1,0 +1,430 @@
+// coral_search.cpp -- the C ABI of include/coral_search.h over the HIP kernels of
+// beam_search.hip.  Host code only; every device allocation of the search path
+// is made here.  There is no CPU fallback: without a usable HIP device every
+// entry point that needs one fails with CORAL_ERR_DEVICE.
+#include "coral_search.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "beam_search.h"
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                       \
+    do {                                                                                    \
+        hipError_t e_ = (expr);                                                             \
+        if (e_ != hipSuccess)                                                               \
+            return fail(e_ == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE,    \
+                        "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__,    \
+                        __LINE__);                                                          \
+    } while (0)
+
+constexpr int kMaxL = 2048;
+constexpr int kMaxLdsBytes = 160 * 1024;
+
+}  // namespace
+
+struct coral_index {
+    int device = 0;
+    int64_t n = 0;
+    int dim = 0, R = 0, M = 0, metric = 0;
+    float* d_vec = nullptr;
+    int32_t* d_nbrs = nullptr;
+    int32_t* d_start = nullptr;
+    uint32_t* d_deleted = nullptr;
+    hipStream_t stream = nullptr;
+    int num_cu = 0;
+
+    // state of search_prepare
+    bool prepared = false;
+    int Q = 0, L = 0;
+    int slots_log2 = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 256, workgroups = 0;
+    size_t lds_bytes = 0;
+    size_t spill_words = 0;
+    uint32_t* d_spill = nullptr;
+    size_t spill_alloc_words = 0;
+    int32_t* d_counters = nullptr;
+    size_t counters_alloc = 0;
+    int* d_scalars = nullptr;  // [0] next_qid, [1] spill_count
+    unsigned long long* d_hit = nullptr;
+    int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
+    int last_Q = 0;
+};
+
+extern "C" {
+
+const char* coral_last_error(void) { return g_err.c_str(); }
+
+static int validate_graph(const int32_t* nbrs, int64_t n, int R, const int32_t* start_ids,
+                          int n_start) {
+    if (n_start <= 0 || !start_ids) return fail(CORAL_ERR_ARG, "no start ids");
+    for (int i = 0; i < n_start; ++i) {
+        if (start_ids[i] < 0 || start_ids[i] >= n)
+            return fail(CORAL_ERR_GRAPH, "start id %d out of range [0,%lld)", start_ids[i],
+                        (long long)n);
+        for (int j = 0; j < i; ++j)
+            if (start_ids[i] == start_ids[j])
+                return fail(CORAL_ERR_GRAPH, "duplicate start id %d", start_ids[i]);
+    }
+    int64_t bad_node = -1;
+    int bad_kind = 0;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) {
+        const int32_t* row = nbrs + i * R;
+        bool ended = false;
+        for (int j = 0; j < R; ++j) {
+            const int32_t v = row[j];
+            if (v < 0) {
+                ended = true;
+            } else if (ended || v >= n) {
+#pragma omp critical
+                if (bad_node < 0) bad_node = i, bad_kind = ended ? 1 : 2;
+            }
+        }
+    }
+    if (bad_node >= 0)
+        return fail(CORAL_ERR_GRAPH,
+                    bad_kind == 1 ? "node %lld: neighbour after the end-of-row marker"
+                                  : "node %lld: neighbour id out of range",
+                    (long long)bad_node);
+    return CORAL_OK;
+}
+
+int coral_index_create(const coral_index_desc* d, coral_index** out) {
+    if (!d || !out) return fail(CORAL_ERR_ARG, "null argument");
+    *out = nullptr;
+    if (!d->base || !d->nbrs) return fail(CORAL_ERR_ARG, "null base or nbrs");
+    if (d->n <= 0 || d->n > 0x7fffffffLL) return fail(CORAL_ERR_ARG, "n out of range");
+    if (d->dim <= 0 || d->dim % 4 != 0 || d->dim > 2048)
+        return fail(CORAL_ERR_ARG, "dim must be a positive multiple of 4, at most 2048 (got %d)",
+                    d->dim);
+    if (d->R <= 0 || d->R > 32) return fail(CORAL_ERR_ARG, "R must be in 1..32 (got %d)", d->R);
+    if (d->metric != CORAL_L2 && d->metric != CORAL_IP) return fail(CORAL_ERR_ARG, "bad metric");
+    if (int rc = validate_graph(d->nbrs, d->n, d->R, d->start_ids, d->n_start)) return rc;
+
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev <= 0)
+        return fail(CORAL_ERR_DEVICE, "no HIP device (%s)", hipGetErrorString(e));
+    if (d->device < 0 || d->device >= ndev) return fail(CORAL_ERR_ARG, "device ordinal out of range");
+    HIP_TRY(hipSetDevice(d->device));
+
+    coral_index* idx = new (std::nothrow) coral_index();
+    if (!idx) return fail(CORAL_ERR_MEMORY, "host allocation failed");
+    idx->device = d->device, idx->n = d->n, idx->dim = d->dim, idx->R = d->R;
+    idx->M = d->n_start, idx->metric = d->metric;
+    hipDeviceProp_t prop;
+    auto cleanup = [&](int rc) {
+        coral_index_destroy(idx);
+        return rc;
+    };
+#define HIP_TRY_C(expr)                                                                      \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return cleanup(fail(e_ == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE, \
+                                "%s failed: %s", #expr, hipGetErrorString(e_)));             \
+    } while (0)
+    HIP_TRY_C(hipGetDeviceProperties(&prop, d->device));
+    idx->num_cu = prop.multiProcessorCount;
+    HIP_TRY_C(hipStreamCreate(&idx->stream));
+    const size_t vec_bytes = (size_t)d->n * d->dim * sizeof(float);
+    const size_t nbr_bytes = (size_t)d->n * d->R * sizeof(int32_t);
+    HIP_TRY_C(hipMalloc(&idx->d_vec, vec_bytes));
+    HIP_TRY_C(hipMalloc(&idx->d_nbrs, nbr_bytes));
+    HIP_TRY_C(hipMalloc(&idx->d_start, (size_t)d->n_start * sizeof(int32_t)));
+    HIP_TRY_C(hipMalloc(&idx->d_scalars, 4 * sizeof(int)));
+    HIP_TRY_C(hipMalloc(&idx->d_hit, sizeof(unsigned long long)));
+    HIP_TRY_C(hipMemcpy(idx->d_vec, d->base, vec_bytes, hipMemcpyHostToDevice));
+    HIP_TRY_C(hipMemcpy(idx->d_nbrs, d->nbrs, nbr_bytes, hipMemcpyHostToDevice));
+    HIP_TRY_C(hipMemcpy(idx->d_start, d->start_ids, (size_t)d->n_start * sizeof(int32_t),
+                        hipMemcpyHostToDevice));
+#undef HIP_TRY_C
+    *out = idx;
+    return CORAL_OK;
+}
+
+void coral_index_destroy(coral_index* idx) {
+    if (!idx) return;
+    (void)hipSetDevice(idx->device);
+    if (idx->stream) (void)hipStreamSynchronize(idx->stream);
+    (void)hipFree(idx->d_vec);
+    (void)hipFree(idx->d_nbrs);
+    (void)hipFree(idx->d_start);
+    (void)hipFree(idx->d_deleted);
+    (void)hipFree(idx->d_spill);
+    (void)hipFree(idx->d_counters);
+    (void)hipFree(idx->d_scalars);
+    (void)hipFree(idx->d_hit);
+    if (idx->h_counters) (void)hipHostFree(idx->h_counters);
+    if (idx->stream) (void)hipStreamDestroy(idx->stream);
+    delete idx;
+}
+
+int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const int32_t* start_ids,
+                          int32_t n_start) {
+    if (!idx || !nbrs) return fail(CORAL_ERR_ARG, "null argument");
+    if (int rc = validate_graph(nbrs, idx->n, idx->R, start_ids, n_start)) return rc;
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    if (n_start != idx->M) {
+        int32_t* p = nullptr;
+        HIP_TRY(hipMalloc(&p, (size_t)n_start * sizeof(int32_t)));
+        (void)hipFree(idx->d_start);
+        idx->d_start = p;
+        idx->M = n_start;
+        idx->prepared = false;
+    }
+    HIP_TRY(hipMemcpy(idx->d_nbrs, nbrs, (size_t)idx->n * idx->R * sizeof(int32_t),
+                      hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(idx->d_start, start_ids, (size_t)n_start * sizeof(int32_t),
+                      hipMemcpyHostToDevice));
+    return CORAL_OK;
+}
+
+int coral_index_set_deleted(coral_index* idx, const uint32_t* host_mask) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    if (!host_mask) {
+        (void)hipFree(idx->d_deleted);
+        idx->d_deleted = nullptr;
+        return CORAL_OK;
+    }
+    const size_t words = ((size_t)idx->n + 31) / 32;
+    if (!idx->d_deleted) HIP_TRY(hipMalloc(&idx->d_deleted, words * sizeof(uint32_t)));
+    HIP_TRY(hipMemcpy(idx->d_deleted, host_mask, words * sizeof(uint32_t), hipMemcpyHostToDevice));
+    return CORAL_OK;
+}
+
+int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* R, int32_t* n_start,
+                     int32_t* metric) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    if (n) *n = idx->n;
+    if (dim) *dim = idx->dim;
+    if (R) *R = idx->R;
+    if (n_start) *n_start = idx->M;
+    if (metric) *metric = idx->metric;
+    return CORAL_OK;
+}
+
+int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tuning* tuning) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
+    if (L <= 0 || L > kMaxL) return fail(CORAL_ERR_ARG, "L must be in 1..%d (got %d)", kMaxL, L);
+    if (idx->M > L)
+        return fail(CORAL_ERR_ARG, "%d start ids do not fit a beam of capacity %d", idx->M, L);
+    coral_tuning t;
+    std::memset(&t, 0, sizeof t);
+    if (tuning) t = *tuning;
+    int threads = t.threads ? t.threads : 256;
+    if (threads != 128 && threads != 256 && threads != 512)
+        return fail(CORAL_ERR_ARG, "threads must be 128, 256 or 512");
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+
+    // todo / candidate buffers: room for the rows of 16 beam entries
+    int tcap = std::max(512, ((idx->M + 3) & ~3));
+    tcap = std::max(tcap, idx->R * 4);
+    int ccap = tcap;
+    int slots_log2 = t.visited_slots_log2;
+    if (slots_log2 == 0) {
+        // degree-32 graphs visit about 30 nodes per beam entry; 48 slots per entry keep
+        // the load factor near one half; shrink only if LDS cannot hold the table
+        slots_log2 = 12;
+        while ((1 << slots_log2) < 48 * L && slots_log2 < 15) ++slots_log2;
+        while (slots_log2 > 11 &&
+               coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap) + 64 > (size_t)kMaxLdsBytes)
+            --slots_log2;
+    }
+    if (slots_log2 < 11 || slots_log2 > 15)
+        return fail(CORAL_ERR_ARG, "visited_slots_log2 must be in 11..15");
+    const int slots = 1 << slots_log2;
+    if (idx->M + tcap + 1 >= slots)
+        return fail(CORAL_ERR_ARG, "visited table of %d slots too small for %d start ids", slots,
+                    idx->M);
+    int vis_limit = std::min(slots - tcap - 1, slots - slots / 8);
+    if (vis_limit < idx->M) vis_limit = idx->M;
+    const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap);
+    if (lds + 64 > (size_t)kMaxLdsBytes)
+        return fail(CORAL_ERR_ARG, "L=%d with a %d-slot visited table needs %zu bytes of LDS", L, slots,
+                    lds);
+    int wg_per_cu = 0;
+    HIP_TRY(coral::search_kernel_prepare(idx->dim, lds, threads, &wg_per_cu));
+    if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
+    int workgroups = t.workgroups > 0 ? t.workgroups : wg_per_cu * idx->num_cu;
+    workgroups = std::min(workgroups, (int)Q);
+
+    const size_t spill_words = ((size_t)idx->n + 31) / 32;
+    const size_t need_words = spill_words * (size_t)workgroups;
+    if (need_words > idx->spill_alloc_words) {
+        (void)hipFree(idx->d_spill);
+        idx->d_spill = nullptr, idx->spill_alloc_words = 0;
+        HIP_TRY(hipMalloc(&idx->d_spill, need_words * sizeof(uint32_t)));
+        idx->spill_alloc_words = need_words;
+        HIP_TRY(coral::launch_fill_u32(idx->d_spill, need_words, 0u, idx->stream));
+    }
+    const size_t need_counters = (size_t)Q * 4;
+    if (need_counters > idx->counters_alloc) {
+        (void)hipFree(idx->d_counters);
+        if (idx->h_counters) (void)hipHostFree(idx->h_counters);
+        idx->d_counters = nullptr, idx->h_counters = nullptr, idx->counters_alloc = 0;
+        HIP_TRY(hipMalloc(&idx->d_counters, need_counters * sizeof(int32_t)));
+        HIP_TRY(hipHostMalloc(&idx->h_counters, need_counters * sizeof(int32_t)));
+        idx->counters_alloc = need_counters;
+    }
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    idx->Q = Q, idx->L = L, idx->slots_log2 = slots_log2, idx->vis_limit = vis_limit;
+    idx->tcap = tcap, idx->ccap = ccap, idx->threads = threads, idx->workgroups = workgroups;
+    idx->lds_bytes = lds, idx->spill_words = spill_words;
+    idx->prepared = true;
+    return CORAL_OK;
+}
+
+int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, float* d_dists,
+                     int32_t Q, int32_t k, int32_t policy, int32_t have_delete, void* stream_,
+                     coral_stats* stats) {
+    if (!idx || !d_queries || !d_ids) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->prepared) return fail(CORAL_ERR_STATE, "coral_search_prepare has not been called");
+    if (Q <= 0 || Q > idx->Q)
+        return fail(CORAL_ERR_ARG, "Q=%d exceeds the prepared batch of %d", Q, idx->Q);
+    if (k <= 0 || k > idx->L) return fail(CORAL_ERR_ARG, "k=%d must be in 1..L=%d", k, idx->L);
+    if (policy != CORAL_POLICY_ROUNDS && policy != CORAL_POLICY_BEST_FIRST)
+        return fail(CORAL_ERR_ARG, "unknown policy %d", policy);
+    if (have_delete && !idx->d_deleted)
+        return fail(CORAL_ERR_STATE, "have_delete set but no tombstone mask was given");
+    HIP_TRY(hipSetDevice(idx->device));
+    hipStream_t stream = stream_ ? (hipStream_t)stream_ : idx->stream;
+
+    coral::SearchArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.vec = idx->d_vec, a.nbrs = idx->d_nbrs, a.start_ids = idx->d_start;
+    a.deleted = have_delete ? idx->d_deleted : nullptr;
+    a.queries = d_queries, a.ids_out = d_ids, a.dists_out = d_dists;
+    a.counters = idx->d_counters, a.spill = idx->d_spill;
+    a.next_qid = idx->d_scalars, a.spill_count = idx->d_scalars + 1;
+    a.spill_words = idx->spill_words, a.n = idx->n;
+    a.dim = idx->dim, a.R = idx->R, a.M = idx->M, a.Q = Q, a.k = k, a.L = idx->L;
+    a.metric = idx->metric, a.policy = policy;
+    a.slots_log2 = idx->slots_log2, a.vis_limit = idx->vis_limit;
+    a.tcap = idx->tcap, a.ccap = idx->ccap;
+
+    hipEvent_t ev0, ev1;
+    HIP_TRY(hipEventCreate(&ev0));
+    HIP_TRY(hipEventCreate(&ev1));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_scalars, 4, 0u, stream));
+    // timed region, same scope as the reference: kernel + counter read-back
+    HIP_TRY(hipEventRecord(ev0, stream));
+    const int wgs = std::min(idx->workgroups, (int)Q);
+    HIP_TRY(coral::launch_search(a, wgs, idx->threads, idx->lds_bytes, stream));
+    HIP_TRY(hipMemcpyAsync(idx->h_counters, idx->d_counters, (size_t)Q * 4 * sizeof(int32_t),
+                           hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipEventRecord(ev1, stream));
+    HIP_TRY(hipEventSynchronize(ev1));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
+    (void)hipEventDestroy(ev0);
+    (void)hipEventDestroy(ev1);
+    int scal[2] = {0, 0};
+    HIP_TRY(hipMemcpyAsync(scal, idx->d_scalars, sizeof scal, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+    idx->last_Q = Q;
+    if (stats) {
+        std::memset(stats, 0, sizeof *stats);
+        stats->time_s = ms / 1000.0;
+        for (int q = 0; q < Q; ++q) {
+            const int32_t* c = idx->h_counters + (size_t)q * 4;
+            stats->hops += c[0], stats->expansions += c[1];
+            stats->dist_evals += c[2], stats->rounds += c[3];
+        }
+        stats->spills = scal[1];
+    }
+    return CORAL_OK;
+}
+
+int coral_search_query_counters(coral_index* idx, int32_t* host_out, int32_t Q) {
+    if (!idx || !host_out) return fail(CORAL_ERR_ARG, "null argument");
+    if (Q <= 0 || Q > idx->last_Q) return fail(CORAL_ERR_ARG, "no counters for %d queries", Q);
+    std::memcpy(host_out, idx->h_counters, (size_t)Q * 4 * sizeof(int32_t));
+    return CORAL_OK;
+}
+
+int coral_search(coral_index* idx, const float* h_queries, int32_t Q, int32_t k, int32_t L,
+                 int32_t policy, int32_t have_delete, int32_t* h_ids, float* h_dists,
+                 coral_stats* stats) {
+    if (!idx || !h_queries || !h_ids) return fail(CORAL_ERR_ARG, "null argument");
+    if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
+    if (k <= 0 || k > L) return fail(CORAL_ERR_ARG, "k=%d must be in 1..L=%d", k, L);
+    HIP_TRY(hipSetDevice(idx->device));
+    if (!idx->prepared || idx->L != L || idx->Q < Q) {
+        if (int rc = coral_search_prepare(idx, Q, L, nullptr)) return rc;
+    }
+    float* d_q = nullptr;
+    int32_t* d_ids = nullptr;
+    float* d_dists = nullptr;
+    int rc = CORAL_OK;
+    const size_t qbytes = (size_t)Q * idx->dim * sizeof(float);
+    auto release = [&]() {
+        (void)hipFree(d_q);
+        (void)hipFree(d_ids);
+        (void)hipFree(d_dists);
+    };
+#define HIP_TRY_R(expr)                                                                         \
+    do {                                                                                        \
+        hipError_t e_ = (expr);                                                                 \
+        if (e_ != hipSuccess) {                                                                 \
+            release();                                                                          \
+            return fail(e_ == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE,        \
+                        "%s failed: %s", #expr, hipGetErrorString(e_));                         \
+        }                                                                                       \
+    } while (0)
+    HIP_TRY_R(hipMalloc(&d_q, qbytes));
+    HIP_TRY_R(hipMalloc(&d_ids, (size_t)Q * k * sizeof(int32_t)));
+    if (h_dists) HIP_TRY_R(hipMalloc(&d_dists, (size_t)Q * k * sizeof(float)));
+    HIP_TRY_R(hipMemcpy(d_q, h_queries, qbytes, hipMemcpyHostToDevice));
+    rc = coral_search_gpu(idx, d_q, d_ids, d_dists, Q, k, policy, have_delete, nullptr, stats);
+    if (rc == CORAL_OK) {
+        HIP_TRY_R(hipMemcpy(h_ids, d_ids, (size_t)Q * k * sizeof(int32_t), hipMemcpyDeviceToHost));
+        if (h_dists)
+            HIP_TRY_R(hipMemcpy(h_dists, d_dists, (size_t)Q * k * sizeof(float), hipMemcpyDeviceToHost));
+    }
+#undef HIP_TRY_R
+    release();
+    return rc;
+}
+
+int coral_search_verify(coral_index* idx, const int32_t* d_ids_res, const int32_t* d_ids_gt, int32_t Q,
+                        int32_t k, int64_t* hits) {
+    if (!idx || !d_ids_res || !d_ids_gt || !hits) return fail(CORAL_ERR_ARG, "null argument");
+    if (Q <= 0 || k <= 0) return fail(CORAL_ERR_ARG, "Q and k must be positive");
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_hit, 2, 0u, idx->stream));
+    HIP_TRY(coral::launch_verify(d_ids_res, d_ids_gt, idx->d_hit, Q, k, idx->stream));
+    unsigned long long h = 0;
+    HIP_TRY(hipMemcpyAsync(&h, idx->d_hit, sizeof h, hipMemcpyDeviceToHost, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    *hits = (int64_t)h;
+    return CORAL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,150 @@
+/*
+ * coral_search.h -- C ABI of libcoral_search.so: CORAL's batched graph beam
+ * search on one MI355X (gfx950), whole index resident in HBM.
+ *
+ * The reference's boundary for this path is a C++ class (efanna2e::IndexGPU over
+ * GPUFuncs, include/index_gpu.h:42-76, include/gpufuncs.cuh:597-893); it has no C
+ * interface.  Each entry point below names the reference member it stands for.
+ * include/efanna2e/index_gpu.h in this repository is the C++ class of the same
+ * name and signatures, implemented on top of these calls.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every function returns a coral_status
+ *     (0 = success) instead of terminating the process the way the reference's
+ *     CUDA_CHECK / fo.eprint do (include/utils.cuh:50-58, src/fileout.cpp:88-98);
+ *     coral_last_error() gives the message of the calling thread's last failure.
+ *   - metric: CORAL_L2 = squared Euclidean, smaller is closer; CORAL_IP = raw
+ *     inner product, larger is closer (include/utils.cuh:380-382, include/uni.h:65-68).
+ *   - graph rows are compact: int32 nbrs[n][R], a row's neighbours are its
+ *     leading non-negative entries (the deg and nbrs[0..deg) fields of the
+ *     reference's 400-byte Slot, include/disk_graph.h:30-52, and nothing else).
+ *   - results are ordered closest first; unfilled slots hold id -1 and the
+ *     farthest sentinel (FLT_MAX for L2, -FLT_MAX for IP).
+ *   - not thread-safe per index, like the reference (src/search.cu:404-408).
+ */
+#ifndef CORAL_SEARCH_H
+#define CORAL_SEARCH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define CORAL_API __attribute__((visibility("default")))
+#else
+#define CORAL_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    CORAL_OK = 0,
+    CORAL_ERR_ARG = 1,      /* null pointer, size out of range, k > L, M > L ... */
+    CORAL_ERR_GRAPH = 2,    /* neighbour id or start id out of range, duplicate start ids */
+    CORAL_ERR_DEVICE = 3,   /* a HIP call failed; message carries hipGetErrorString */
+    CORAL_ERR_MEMORY = 4,   /* host or device allocation failed */
+    CORAL_ERR_IO = 5,       /* file missing, short, or malformed */
+    CORAL_ERR_STATE = 6     /* call order: search before prepare, and the like */
+} coral_status;
+
+enum { CORAL_L2 = 0, CORAL_IP = 1 };
+
+/* Traversal policy.
+ * CORAL_POLICY_ROUNDS: every beam entry not yet expanded is expanded in one
+ *   round, candidates are pre-filtered against the threshold frozen at the start
+ *   of the round, then merged (the CUDA kernel, src/search_gpu.cu:347-580).
+ * CORAL_POLICY_BEST_FIRST: one expansion at a time, always the closest entry not
+ *   yet expanded (the CPU path, src/search_in_cpu.cpp:63-108). */
+enum { CORAL_POLICY_ROUNDS = 0, CORAL_POLICY_BEST_FIRST = 1 };
+
+typedef struct coral_index coral_index;
+
+/* Host-side description of an index; all pointers are borrowed for the duration
+ * of coral_index_create only (the data is copied into HBM). */
+typedef struct {
+    const float* base;        /* [n][dim] fp32 row major; dim % 4 == 0 */
+    const int32_t* nbrs;      /* [n][R] compact rows, -1 padded */
+    int64_t n;
+    int32_t dim;
+    int32_t R;                /* row width, <= 32 (MAX_DEGREE, include/uni.h:60) */
+    const int32_t* start_ids; /* graph.search_start_ids, src/graph.cpp:329-351 */
+    int32_t n_start;
+    int32_t metric;
+    int32_t device;           /* HIP device ordinal; the reference hard-codes 0 */
+} coral_index_desc;
+
+/* Counters of one search call.  time_s has the scope of the reference's own
+ * timer (src/search_gpu.cu:861-877): the kernel plus the read-back of the
+ * per-query counters, measured with a HIP event pair on the search stream. */
+typedef struct {
+    double time_s;
+    int64_t hops;        /* what Test_Result.hops holds for this policy */
+    int64_t expansions;  /* graph rows read */
+    int64_t dist_evals;  /* vector rows read (first visits + start ids) */
+    int64_t rounds;      /* merge rounds (ROUNDS) or expansion steps (BEST_FIRST) */
+    int64_t spills;      /* queries whose visited set outgrew LDS */
+} coral_stats;
+
+/* Optional launch tuning; zero-initialise for defaults. */
+typedef struct {
+    int32_t visited_slots_log2; /* LDS visited table size; 0 = chosen from L */
+    int32_t workgroups;         /* persistent workgroups; 0 = chosen from Q and the device */
+    int32_t threads;            /* threads per workgroup: 0 (=256), 128, 256 or 512 */
+    int32_t reserved[5];
+} coral_tuning;
+
+CORAL_API const char* coral_last_error(void);
+
+/* Graph ctor, GPU branch (include/graph.cuh:240-261): device allocation and
+ * upload of the graph rows and vectors; also validates ids, which the reference
+ * does not.  For CORAL_IP the caller has already normalised base, as
+ * IndexGPU::LoadVectorData does (src/index_gpu.cpp:641). */
+CORAL_API int coral_index_create(const coral_index_desc* desc, coral_index** out);
+CORAL_API void coral_index_destroy(coral_index* idx);
+
+/* Replace the graph rows of an existing index (Graph::LoadRoarGraph's upload,
+ * src/graph.cu:737-742) and its start ids. */
+CORAL_API int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const int32_t* start_ids,
+                          int32_t n_start);
+
+/* Tombstone mask, bit (id & 31) of word (id >> 5) (src/update.cu:406-412);
+ * host_mask holds ceil(n/32) words, or NULL to clear. */
+CORAL_API int coral_index_set_deleted(coral_index* idx, const uint32_t* host_mask);
+
+CORAL_API int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* R,
+                     int32_t* n_start, int32_t* metric);
+
+/* GPUFuncs::search_prepare(Q, L) (src/search.cu:400-408): fixes the beam
+ * capacity and (re)allocates per-workgroup scratch. */
+CORAL_API int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tuning* tuning);
+
+/* GPUFuncs::search_gpu (src/search_gpu.cu:835-886): device pointers in and out,
+ * one persistent launch.  d_dists may be NULL.  have_delete selects the
+ * tombstone-aware output (src/search_gpu.cu:582-833).  stream is a hipStream_t
+ * (NULL = the index's own stream, like streams["search"]). */
+CORAL_API int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, float* d_dists,
+                     int32_t Q, int32_t k, int32_t policy, int32_t have_delete, void* stream,
+                     coral_stats* stats);
+
+/* Per-query counters of the last coral_search_gpu call, int32 [Q][4] on the
+ * host: hops, expansions, dist_evals, rounds. */
+CORAL_API int coral_search_query_counters(coral_index* idx, int32_t* host_out, int32_t Q);
+
+/* IndexGPU::Search (src/index_gpu.cpp:117-136): host buffers in and out; uploads
+ * the queries, prepares for (Q, L), searches, downloads ids (and distances when
+ * h_dists is not NULL). */
+CORAL_API int coral_search(coral_index* idx, const float* h_queries, int32_t Q, int32_t k, int32_t L,
+                 int32_t policy, int32_t have_delete, int32_t* h_ids, float* h_dists,
+                 coral_stats* stats);
+
+/* GPUFuncs::search_verify / ids_verify_kernel (src/search_gpu.cu:888-922):
+ * hits = sum over queries of |res[q][0..k) n gt[q][0..k)|, both device arrays
+ * with row stride k. */
+CORAL_API int coral_search_verify(coral_index* idx, const int32_t* d_ids_res, const int32_t* d_ids_gt,
+                        int32_t Q, int32_t k, int64_t* hits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CORAL_SEARCH_H */

@@ -1,0 +1,659 @@
+/*
+ * coral_oracle.c -- CPU restatement of CORAL's batched graph beam search.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is the checker the HIP path is compared
+ * against (tests/, the smoke check, and the "cpu_baseline" leg of bench.py).
+ * Nothing in the shipped library links, loads or calls it.
+ *
+ * What is restated, and from where (paths relative to the reference tree):
+ *   - policy A, "best-first":  src/search_in_cpu.cpp:23-119 over the sorted
+ *     queue of include/efanna2e/neighbor.h:148-237 (order: include/efanna2e/neighbor.h:39-41)
+ *   - policy B, "expand-all rounds": src/search_gpu.cu:347-580 (bitmap variant)
+ *     and :582-833 (tombstone variant; bit layout src/update.cu:406-412)
+ *   - distances: include/utils.cuh:254-275 (l2_distance), :307-323 (ip_distance),
+ *     src/search_gpu.cu:14-23 (warp_calc_dist), include/efanna2e/distance.h:39-89
+ *     (DistanceL2::compare), comparisons include/utils.cuh:368-386 and the
+ *     sentinels of include/uni.h:65-68
+ *   - recall: tests/test_search_pipeline.cpp:25-39; normalisation src/uni.cpp:38-54
+ *
+ * Pinning status (what fixes each function besides this text):
+ *   - oracle_dist ORDER_CPU_AVX512, oracle_queue_*, oracle_search_A: bit-exact
+ *     against oracle/_ref (the reference's own neighbor.h + distance.h compiled
+ *     in place) and against the committed fixtures tests/golden/policyA_*.json
+ *     that were written from it; plus brute-force invariants.
+ *   - oracle_dist ORDER_GPU_SEQ / ORDER_GPU_WARP32 / ORDER_WAVE64: fp64 closed
+ *     form within 1e-5 relative; special cases (identical vectors, unit vectors,
+ *     one-hot vectors that expose index or sign mistakes).  The exact rounding of
+ *     the two CUDA orders cannot be executed anywhere here: they are pinned by
+ *     code reading only; the 1e-5 tolerance of the search contract covers it.
+ *   - oracle_search_B: nothing executable exists for it (the CUDA kernel cannot
+ *     be built or run here).  Pinned by code reading plus invariants: result ==
+ *     top-k of top-L(visited) under (distance,id); every beam entry expanded at
+ *     exit; equality with exact kNN on complete graphs and when L >= N;
+ *     hand-computed traversals on path/ring graphs; an independent
+ *     set-based pure-Python simulator on tiny inputs.
+ *
+ * Graph rows are the compact form used on the device: int32 nbrs[N][R] where
+ * a row's neighbours are its leading non-negative entries (deg = index of the
+ * first negative entry, or R).  This carries exactly the fields of the
+ * reference's Slot that search reads (deg, nbrs[0..deg)), include/disk_graph.h:30-52.
+ */
+#include <float.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+enum { ORACLE_L2 = 0, ORACLE_IP = 1 };
+enum {
+    ORDER_GPU_SEQ = 0,    /* one thread walks the row: include/utils.cuh:254-275, 307-323 */
+    ORDER_GPU_WARP32 = 1, /* 32 lane-strided partials + shuffle-down tree: src/search_gpu.cu:14-23 */
+    ORDER_CPU_AVX512 = 2, /* 16/8/4-lane partials + two hadd: include/efanna2e/distance.h:39-89 */
+    ORDER_WAVE64 = 3      /* the summation order of this repository's HIP kernel */
+};
+
+typedef struct {
+    const float* base;   /* [n][dim] row major */
+    const int32_t* nbrs; /* [n][R], -1 padded */
+    int64_t n;
+    int32_t dim;
+    int32_t R;
+    const int32_t* start_ids;
+    int32_t n_start;
+    const uint32_t* deleted; /* optional tombstone mask, bit (id&31) of word id>>5 */
+} oracle_index;
+
+/* ---------------------------------------------------------------- distances */
+
+/* include/utils.cuh:254-275 (L2) and :307-323 (IP): sequential accumulation in
+ * x,y,z,w order.  `sum += t*t` is contracted to one fused multiply-add by the
+ * CUDA compiler's default -fmad=true; the IP form is written with fmaf in the
+ * reference.  The scalar tail of the L2 form continues the same chain. */
+static float dist_gpu_seq(const float* q, const float* b, int dim, int metric) {
+    float sum = 0.0f;
+    if (metric == ORACLE_L2) {
+        for (int i = 0; i < dim; ++i) {
+            float t = q[i] - b[i];
+            sum = fmaf(t, t, sum);
+        }
+    } else {
+        for (int i = 0; i < dim; ++i) sum = fmaf(q[i], b[i], sum);
+    }
+    return sum;
+}
+
+/* src/search_gpu.cu:14-23: lane l sums d = l, l+32, ...; then
+ * sum += shfl_down(sum, off) for off = 16..1; lane 0 holds the result. */
+static float dist_gpu_warp32(const float* q, const float* b, int dim, int metric) {
+    float p[32];
+    for (int l = 0; l < 32; ++l) {
+        float sum = 0.0f;
+        for (int d = l; d < dim; d += 32) {
+            if (metric == ORACLE_L2) {
+                float t = q[d] - b[d];
+                sum = fmaf(t, t, sum);
+            } else {
+                sum = fmaf(q[d], b[d], sum);
+            }
+        }
+        p[l] = sum;
+    }
+    for (int off = 16; off > 0; off >>= 1)
+        for (int l = 0; l < off; ++l) p[l] = p[l] + p[l + off];
+    return p[0];
+}
+
+/* include/efanna2e/distance.h:39-89, lane by lane.  The vector expression
+ * `msum += d*d` is contracted to vfmadd by gcc at -O2 with AVX-512F. */
+static float dist_cpu_avx512_scalar(const float* x, const float* y, unsigned d) {
+    float m0[16], m1[8], m2[4];
+    for (int i = 0; i < 16; ++i) m0[i] = 0.0f;
+    while (d >= 16) {
+        for (int i = 0; i < 16; ++i) {
+            float t = x[i] - y[i];
+            m0[i] = fmaf(t, t, m0[i]);
+        }
+        x += 16, y += 16, d -= 16;
+    }
+    for (int i = 0; i < 8; ++i) m1[i] = m0[i + 8] + m0[i];
+    if (d >= 8) {
+        for (int i = 0; i < 8; ++i) {
+            float t = x[i] - y[i];
+            m1[i] = fmaf(t, t, m1[i]);
+        }
+        x += 8, y += 8, d -= 8;
+    }
+    for (int i = 0; i < 4; ++i) m2[i] = m1[i + 4] + m1[i];
+    if (d >= 4) {
+        for (int i = 0; i < 4; ++i) {
+            float t = x[i] - y[i];
+            m2[i] = fmaf(t, t, m2[i]);
+        }
+        x += 4, y += 4, d -= 4;
+    }
+    if (d > 0) {
+        for (unsigned i = 0; i < d; ++i) {
+            float t = x[i] - y[i];
+            m2[i] = fmaf(t, t, m2[i]);
+        }
+    }
+    /* two _mm_hadd_ps: (a0+a1)+(a2+a3) */
+    return (m2[0] + m2[1]) + (m2[2] + m2[3]);
+}
+
+#if defined(__x86_64__)
+/* Same arithmetic with intrinsics, used only to make the timed CPU baseline run
+ * at the speed the reference's own AVX-512 routine would.  Must agree bit for
+ * bit with dist_cpu_avx512_scalar (tests check it). */
+__attribute__((target("avx512f,avx512dq,fma"))) static float dist_cpu_avx512_simd(const float* x,
+                                                                                  const float* y,
+                                                                                  unsigned d) {
+    __m512 s0 = _mm512_setzero_ps();
+    while (d >= 16) {
+        __m512 t = _mm512_sub_ps(_mm512_loadu_ps(x), _mm512_loadu_ps(y));
+        s0 = _mm512_fmadd_ps(t, t, s0);
+        x += 16, y += 16, d -= 16;
+    }
+    __m256 s1 = _mm256_add_ps(_mm512_extractf32x8_ps(s0, 1), _mm512_extractf32x8_ps(s0, 0));
+    if (d >= 8) {
+        __m256 t = _mm256_sub_ps(_mm256_loadu_ps(x), _mm256_loadu_ps(y));
+        s1 = _mm256_fmadd_ps(t, t, s1);
+        x += 8, y += 8, d -= 8;
+    }
+    __m128 s2 = _mm_add_ps(_mm256_extractf128_ps(s1, 1), _mm256_extractf128_ps(s1, 0));
+    if (d >= 4) {
+        __m128 t = _mm_sub_ps(_mm_loadu_ps(x), _mm_loadu_ps(y));
+        s2 = _mm_fmadd_ps(t, t, s2);
+        x += 4, y += 4, d -= 4;
+    }
+    if (d > 0) {
+        float bx[4] = {0, 0, 0, 0}, by[4] = {0, 0, 0, 0};
+        for (unsigned i = 0; i < d; ++i) bx[i] = x[i], by[i] = y[i];
+        __m128 t = _mm_sub_ps(_mm_loadu_ps(bx), _mm_loadu_ps(by));
+        s2 = _mm_fmadd_ps(t, t, s2);
+    }
+    s2 = _mm_hadd_ps(s2, s2);
+    s2 = _mm_hadd_ps(s2, s2);
+    return _mm_cvtss_f32(s2);
+}
+#endif
+
+static int g_have_avx512 = -1;
+static int have_avx512(void) {
+#if defined(__x86_64__)
+    if (g_have_avx512 < 0)
+        g_have_avx512 = __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512dq");
+    return g_have_avx512;
+#else
+    return 0;
+#endif
+}
+
+/* The HIP kernel's order.  A row is read as float4 chunks; a group of G lanes
+ * (G = 16, 32 or 64, the smallest that covers dim/4 chunks, capped at 64) owns
+ * the row; lane l accumulates chunks l, l+G, ... with four fused multiply-adds
+ * per chunk in x,y,z,w order; the G partials are then combined by a butterfly,
+ * p[l] += p[l ^ off] for off = G/2 .. 1. */
+static int wave64_group(int dim) {
+    int chunks = dim / 4;
+    if (chunks <= 16) return 16;
+    if (chunks <= 32) return 32;
+    return 64;
+}
+static float dist_wave64(const float* q, const float* b, int dim, int metric) {
+    const int G = wave64_group(dim), chunks = dim / 4;
+    float p[64];
+    for (int l = 0; l < G; ++l) {
+        float acc = 0.0f;
+        for (int c = l; c < chunks; c += G) {
+            for (int j = 0; j < 4; ++j) {
+                const float qv = q[4 * c + j], bv = b[4 * c + j];
+                if (metric == ORACLE_L2) {
+                    float t = qv - bv;
+                    acc = fmaf(t, t, acc);
+                } else {
+                    acc = fmaf(qv, bv, acc);
+                }
+            }
+        }
+        p[l] = acc;
+    }
+    for (int off = G / 2; off > 0; off >>= 1)
+        for (int l = 0; l < off; ++l) p[l] = p[l] + p[l + off];
+    return p[0];
+}
+
+static inline float dist_any(const float* q, const float* b, int dim, int metric, int order) {
+    switch (order) {
+        case ORDER_GPU_SEQ: return dist_gpu_seq(q, b, dim, metric);
+        case ORDER_GPU_WARP32: return dist_gpu_warp32(q, b, dim, metric);
+        case ORDER_WAVE64: return dist_wave64(q, b, dim, metric);
+        default:
+            /* DistanceL2 only: src/search_in_cpu.cpp:52 builds a DistanceL2 whatever the metric */
+#if defined(__x86_64__)
+            if (have_avx512()) return dist_cpu_avx512_simd(b, q, (unsigned)dim);
+#endif
+            return dist_cpu_avx512_scalar(b, q, (unsigned)dim);
+    }
+}
+
+ORACLE_API float oracle_dist(const float* q, const float* b, int dim, int metric, int order) {
+    return dist_any(q, b, dim, metric, order);
+}
+/* scalar form of ORDER_CPU_AVX512 whatever the host supports (for the agreement test) */
+ORACLE_API float oracle_dist_avx512_scalar(const float* x, const float* y, int dim) {
+    return dist_cpu_avx512_scalar(x, y, (unsigned)dim);
+}
+ORACLE_API int oracle_have_avx512(void) { return have_avx512(); }
+
+/* include/utils.cuh:380-382: "d1 is closer than d0" */
+static inline int closer(float d0, float d1, int metric) {
+    return metric == ORACLE_L2 ? d0 > d1 : d0 < d1;
+}
+/* include/uni.h:65-68 */
+static inline float farthest(int metric) { return metric == ORACLE_L2 ? FLT_MAX : -FLT_MAX; }
+
+/* src/uni.cpp:38-54 */
+ORACLE_API void oracle_normalize_l2(float* x, int64_t n, int64_t d) {
+    for (int64_t i = 0; i < n; ++i) {
+        float* row = x + i * d;
+        float norm2 = 0.0f;
+        for (int64_t j = 0; j < d; ++j) norm2 += row[j] * row[j];
+        float norm = sqrtf(norm2);
+        if (norm > 0.0f) {
+            float inv = 1.0f / norm;
+            for (int64_t j = 0; j < d; ++j) row[j] *= inv;
+        }
+    }
+}
+
+/* ------------------------------------------------------- policy A: the queue */
+
+typedef struct {
+    int32_t id;
+    float distance;
+    int32_t flag;
+} qent;
+
+typedef struct {
+    size_t size, capacity, cur;
+    qent* data; /* capacity + 1 entries */
+} pqueue;
+
+/* include/efanna2e/neighbor.h:39-41 */
+static inline int ent_less(const qent* a, const qent* b) {
+    return a->distance < b->distance || (a->distance == b->distance && a->id < b->id);
+}
+
+/* include/efanna2e/neighbor.h:162-195 */
+static void pq_insert(pqueue* q, int32_t id, float dist) {
+    qent nbr = {id, dist, 0};
+    if (q->size == q->capacity && ent_less(&q->data[q->size - 1], &nbr)) return;
+    size_t lo = 0, hi = q->size;
+    while (lo < hi) {
+        size_t mid = (lo + hi) >> 1;
+        if (ent_less(&nbr, &q->data[mid]))
+            hi = mid;
+        else if (q->data[mid].id == nbr.id)
+            return;
+        else
+            lo = mid + 1;
+    }
+    if (lo < q->capacity) memmove(&q->data[lo + 1], &q->data[lo], (q->size - lo) * sizeof(qent));
+    q->data[lo] = nbr;
+    if (q->size < q->capacity) q->size++;
+    if (lo < q->cur) q->cur = lo;
+}
+
+/* include/efanna2e/neighbor.h:197-204 */
+static qent pq_closest_unexpanded(pqueue* q) {
+    q->data[q->cur].flag = 1;
+    size_t pre = q->cur;
+    while (q->cur < q->size && q->data[q->cur].flag) q->cur++;
+    return q->data[pre];
+}
+
+/* Exposed so tests can drive the queue with arbitrary insert/pop sequences.
+ * ops[i] >= 0: insert (id = ops[i], dist = dists[i]); ops[i] == -1: closest_unexpanded
+ * (only issued when cur < size; the popped id is appended to popped[]).
+ * Returns the final size; ids/dist/flags get the final contents, *cur_out the cursor. */
+ORACLE_API int oracle_queue_run(int capacity, const int32_t* ops, const float* dists, int n_ops,
+                                int32_t* ids_out, float* dists_out, int32_t* flags_out,
+                                int32_t* cur_out, int32_t* popped, int32_t* n_popped) {
+    pqueue q = {0, (size_t)capacity, 0, (qent*)calloc((size_t)capacity + 1, sizeof(qent))};
+    int np = 0;
+    for (int i = 0; i < n_ops; ++i) {
+        if (ops[i] >= 0)
+            pq_insert(&q, ops[i], dists[i]);
+        else if (q.cur < q.size)
+            popped[np++] = pq_closest_unexpanded(&q).id;
+    }
+    for (size_t i = 0; i < q.size; ++i) {
+        ids_out[i] = q.data[i].id;
+        dists_out[i] = q.data[i].distance;
+        flags_out[i] = q.data[i].flag;
+    }
+    *cur_out = (int32_t)q.cur;
+    *n_popped = np;
+    int sz = (int)q.size;
+    free(q.data);
+    return sz;
+}
+
+static inline int is_deleted(const uint32_t* del, int32_t id) {
+    return del && ((del[id >> 5] >> (id & 31)) & 1u);
+}
+
+static double now_s(void) {
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+
+/* stats layout per query: [0] hops as the reference reports them, [1] node
+ * expansions (graph rows read), [2] distance evaluations, [3] rounds/steps */
+#define NSTAT 4
+
+/*
+ * Policy A.  src/search_in_cpu.cpp:23-119.
+ *   M          number of start ids used (the reference takes PC.search_start_nodes_num, :26)
+ *   order      ORDER_CPU_AVX512 is what the reference runs (always squared L2, :52);
+ *              other orders honour `metric` and exist to compare against the GPU path
+ *   nthreads   <= 0: all OpenMP threads
+ * Unfilled result slots keep id -1 / dist +inf (:33-35).
+ * Tombstones do not exist on the reference's CPU path; when idx->deleted is set
+ * the rule of the GPU kernel is applied (src/search_gpu.cu:695-725): traversal
+ * ignores the mask, deleted ids are skipped while emitting the final list.
+ */
+ORACLE_API int oracle_search_A(const oracle_index* idx, const float* queries, int Q, int k, int L,
+                               int M, int metric, int order, int32_t* ids, float* dists,
+                               int32_t* stats, int nthreads, double* time_s) {
+    if (!idx || !queries || !ids || k <= 0 || L <= 0 || M <= 0 || M > idx->n_start) return -1;
+    const int dim = idx->dim, R = idx->R;
+    const int dmetric = (order == ORDER_CPU_AVX512) ? ORACLE_L2 : metric;
+    for (size_t i = 0; i < (size_t)Q * k; ++i) ids[i] = -1;
+    if (dists)
+        for (size_t i = 0; i < (size_t)Q * k; ++i) dists[i] = INFINITY;
+#ifdef _OPENMP
+    int nt = nthreads > 0 ? nthreads : omp_get_max_threads();
+#else
+    int nt = 1;
+#endif
+    double elapsed = 0.0;
+#pragma omp parallel num_threads(nt)
+    {
+        uint8_t* visited = (uint8_t*)calloc((size_t)idx->n, 1);
+        uint8_t tag = 1;
+        pqueue pq = {0, (size_t)L, 0, (qent*)malloc(((size_t)L + 1) * sizeof(qent))};
+#pragma omp barrier
+        double t0 = now_s();
+#pragma omp for schedule(dynamic, 1)
+        for (int qi = 0; qi < Q; ++qi) {
+            const float* query = queries + (size_t)qi * dim;
+            pq.size = 0, pq.cur = 0;
+            if (++tag == 0) {
+                memset(visited, 0, (size_t)idx->n);
+                tag = 1;
+            }
+            int64_t nd = 0, ne = 0;
+            for (int i = 0; i < M; ++i) {
+                const int32_t id = idx->start_ids[i];
+                float d = dist_any(query, idx->base + (size_t)id * dim, dim, dmetric, order);
+                if (dmetric == ORACLE_IP) d = -d; /* queue orders ascending */
+                pq_insert(&pq, id, d);
+                visited[id] = tag;
+                ++nd;
+            }
+            uint32_t hops = (uint32_t)M;
+            while (pq.cur < pq.size) {
+                qent cur = pq_closest_unexpanded(&pq);
+                const int32_t* row = idx->nbrs + (size_t)cur.id * R;
+                ++hops, ++ne;
+                for (int i = 0; i < R && row[i] >= 0; ++i) {
+                    const int32_t v = row[i];
+                    if (visited[v] == tag) continue;
+                    float d = dist_any(query, idx->base + (size_t)v * dim, dim, dmetric, order);
+                    if (dmetric == ORACLE_IP) d = -d;
+                    pq_insert(&pq, v, d);
+                    visited[v] = tag;
+                    ++nd;
+                }
+            }
+            int out = 0;
+            for (size_t i = 0; i < pq.size && out < k; ++i) {
+                if (is_deleted(idx->deleted, pq.data[i].id)) continue;
+                ids[(size_t)qi * k + out] = pq.data[i].id;
+                if (dists)
+                    dists[(size_t)qi * k + out] =
+                        dmetric == ORACLE_IP ? -pq.data[i].distance : pq.data[i].distance;
+                ++out;
+            }
+            if (stats) {
+                stats[(size_t)qi * NSTAT + 0] = (int32_t)hops;
+                stats[(size_t)qi * NSTAT + 1] = (int32_t)ne;
+                stats[(size_t)qi * NSTAT + 2] = (int32_t)nd;
+                stats[(size_t)qi * NSTAT + 3] = (int32_t)ne;
+            }
+        }
+        double t1 = now_s(); /* after the implicit barrier of the omp for */
+#pragma omp master
+        elapsed = t1 - t0;
+        free(visited);
+        free(pq.data);
+    }
+    if (time_s) *time_s = elapsed;
+    return 0;
+}
+
+/* ------------------------------------------------------------- policy B */
+
+typedef struct {
+    int32_t id;
+    float s; /* signed distance, smaller is closer: d for L2, -ip for IP */
+    int32_t expanded;
+} bent;
+
+static int bent_cmp(const void* a, const void* b) {
+    const bent *x = (const bent*)a, *y = (const bent*)b;
+    if (x->s < y->s) return -1;
+    if (x->s > y->s) return 1;
+    return (x->id > y->id) - (x->id < y->id);
+}
+
+/*
+ * Policy B.  src/search_gpu.cu:347-580; with idx->deleted the tombstone variant :582-833.
+ *
+ *   beam <- the M start ids (all of idx->start_ids, :843), distances in start_order
+ *           (the reference uses warp_calc_dist for them, :400-401)
+ *   thr  <- farthest
+ *   repeat
+ *     C <- {}
+ *     for every beam entry not yet expanded (:416-438): mark it expanded; for each
+ *       neighbour v: if test-and-set(visited, v) was clear: d <- dist(v) in nbr_order;
+ *       if d strictly closer than thr (thr is frozen for the round, :432): C += (v,d)
+ *     if C is empty: stop (:442)
+ *     hops += |C| (:481, :574)
+ *     if |beam| + |C| <= L: append (:477-483), thr unchanged
+ *     else: beam <- the L closest of beam u C (:525-570); thr <- worst of beam (:572-576)
+ *   output the k closest of the beam, closest first (:447-472), skipping tombstoned
+ *   ids when a mask is given (:695-725).
+ *
+ * Two deliberate choices where the reference is loose:
+ *   - ties are ordered by (distance, id); the reference's order among equal
+ *     distances depends on thread timing;
+ *   - an entry keeps its own expanded flag when the beam is rebuilt.  The
+ *     reference's full re-selection branch (:739-777) copies flags in place and
+ *     can hand an entry another entry's flag; that branch is unreachable without
+ *     tombstones (total <= 2L by :441) and the outcome here is what the intended
+ *     algorithm gives;
+ *   - fewer than k live entries: remaining slots get id -1 and the farthest
+ *     sentinel (the reference asserts a full beam, :444, and would emit garbage).
+ * The start ids must be distinct (the reference's farthest-point sampling always
+ * produces distinct ids); duplicates are rejected.
+ */
+ORACLE_API int oracle_search_B(const oracle_index* idx, const float* queries, int Q, int k, int L,
+                               int metric, int start_order, int nbr_order, int32_t* ids,
+                               float* dists, int32_t* stats, int nthreads, double* time_s) {
+    if (!idx || !queries || !ids || k <= 0 || L <= 0 || idx->n_start <= 0) return -1;
+    const int dim = idx->dim, R = idx->R, M = idx->n_start;
+    if (M > L) return -2;
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < i; ++j)
+            if (idx->start_ids[i] == idx->start_ids[j]) return -3;
+#ifdef _OPENMP
+    int nt = nthreads > 0 ? nthreads : omp_get_max_threads();
+#else
+    int nt = 1;
+#endif
+    const size_t vwords = ((size_t)idx->n + 31) / 32;
+    double t0 = now_s();
+#pragma omp parallel num_threads(nt)
+    {
+        uint32_t* visited = (uint32_t*)malloc(vwords * 4);
+        size_t cap = (size_t)L * R + L;
+        bent* beam = (bent*)malloc(cap * sizeof(bent));
+        bent* cand = (bent*)malloc((size_t)L * R * sizeof(bent));
+#pragma omp for schedule(dynamic, 1)
+        for (int qi = 0; qi < Q; ++qi) {
+            const float* query = queries + (size_t)qi * dim;
+            memset(visited, 0, vwords * 4);
+            int nb = 0;
+            int64_t hops = 0, ne = 0, nd = 0, rounds = 0;
+            for (int i = 0; i < M; ++i) {
+                const int32_t id = idx->start_ids[i];
+                visited[id >> 5] |= 1u << (id & 31);
+                float d = dist_any(query, idx->base + (size_t)id * dim, dim, metric, start_order);
+                beam[nb].id = id;
+                beam[nb].s = metric == ORACLE_IP ? 0.0f - d : d;
+                beam[nb].expanded = 0;
+                ++nb, ++nd;
+            }
+            float thr = FLT_MAX; /* signed form of the farthest sentinel for both metrics */
+            for (;;) {
+                int nc = 0;
+                const int nb0 = nb;
+                for (int bi = 0; bi < nb0; ++bi) {
+                    if (beam[bi].expanded) continue;
+                    beam[bi].expanded = 1;
+                    const int32_t* row = idx->nbrs + (size_t)beam[bi].id * R;
+                    ++ne; /* the row is read to learn its degree, :420 */
+                    for (int j = 0; j < R && row[j] >= 0; ++j) {
+                        const int32_t v = row[j];
+                        const uint32_t m = 1u << (v & 31);
+                        if (visited[v >> 5] & m) continue;
+                        visited[v >> 5] |= m;
+                        float d =
+                            dist_any(query, idx->base + (size_t)v * dim, dim, metric, nbr_order);
+                        ++nd;
+                        const float s = metric == ORACLE_IP ? 0.0f - d : d;
+                        if (thr > s) {
+                            cand[nc].id = v, cand[nc].s = s, cand[nc].expanded = 0;
+                            ++nc;
+                        }
+                    }
+                }
+                ++rounds;
+                if (nc == 0) break;
+                hops += nc;
+                memcpy(beam + nb, cand, (size_t)nc * sizeof(bent));
+                if (nb + nc <= L) {
+                    nb += nc;
+                } else {
+                    qsort(beam, (size_t)(nb + nc), sizeof(bent), bent_cmp);
+                    nb = L;
+                    thr = beam[L - 1].s;
+                }
+            }
+            qsort(beam, (size_t)nb, sizeof(bent), bent_cmp);
+            int out = 0;
+            for (int i = 0; i < nb && out < k; ++i) {
+                if (is_deleted(idx->deleted, beam[i].id)) continue;
+                ids[(size_t)qi * k + out] = beam[i].id;
+                if (dists)
+                    dists[(size_t)qi * k + out] = metric == ORACLE_IP ? 0.0f - beam[i].s : beam[i].s;
+                ++out;
+            }
+            for (; out < k; ++out) {
+                ids[(size_t)qi * k + out] = -1;
+                if (dists) dists[(size_t)qi * k + out] = farthest(metric);
+            }
+            if (stats) {
+                stats[(size_t)qi * NSTAT + 0] = (int32_t)hops;
+                stats[(size_t)qi * NSTAT + 1] = (int32_t)ne;
+                stats[(size_t)qi * NSTAT + 2] = (int32_t)nd;
+                stats[(size_t)qi * NSTAT + 3] = (int32_t)rounds;
+            }
+        }
+        free(visited);
+        free(beam);
+        free(cand);
+    }
+    if (time_s) *time_s = now_s() - t0;
+    return 0;
+}
+
+/* tests/test_search_pipeline.cpp:25-39: hits = sum over queries of |gt[0..k) n res[0..k)|,
+ * gt rows are gt_dim apart.  Returns the hit count; recall = hits / (q_num*k). */
+ORACLE_API int64_t oracle_recall_hits(int q_num, int k, int gt_dim, const int32_t* res,
+                                      const int32_t* gt) {
+    int64_t total = 0;
+    for (int i = 0; i < q_num; ++i) {
+        const int32_t* g = gt + (size_t)i * gt_dim;
+        const int32_t* r = res + (size_t)i * k;
+        for (int a = 0; a < k; ++a) {
+            for (int b = 0; b < k; ++b)
+                if (r[b] == g[a]) {
+                    ++total;
+                    break;
+                }
+        }
+    }
+    return total;
+}
+
+/* Exact brute-force kNN under (distance,id), fp64 accumulation then rounded to
+ * fp32: the closed form every approximate result is scored against. */
+ORACLE_API void oracle_bruteforce(const float* base, int64_t n, int dim, const float* queries,
+                                  int Q, int k, int metric, const uint32_t* deleted, int32_t* ids,
+                                  float* dists) {
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int qi = 0; qi < Q; ++qi) {
+        bent* all = (bent*)malloc((size_t)n * sizeof(bent));
+        int64_t m = 0;
+        for (int64_t i = 0; i < n; ++i) {
+            if (is_deleted(deleted, (int32_t)i)) continue;
+            double acc = 0.0;
+            const float *q = queries + (size_t)qi * dim, *b = base + (size_t)i * dim;
+            for (int d = 0; d < dim; ++d)
+                acc += metric == ORACLE_L2 ? ((double)q[d] - b[d]) * ((double)q[d] - b[d])
+                                           : -(double)q[d] * b[d];
+            all[m].id = (int32_t)i, all[m].s = (float)acc, all[m].expanded = 0;
+            ++m;
+        }
+        qsort(all, (size_t)m, sizeof(bent), bent_cmp);
+        for (int j = 0; j < k; ++j) {
+            ids[(size_t)qi * k + j] = j < m ? all[j].id : -1;
+            if (dists)
+                dists[(size_t)qi * k + j] =
+                    j < m ? (metric == ORACLE_IP ? -all[j].s : all[j].s) : farthest(metric);
+        }
+        free(all);
+    }
+}
+
+ORACLE_API int oracle_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
