@@ -21,6 +21,9 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-
 # packed fp32 code generation is switched off for all device code
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
+# host-only translation units: plain C++ that may call the HIP runtime API
+HOST = ["-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include"]
+
 LIB_SOURCES = ["beam_search.hip", "coral_search.cpp", "formats.cpp", "index_gpu.cpp"]
 CLI_SOURCES = ["test_search_pipeline.cpp"]
 
@@ -44,15 +47,14 @@ def build(verbose=True):
             continue
         obj = os.path.join(LIBDIR, src + ".o")
         cmd = [HIPCC] + COMMON + ["-fopenmp", "-fvisibility=hidden", "-DCORAL_BUILD"]
-        cmd += DEVICE if src.endswith(".hip") else ["-x", "hip"] + DEVICE
+        cmd += DEVICE if src.endswith(".hip") else HOST
         _run(cmd + ["-c", path, "-o", obj])
         objs.append(obj)
     _run([HIPCC, "-shared", "-fopenmp", "-o", LIB] + objs)
     for src in CLI_SOURCES:
         path = os.path.join(CSRC, src)
         if os.path.exists(path):
-            _run([HIPCC] + COMMON + ["-x", "hip"] + DEVICE + [path, "-o", CLI, "-L" + LIBDIR, "-lcoral_search",
-                  "-Wl,-rpath,$ORIGIN"])
+            _run([HIPCC] + COMMON + HOST + [path, "-o", CLI, "-L" + LIBDIR, "-lcoral_search", "-Wl,-rpath,$ORIGIN"])
     return LIB
 
 

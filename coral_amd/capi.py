@@ -105,8 +105,8 @@ class Index:
         self.n_start = int(start_ids.size)
 
     def close(self):
-        if getattr(self, "_h", None):
-            lib().coral_index_destroy(self._h)
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.coral_index_destroy(self._h)
             self._h = None
 
     __del__ = close

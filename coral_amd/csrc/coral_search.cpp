@@ -15,13 +15,15 @@
 #include <vector>
 
 #include "beam_search.h"
+#include "error.h"
 
 namespace {
-
 thread_local std::string g_err;
+}
 
+namespace coral {
 int fail(int code, const char* fmt, ...) {
-    char buf[512];
+    char buf[768];
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(buf, sizeof buf, fmt, ap);
@@ -29,6 +31,10 @@ int fail(int code, const char* fmt, ...) {
     g_err = buf;
     return code;
 }
+}  // namespace coral
+
+namespace {
+using coral::fail;
 
 #define HIP_TRY(expr)                                                                       \
     do {                                                                                    \

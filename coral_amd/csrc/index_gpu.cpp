@@ -1,0 +1,221 @@
+// index_gpu.cpp -- efanna2e::IndexGPU over the C ABI (see include/efanna2e/index_gpu.h).
+#include "efanna2e/index_gpu.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cctype>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+#include <stdexcept>
+
+#include "coral_formats.h"
+
+namespace efanna2e {
+
+namespace {
+
+ProConfig g_config;
+
+[[noreturn]] void raise(const char* what) {
+    throw std::runtime_error(std::string(what) + ": " + coral_last_error());
+}
+
+// config.json is one flat object of numbers (config.json:1-40): a scanner for
+// "key": number pairs is all that is needed; unknown keys are ignored like
+// nlohmann's j.value(key, default) ignores them.
+bool json_number(const std::string& text, const char* key, double* out) {
+    const std::string needle = std::string("\"") + key + "\"";
+    size_t p = text.find(needle);
+    if (p == std::string::npos) return false;
+    p = text.find(':', p + needle.size());
+    if (p == std::string::npos) return false;
+    ++p;
+    while (p < text.size() && std::isspace((unsigned char)text[p])) ++p;
+    char* end = nullptr;
+    const double v = std::strtod(text.c_str() + p, &end);
+    if (end == text.c_str() + p) return false;
+    *out = v;
+    return true;
+}
+
+}  // namespace
+
+ProConfig& GetProConfig() { return g_config; }
+
+IndexGPU::IndexGPU(const size_t dimension, const size_t n, Metric m, void* initializer)
+    : dimension_(dimension), nd_(n), metric_enum_(m) {
+    (void)initializer;
+    if (m == COSINE) need_normalize = true;
+}
+
+IndexGPU::~IndexGPU() { RunFree(); }
+
+void IndexGPU::RunFree() {
+    if (index_) coral_index_destroy(index_);
+    index_ = nullptr;
+    std::free(h_base_);
+    h_base_ = nullptr;
+}
+
+void IndexGPU::load_config(const std::string& config_file) {
+    std::ifstream f(config_file == "default" ? "../config.json" : config_file);
+    if (!f.is_open()) {
+        std::cerr << "Cannot open config file, using defaults" << std::endl;
+        return;
+    }
+    std::stringstream ss;
+    ss << f.rdbuf();
+    const std::string text = ss.str();
+    double v;
+    ProConfig& pc = g_config;
+    if (json_number(text, "dim", &v)) pc.dim = (int)v;
+    if (json_number(text, "k", &v)) pc.k = (int)v;
+    if (json_number(text, "max_degree", &v)) pc.max_degree = (int)v;
+    if (json_number(text, "beam_capacity", &v)) pc.beam_capacity = (int)v;
+    if (json_number(text, "batch", &v)) pc.batch = (int)v;
+    if (json_number(text, "test_beam_capacity", &v)) pc.test_beam_capacity = (int)v;
+    if (json_number(text, "search_start_nodes_num", &v)) pc.search_start_nodes_num = (int)v;
+    if (json_number(text, "search_in_cpu", &v)) pc.search_in_cpu = (int)v;
+}
+
+void IndexGPU::LoadSearchNeededData(const char* base_file, const char* sampled_query_file, DIST_METRIC m) {
+    int64_t n = 0;
+    int32_t dim = 0;
+    if (coral_fbin_read_meta(base_file, &n, &dim)) raise("load_meta");
+    if (sampled_query_file && std::strlen(sampled_query_file) != 0) {
+        int64_t nq = 0;
+        int32_t qdim = 0;
+        if (coral_fbin_read_meta(sampled_query_file, &nq, &qdim)) raise("load_meta");
+        if (qdim != dim) throw std::runtime_error("base and query dimension mismatch");
+    }
+    // rows are padded with zeros to a multiple of 4 floats (include/efanna2e/util.h:194-208);
+    // unlike the reference the padded width is then used consistently
+    const int32_t stride = (dim + 3) / 4 * 4;
+    if ((size_t)stride != ((dimension_ + 3) / 4 * 4))
+        throw std::runtime_error("base dimension does not match the index dimension");
+    std::free(h_base_);
+    h_base_ = nullptr;
+    if (posix_memalign((void**)&h_base_, 32, (size_t)n * stride * sizeof(float)) != 0)
+        throw std::runtime_error("out of host memory for the base vectors");
+    if (coral_fbin_read(base_file, h_base_, n, dim, stride)) raise("load_data");
+    if (m == DIST_METRIC::IP_) coral_normalize_l2(h_base_, n, stride);
+    dimension_ = (size_t)stride;
+    nd_ = (size_t)n;
+    metric_ = m;
+}
+
+void IndexGPU::RunPrepare(Parameters& parameters, Mode mode, size_t n_bp, float* bp_data) {
+    if (mode != Mode::SEARCH) throw std::runtime_error("only Mode::SEARCH is provided by this library");
+    SetParameters(parameters);
+    load_config(parameters.Get<std::string>("config_file", std::string("default")));
+    graph_dir_ = parameters.Get<std::string>("graph_file");
+    k_ = parameters.Get<int>("k");
+    max_degree_ = parameters.Get<int>("max_degree");
+    metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
+    if (n_bp > 0) {  // caller-owned vectors (src/index_gpu.cpp:246-251); copied, rows dimension_ wide
+        std::free(h_base_);
+        h_base_ = nullptr;
+        if (posix_memalign((void**)&h_base_, 32, n_bp * dimension_ * sizeof(float)) != 0)
+            throw std::runtime_error("out of host memory for the base vectors");
+        std::memcpy(h_base_, bp_data, n_bp * dimension_ * sizeof(float));
+        nd_ = n_bp;
+    }
+    if (!h_base_) throw std::runtime_error("RunPrepare before LoadSearchNeededData");
+    nbrs_.assign(nd_ * (size_t)max_degree_, -1);
+    if (coral_graph_dir_read(graph_dir_.c_str(), (int64_t)nd_, max_degree_, nbrs_.data(), nullptr))
+        raise("load graph");
+    start_ids_.assign(4096, 0);
+    int32_t m = 0;
+    if (coral_start_ids_read(graph_dir_.c_str(), start_ids_.data(), (int32_t)start_ids_.size(), &m))
+        raise("load start ids");
+    start_ids_.resize((size_t)m);
+    if (start_ids_.empty()) throw std::runtime_error("graph.search_start_ids is missing or empty in " + graph_dir_);
+    coral_index_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.base = h_base_, d.nbrs = nbrs_.data(), d.n = (int64_t)nd_, d.dim = (int32_t)dimension_;
+    d.R = max_degree_, d.start_ids = start_ids_.data(), d.n_start = (int32_t)start_ids_.size();
+    d.metric = metric_ == DIST_METRIC::L2_ ? CORAL_L2 : CORAL_IP, d.device = 0;
+    if (index_) coral_index_destroy(index_);
+    index_ = nullptr;
+    if (coral_index_create(&d, &index_)) raise("create index");
+}
+
+void IndexGPU::LoadRoarGraph(std::string filename) {
+    if (!index_) throw std::runtime_error("LoadRoarGraph before RunPrepare");
+    int32_t ep = 0;
+    if (coral_roargraph_read(filename.c_str(), (int64_t)nd_, max_degree_, nbrs_.data(), &ep)) raise("LoadRoarGraph");
+    start_ids_.assign(1, ep);
+    if (coral_index_set_graph(index_, nbrs_.data(), start_ids_.data(), 1)) raise("LoadRoarGraph");
+}
+
+void IndexGPU::SetDeleted(const uint32_t* mask_words) {
+    if (!index_) throw std::runtime_error("SetDeleted before RunPrepare");
+    if (coral_index_set_deleted(index_, mask_words)) raise("SetDeleted");
+    have_delete_ = mask_words != nullptr;
+}
+
+Test_Result IndexGPU::run(const float* queries, int num, int L, int* ids_res, float* dists_res) {
+    if (!index_) throw std::runtime_error("Search before RunPrepare");
+    coral_stats st;
+    if (coral_search(index_, queries, num, k_, L, policy_, have_delete_ ? 1 : 0, ids_res, dists_res, &st))
+        raise("Search");
+    Test_Result tr(-1, (size_t)st.hops, (float)st.time_s);
+    tr.expansions = (size_t)st.expansions, tr.dist_evals = (size_t)st.dist_evals;
+    tr.rounds = (size_t)st.rounds, tr.spills = (size_t)st.spills;
+    return tr;
+}
+
+Test_Result IndexGPU::Search(const float* queries, int num, int beam_capacity, int* ids_res, int M) {
+    (void)M;  // the reference fills a default and then ignores it too (src/index_gpu.cpp:119,127)
+    return run(queries, num, beam_capacity, ids_res, nullptr);
+}
+
+Test_Result IndexGPU::SearchWithDists(const float* queries, int num, int beam_capacity, int* ids_res,
+                                      float* dists_res) {
+    return run(queries, num, beam_capacity, ids_res, dists_res);
+}
+
+Test_Result IndexGPU::Search_and_Verify(const float* queries, const int* gts, int num, int beam_capacity) {
+    if (!index_) throw std::runtime_error("Search_and_Verify before RunPrepare");
+    const int L = beam_capacity > 0 ? beam_capacity : PC.test_beam_capacity;
+    float* d_q = nullptr;
+    int32_t *d_ids = nullptr, *d_gt = nullptr;
+    const size_t qb = (size_t)num * dimension_ * sizeof(float), ib = (size_t)num * k_ * sizeof(int32_t);
+    auto release = [&]() {
+        (void)hipFree(d_q);
+        (void)hipFree(d_ids);
+        (void)hipFree(d_gt);
+    };
+    if (hipMalloc(&d_q, qb) != hipSuccess || hipMalloc(&d_ids, ib) != hipSuccess ||
+        hipMalloc(&d_gt, ib) != hipSuccess || hipMemcpy(d_q, queries, qb, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(d_gt, gts, ib, hipMemcpyHostToDevice) != hipSuccess) {
+        release();
+        throw std::runtime_error("Search_and_Verify: device allocation or upload failed");
+    }
+    // the reference prepares once per process (a function-local static, src/index_gpu.cpp:101-108)
+    // and breaks if a later call is larger; here a change of (num, L) prepares again
+    if (!verify_prepared_ || verify_Q_ < num || verify_L_ != L) {
+        if (coral_search_prepare(index_, num, L, nullptr)) {
+            release();
+            raise("search_prepare");
+        }
+        verify_prepared_ = true, verify_Q_ = num, verify_L_ = L;
+    }
+    coral_stats st;
+    int64_t hits = 0;
+    if (coral_search_gpu(index_, d_q, d_ids, nullptr, num, k_, policy_, have_delete_ ? 1 : 0, nullptr, &st) ||
+        coral_search_verify(index_, d_ids, d_gt, num, k_, &hits)) {
+        release();
+        raise("Search_and_Verify");
+    }
+    release();
+    Test_Result tr((int)hits, (size_t)st.hops, (float)st.time_s);
+    tr.expansions = (size_t)st.expansions, tr.dist_evals = (size_t)st.dist_evals;
+    tr.rounds = (size_t)st.rounds, tr.spills = (size_t)st.spills;
+    return tr;
+}
+
+}  // namespace efanna2e

@@ -1,0 +1,134 @@
+// efanna2e::IndexGPU -- the search-side surface of the reference's index class
+// (include/index_gpu.h:42-76, src/index_gpu.cpp), implemented on the MI355X path
+// of libcoral_search.so.  A caller written against the reference's
+// test_search_pipeline.cpp:241-292 compiles against this header unchanged:
+//
+//     efanna2e::IndexGPU index(dim, n, efanna2e::L2, nullptr);
+//     index.LoadSearchNeededData(base_file, "", DIST_METRIC::L2_);
+//     index.RunPrepare(parameters, Mode::SEARCH);
+//     Test_Result tr = index.Search(queries, Q, L, ids);
+//
+// Differences, all on purpose:
+//   * the whole index is HBM resident for every N; the reference switches to a
+//     CPU or disk tier above 10.01M / 100M nodes (src/index_gpu.cpp:256-257).
+//     SetPolicy() chooses the traversal instead: ROUNDS (the reference's GPU
+//     kernel) by default, BEST_FIRST (its CPU path) on request;
+//   * build, insert and delete are not part of this library;
+//   * failures throw std::runtime_error with the library's message where the
+//     reference prints and exits (include/utils.cuh:50-58).
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../coral_search.h"
+#include "parameters.h"
+
+enum DIST_METRIC { L2_, IP_, COS_ };  // include/uni.h:93
+
+namespace efanna2e {
+
+enum Metric { L2 = 0, INNER_PRODUCT = 1, FAST_L2 = 2, PQ = 3, COSINE = 4 };  // efanna2e/distance.h:15
+enum Mode { CONS, SEARCH, UPD, CE };                                          // include/uni.h:147
+enum GraphType { GPU, CPU, DISK };                                            // include/uni.h:149
+
+// The keys of config.json that search reads (src/index_gpu.cpp:40-87); defaults
+// are the reference's (include/uni.h:97-132).
+struct ProConfig {
+    int dim = 200;
+    int k = 100;
+    int max_degree = 32;
+    int beam_capacity = 1024;
+    int batch = 1024;
+    int test_beam_capacity = 512;
+    int search_start_nodes_num = 16;
+    int search_in_cpu = 0;
+};
+CORAL_API ProConfig& GetProConfig();
+#define PC (::efanna2e::GetProConfig())
+
+// include/uni.h:411-437
+class CORAL_API Test_Result {
+   public:
+    Test_Result() : recall(0.0f), time(0.0f), hits(0), hops(0) {}
+    Test_Result(const int hits, const size_t hops, const float time)
+        : recall(0.0f), time(time), hits(hits), hops(hops) {}
+    Test_Result(const int hits, const size_t hops) : recall(0.0f), time(0.0f), hits(hits), hops(hops) {}
+    float get_recall() const { return recall; }
+    size_t get_hops() const { return hops; }
+    float get_time() const { return time; }
+    float calc_recall(int total_num) { return recall = 100.0 * hits / total_num; }
+    float avg_hops(int search_num) { return 1.0 * hops / search_num; }
+    void accumulate(const Test_Result& res) {
+        hops += res.hops;
+        time += res.time;
+        hits += res.hits;
+    }
+
+    float recall, time;
+    int hits;
+    size_t hops;
+    // beyond the reference: counters behind the roofline figures of the last call
+    size_t expansions = 0, dist_evals = 0, rounds = 0, spills = 0;
+};
+
+class CORAL_API IndexGPU {
+   public:
+    // `initializer` is kept for signature compatibility and must be nullptr
+    explicit IndexGPU(const size_t dimension, const size_t n, Metric m, void* initializer);
+    ~IndexGPU();
+    IndexGPU(const IndexGPU&) = delete;
+    IndexGPU& operator=(const IndexGPU&) = delete;
+
+    // src/index_gpu.cpp:625-650: reads base_file (.fbin), L2-normalises it for IP_
+    void LoadSearchNeededData(const char* base_file, const char* sampled_query_file,
+                              DIST_METRIC m = DIST_METRIC::L2_);
+    // src/index_gpu.cpp:226-262: reads config_file, graph_file (index directory), k,
+    // max_degree, dist from `parameters`; uploads vectors and graph
+    void RunPrepare(Parameters& parameters, Mode mode, size_t n_bp = 0, float* bp_data = nullptr);
+    void RunFree();
+    void SetParameters(Parameters& parameters) { parameters_ = parameters; }
+    void load_config(const std::string& config_file);
+
+    // src/index_gpu.cpp:117-136; ids_res holds num*k ints, best first
+    Test_Result Search(const float* queries, int num, int beam_capacity, int* ids_res, int M = 0);
+    // src/index_gpu.cpp:89-115; gts holds num*k ints; hits are counted on the device
+    Test_Result Search_and_Verify(const float* queries, const int* gts, int num, int beam_capacity = 0);
+    // src/graph.cu:709-743
+    void LoadRoarGraph(std::string filename);
+
+    // --- beyond the reference ---
+    void SetPolicy(int coral_policy) { policy_ = coral_policy; }
+    // tombstones (src/update.cu:406-412): ceil(n/32) words, or nullptr to clear
+    void SetDeleted(const uint32_t* mask_words);
+    // as Search, also returning distances (num*k floats)
+    Test_Result SearchWithDists(const float* queries, int num, int beam_capacity, int* ids_res,
+                                float* dists_res);
+
+    Metric GetMetric() const { return metric_enum_; }
+    size_t GetDimension() const { return dimension_; }
+    size_t GetSizeOfDataset() const { return nd_; }
+    const float* GetBasePointSet() const { return h_base_; }
+    const std::vector<int>& GetStartIds() const { return start_ids_; }
+    bool need_normalize = false;
+
+   private:
+    Test_Result run(const float* queries, int num, int L, int* ids_res, float* dists_res);
+    size_t dimension_, nd_;
+    Metric metric_enum_;
+    DIST_METRIC metric_ = DIST_METRIC::L2_;
+    Parameters parameters_;
+    int k_ = 0, max_degree_ = 32;
+    int policy_ = CORAL_POLICY_ROUNDS;
+    bool have_delete_ = false;
+    float* h_base_ = nullptr;
+    std::vector<int> start_ids_;
+    std::vector<int32_t> nbrs_;
+    std::string graph_dir_;
+    coral_index* index_ = nullptr;
+    bool verify_prepared_ = false;
+    int verify_Q_ = 0, verify_L_ = 0;
+};
+
+}  // namespace efanna2e

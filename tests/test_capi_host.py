@@ -1,0 +1,109 @@
+"""Host-side checks that need no GPU: the shared library loads, exports every
+symbol the public headers declare, and rejects bad arguments before touching a
+device."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from coral_amd import capi, formats
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = []
+    for h in ("coral_search.h", "coral_formats.h"):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        names += re.findall(r"CORAL_API\s+[\w\s\*]+?\b(coral_\w+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.lib()
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), n
+    bound = set(capi.SIGNATURES) | set(formats.SIGNATURES)
+    assert set(names) == bound
+
+
+def test_cxx_class_symbols_are_exported():
+    out = subprocess.run(["nm", "-DC", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    for sym in ("efanna2e::IndexGPU::Search(float const*, int, int, int*, int)",
+                "efanna2e::IndexGPU::Search_and_Verify(float const*, int const*, int, int)",
+                "efanna2e::IndexGPU::RunPrepare(efanna2e::Parameters&, efanna2e::Mode, unsigned long, float*)",
+                "efanna2e::IndexGPU::LoadSearchNeededData(char const*, char const*, DIST_METRIC)",
+                "efanna2e::IndexGPU::LoadRoarGraph(", "efanna2e::IndexGPU::load_config(",
+                "efanna2e::IndexGPU::RunFree()", "efanna2e::GetProConfig()"):
+        assert sym in out, sym
+
+
+def test_index_create_validates_before_any_device_call():
+    base = np.zeros((10, 8), np.float32)
+    good = np.full((10, 4), -1, np.int32)
+    good[:, 0] = (np.arange(10) + 1) % 10
+
+    def create(base, nbrs, starts, metric=0):
+        try:
+            capi.Index(base, nbrs, starts, metric).close()
+        except capi.CoralError as e:
+            return e.code, str(e)
+        return 0, ""
+
+    bad = good.copy()
+    bad[3, 0] = 10
+    assert create(base, bad, [0])[0] == capi.ERR_GRAPH
+    bad = good.copy()
+    bad[3, 0], bad[3, 1] = -1, 2
+    code, msg = create(base, bad, [0])
+    assert code == capi.ERR_GRAPH and "end-of-row" in msg
+    assert create(base, good, [10])[0] == capi.ERR_GRAPH
+    code, msg = create(base, good, [2, 2])
+    assert code == capi.ERR_GRAPH and "duplicate" in msg
+    assert create(base, good, [])[0] == capi.ERR_ARG
+    assert create(np.zeros((10, 6), np.float32), good, [0])[0] == capi.ERR_ARG  # dim % 4
+    assert create(base, np.full((10, 33), -1, np.int32), [0])[0] == capi.ERR_ARG  # R > 32
+    assert create(base, good, [0], metric=7)[0] == capi.ERR_ARG
+
+
+def test_null_arguments_are_errors_not_crashes():
+    lib = capi.lib()
+    assert lib.coral_index_create(None, None) == capi.ERR_ARG
+    assert lib.coral_search_prepare(None, 1, 1, None) == capi.ERR_ARG
+    assert lib.coral_search_gpu(None, None, None, None, 1, 1, 0, 0, None, None) == capi.ERR_ARG
+    assert lib.coral_search(None, None, 1, 1, 1, 0, 0, None, None, None) == capi.ERR_ARG
+    assert b"null" in lib.coral_last_error()
+    lib.coral_index_destroy(None)
+
+
+CLI = os.path.join(ROOT, "coral_amd", "lib", "test_search_pipeline")
+
+
+def run_cli(*args):
+    return subprocess.run([CLI] + list(args), capture_output=True, text=True)
+
+
+def test_cli_flag_handling():
+    r = run_cli("--help")
+    assert r.returncode == 0
+    for flag in ("--data_type", "--dist", "--base_data_path", "--dataset", "--query_path", "--gt_path", "--L",
+                 "--k", "--max_degree", "--query_thres", "--CE", "--config_file", "--index_type", "--log_file",
+                 "--res_file", "--recall_thres", "--max_recall", "--max_hop"):
+        assert flag in r.stdout
+    r = run_cli("--dist", "l2")
+    assert r.returncode == 255 and "required but missing" in r.stderr  # the reference returns -1
+    r = run_cli("--bogus", "1")
+    assert r.returncode == 255 and "unrecognised option" in r.stderr
+    base = ["--data_type", "float", "--base_data_path", "/nonexistent.fbin", "--dataset", "t", "--query_path",
+            "/nonexistent_q.fbin", "--gt_path", "/nonexistent_gt", "--k", "10", "--L", "32", "64", "-T", "16"]
+    r = run_cli(*base, "--dist", "cosine")
+    assert r.returncode == 255 and "Unknown distance type" in r.stdout
+    r = run_cli(*base, "--dist", "l2")
+    assert r.returncode == 1 and "open file error" in r.stderr
+    r = run_cli(*base, "--dist=l2", "--k", "ten")
+    assert r.returncode == 255

@@ -1,0 +1,60 @@
+"""The headline workload at its real size (1M x 200 fp32, R = 32, 10 000 queries,
+k = 100, L = 256) checked through size-independent properties plus exact parity
+on a subsample that the oracle finishes in seconds."""
+import numpy as np
+import pytest
+
+from coral_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def test_full_size_properties(orc):
+    import torch
+    from concurrent.futures import ThreadPoolExecutor
+    n, dim, Q, k, L = 1000000, 200, 10000, 100, 256
+    base = np.empty((n, dim), np.float32)
+    step = 1 << 15
+    with ThreadPoolExecutor(16) as ex:
+        list(ex.map(lambda r: synth.gaussian_matrix(2001, min(step, n - r), dim, row0=r, out=base[r:r + step]),
+                    range(0, n, step)))
+    q = synth.shifted_queries(Q, dim, 2002, 2003, 2004)
+    print("building the 1M exact 32-NN graph on the GPU", flush=True)
+    nbrs = synth.exact_knn_graph(base, 32, device="cuda", block=4096)
+    starts = np.random.RandomState(1).choice(n, 16, replace=False).astype(np.int32)
+    idx = capi.Index(base, nbrs, starts)
+    print("searching", flush=True)
+    ids, dists, st = idx.search(q, k, L)
+    cnt = idx.query_counters(Q)
+    # sorted, unique, in range, full
+    assert (ids >= 0).all() and (ids < n).all()
+    assert (np.diff(dists, axis=1) >= 0).all()
+    assert all(len(set(r.tolist())) == k for r in ids[::97])
+    # the distances are the distances of the ids (recomputed in fp64 on a stride of queries)
+    for qi in range(0, Q, 501):
+        want = ((base[ids[qi]].astype(np.float64) - q[qi].astype(np.float64)) ** 2).sum(1)
+        assert np.allclose(dists[qi], want, rtol=1e-5)
+    # counters: every query measured its start ids and at least one round; totals add up
+    assert (cnt[:, 2] >= 16).all() and (cnt[:, 3] >= 1).all()
+    assert st.dist_evals == int(cnt[:, 2].astype(np.int64).sum())
+    # idempotence: the same call returns the same bytes
+    ids2, dists2, _ = idx.search(q, k, L)
+    assert np.array_equal(ids, ids2) and dists.tobytes() == dists2.tobytes()
+    # a permutation of the batch permutes the answers
+    perm = np.random.RandomState(0).permutation(Q)
+    ids3, _, _ = idx.search(q[perm], k, L)
+    assert np.array_equal(ids3, ids[perm])
+    # exact parity with the oracle on a subsample
+    sub = np.arange(0, Q, 157)
+    prob = orc.Problem(base, nbrs, starts)
+    oi, od, os_, _ = orc.search_B(prob, q[sub], k, L, start_order=3, nbr_order=3)
+    assert np.array_equal(ids[sub], oi) and dists[sub].tobytes() == od.tobytes()
+    assert np.array_equal(cnt[sub], os_)
+    # device-side recall equals the host-side count against brute-force ground truth
+    tq = torch.from_numpy(q[sub]).cuda()
+    tb = torch.from_numpy(base).cuda()
+    d = (tb * tb).sum(1)[None, :] - 2.0 * (tq @ tb.T)
+    gt = torch.topk(d, k, dim=1, largest=False).indices.to(torch.int32)
+    hits = idx.verify(torch.from_numpy(ids[sub]).cuda().data_ptr(), gt.data_ptr(), len(sub), k)
+    assert hits == orc.recall_hits(ids[sub], gt.cpu().numpy(), k)
+    idx.close()
