@@ -26,12 +26,16 @@ struct SearchArgs {
     int32_t dim, R, M, Q, k, L;
     int32_t metric;            // 0 = L2, 1 = IP
     int32_t policy;            // 0 = rounds, 1 = best first
-    int32_t slots_log2;        // LDS visited table size
-    int32_t vis_limit;         // inserts after which the table is frozen
+    int32_t slots_log2;        // LDS visited table: number of 16-bit cells
+    int32_t vis_limit;         // first visits after which the table takes no more inserts
+    int32_t id_bits;           // ceil(log2 n): width of the id mixing bijection
+    int32_t rem_bits;          // low bits of the mixed id kept in a cell
+    int32_t dmax;              // largest displacement a cell can encode (-1: table unused)
+    int32_t ocap;              // LDS list of ids sent to the global bitmap (multiple of 4)
     int32_t tcap, ccap;        // LDS todo / candidate capacities (multiples of 4, ccap >= tcap)
 };
 
-size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap);
+size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap, int ocap);
 hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu);
 hipError_t launch_search(const SearchArgs& a, int workgroups, int threads, size_t lds_bytes,
                          hipStream_t stream);

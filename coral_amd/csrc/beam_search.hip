@@ -28,7 +28,6 @@
 
 namespace coral {
 
-constexpr uint32_t kEmpty = 0xFFFFFFFFu;
 constexpr uint64_t kKeyMax = ~0ull;
 
 // float -> uint32 whose unsigned order is the float order
@@ -47,40 +46,69 @@ __device__ __forceinline__ uint64_t make_key(float s, int32_t id, uint32_t flag)
 __device__ __forceinline__ int32_t key_id(uint64_t k) { return (int32_t)((uint32_t)k >> 1); }
 __device__ __forceinline__ float key_s(uint64_t k) { return unord32((uint32_t)(k >> 32)); }
 
-__device__ __forceinline__ uint32_t hash_slot(uint32_t id, int shift) {
-    return (id * 0x9E3779B1u) >> shift;
-}
+// The visited set of one query.
+//
+// First level, in LDS: an open-addressing table of 16-bit cells.  A node id is
+// mixed by a bijection on its b = ceil(log2 n) bits; the high bits of the result
+// pick the home cell and only the remaining `rb` low bits (the remainder) are
+// stored, together with the displacement d of the cell from its home:
+//     cell = 1 + ((d << rb) | remainder),   0 = empty.
+// (cell index, d, remainder) determine the mixed value and hence the id, so the
+// table is exact; it holds twice the ids a table of 32-bit ids would.  Probing is
+// linear and bounded by dmax (the largest d the 16 bits can carry).
+// Second level, in global memory: this workgroup's n-bit bitmap, used for ids
+// that find no cell within dmax and for every new id once the table has been
+// frozen (load limit reached).  Ids sent there are remembered in a short LDS list
+// so that the bitmap can be cleaned word by word when the query ends.
+struct VisitedSet {
+    uint32_t* words;   // LDS: slots/2 words
+    uint32_t* olist;   // LDS: ids that went to the bitmap
+    int* ocount;       // LDS: how many did (may exceed ocap)
+    uint32_t* bitmap;  // global
+    uint32_t smask, bmask, rmask;
+    int rb, xs, dmax, ocap;
 
-// 1 if id was not in the table (and is now), 0 if it was there
-__device__ __forceinline__ int visit_lds(uint32_t* table, uint32_t mask, int shift, uint32_t id) {
-    uint32_t h = hash_slot(id, shift);
-    for (;;) {
-        const uint32_t x = table[h];
-        if (x == id) return 0;
-        if (x == kEmpty) {
-            const uint32_t old = atomicCAS(&table[h], kEmpty, id);
-            if (old == kEmpty) return 1;
-            if (old == id) return 0;
+    __device__ __forceinline__ uint32_t mix(uint32_t id) const {
+        uint32_t h = (id * 0x9E3779B1u) & bmask;
+        h ^= h >> xs;
+        h = (h * 0x85EBCA6Bu) & bmask;
+        h ^= h >> xs;
+        return h;
+    }
+
+    // 1 if id was not yet in the set (and now is), 0 if it was
+    __device__ __forceinline__ int test_and_set(uint32_t id, bool frozen) {
+        const uint32_t h = mix(id);
+        const uint32_t home = h >> rb, rem = h & rmask;
+        const uint16_t* cells = reinterpret_cast<const uint16_t*>(words);
+        for (int d = 0; d <= dmax; ++d) {
+            const uint32_t s = (home + (uint32_t)d) & smask;
+            const uint32_t want = 1u + (((uint32_t)d << rb) | rem);
+            uint32_t cur = cells[s];
+            if (cur == want) return 0;
+            if (cur == 0u) {
+                if (frozen) break;
+                uint32_t* w = words + (s >> 1);
+                const int sh = (int)(s & 1u) * 16;
+                uint32_t old = *w;
+                for (;;) {
+                    cur = (old >> sh) & 0xffffu;
+                    if (cur != 0u) break;
+                    const uint32_t prev = atomicCAS(w, old, old | (want << sh));
+                    if (prev == old) return 1;
+                    old = prev;
+                }
+                if (cur == want) return 0;
+            }
         }
-        h = (h + 1) & mask;
+        const uint32_t bit = 1u << (id & 31);
+        const uint32_t old = atomicOr(&bitmap[id >> 5], bit);
+        if (old & bit) return 0;
+        const int p = atomicAdd(ocount, 1);
+        if (p < ocap) olist[p] = id;
+        return 1;
     }
-}
-
-// after the LDS table stopped taking inserts: look it up, then test-and-set the
-// workgroup's bitmap in global memory
-__device__ __forceinline__ int visit_spill(const uint32_t* table, uint32_t mask, int shift,
-                                           uint32_t* bitmap, uint32_t id) {
-    uint32_t h = hash_slot(id, shift);
-    for (;;) {
-        const uint32_t x = table[h];
-        if (x == id) return 0;
-        if (x == kEmpty) break;
-        h = (h + 1) & mask;
-    }
-    const uint32_t bit = 1u << (id & 31);
-    const uint32_t old = atomicOr(&bitmap[id >> 5], bit);
-    return (old & bit) == 0;
-}
+};
 
 // number of set bits of m below the calling lane
 __device__ __forceinline__ int prefix_popc(uint64_t m) {
@@ -107,28 +135,32 @@ struct WgState {
 };
 
 template <int G, int CPL>
-__global__ __launch_bounds__(512) void beam_search_kernel(const SearchArgs a) {
+__global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, NT = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, NW = NT >> 6;
     const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2;
     const int Lp = (L + 3) & ~3;
     const int slots = 1 << a.slots_log2;
-    const uint32_t hmask = (uint32_t)slots - 1u;
-    const int hshift = 32 - a.slots_log2;
     const int TCAP = a.tcap, CCAP = a.ccap;
 
     uint64_t* beam0 = (uint64_t*)smem;
     uint64_t* beam1 = beam0 + Lp;
     uint64_t* cand = beam1 + Lp;
-    uint32_t* table = (uint32_t*)(cand + CCAP);
-    uint32_t* todo = table + slots;
+    uint32_t* table = (uint32_t*)(cand + CCAP);  // slots 16-bit cells
+    uint32_t* todo = table + (slots >> 1);
     uint32_t* elist = todo + TCAP;
-    float* qs = (float*)(elist + Lp);
+    uint32_t* olist = elist + Lp;
+    float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_ne, s_first, s_outpos;
+    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_ne, s_first, s_outpos, s_nover;
 
-    uint32_t* bitmap = a.spill + (size_t)blockIdx.x * a.spill_words;
+    VisitedSet vs;
+    vs.words = table, vs.olist = olist, vs.ocount = &s_nover;
+    vs.bitmap = a.spill + (size_t)blockIdx.x * a.spill_words;
+    vs.smask = (uint32_t)slots - 1u, vs.bmask = a.id_bits >= 32 ? 0xffffffffu : (1u << a.id_bits) - 1u;
+    vs.rb = a.rem_bits, vs.rmask = (1u << a.rem_bits) - 1u;
+    vs.xs = a.id_bits > 1 ? a.id_bits / 2 : 1, vs.dmax = a.dmax, vs.ocap = a.ocap;
 
     constexpr int GPW = 64 / G;                    // row groups per wave
     constexpr int U = (CPL >= 8) ? 1 : (8 / CPL);  // rows in flight per group
@@ -142,9 +174,9 @@ __global__ __launch_bounds__(512) void beam_search_kernel(const SearchArgs a) {
         const int qid = s_qid;
         if (qid >= a.Q) break;
 
-        for (int i = tid; i < slots; i += NT) table[i] = kEmpty;
+        for (int i = tid; i < (slots >> 1); i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
-        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_ne = 0;
+        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_ne = 0, s_nover = 0;
         __syncthreads();
 
         float4 qreg[CPL];
@@ -272,7 +304,7 @@ __global__ __launch_bounds__(512) void beam_search_kernel(const SearchArgs a) {
         const int M = a.M;
         for (int i = tid; i < M; i += NT) {
             const uint32_t id = (uint32_t)a.start_ids[i];
-            visit_lds(table, hmask, hshift, id);
+            vs.test_and_set(id, false);
             todo[i] = id;
         }
         __syncthreads();
@@ -341,9 +373,7 @@ __global__ __launch_bounds__(512) void beam_search_kernel(const SearchArgs a) {
                         head = j == 0;
                     }
                     bool isnew = false;
-                    if (v >= 0)
-                        isnew = spill ? visit_spill(table, hmask, hshift, bitmap, (uint32_t)v)
-                                      : visit_lds(table, hmask, hshift, (uint32_t)v);
+                    if (v >= 0) isnew = vs.test_and_set((uint32_t)v, spill) != 0;
                     const uint64_t mh = __ballot(head);
                     const uint64_t m = __ballot(isnew);
                     if (lane == 0 && mh) atomicAdd(&s_ne, __popcll(mh));
@@ -422,11 +452,16 @@ __global__ __launch_bounds__(512) void beam_search_kernel(const SearchArgs a) {
             if (tid == 0) {
                 int32_t* c = a.counters + (size_t)qid * 4;
                 c[0] = hops, c[1] = s_ne, c[2] = nd, c[3] = rounds;
-                if (spill) atomicAdd(a.spill_count, 1);
+                if (s_nover > 0) atomicAdd(a.spill_count, 1);
             }
-            if (spill) {
-                for (size_t i = tid; i < a.spill_words; i += NT) bitmap[i] = 0u;
+            // leave the global bitmap clean: word by word from the list, or all of it
+            const int nover = s_nover;
+            if (nover > a.ocap) {
+                for (size_t i = tid; i < a.spill_words; i += NT) vs.bitmap[i] = 0u;
+            } else {
+                for (int i = tid; i < nover; i += NT) atomicExch(&vs.bitmap[olist[i] >> 5], 0u);
             }
+            if (nover > 0) __threadfence();
         }
     }
 }
@@ -476,10 +511,10 @@ static kernel_fn pick_kernel(int dim) {
     return nullptr;
 }
 
-size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap) {
+size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap, int ocap) {
     const size_t Lp = (size_t)((L + 3) & ~3);
-    return Lp * 8 * 2 + (size_t)ccap * 8 + ((size_t)4 << slots_log2) + (size_t)tcap * 4 + Lp * 4 +
-           (size_t)((dim + 3) & ~3) * 4;
+    return Lp * 8 * 2 + (size_t)ccap * 8 + ((size_t)2 << slots_log2) + (size_t)tcap * 4 + Lp * 4 +
+           (size_t)ocap * 4 + (size_t)((dim + 3) & ~3) * 4;
 }
 
 hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu) {

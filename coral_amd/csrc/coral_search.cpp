@@ -64,7 +64,8 @@ struct coral_index {
     // state of search_prepare
     bool prepared = false;
     int Q = 0, L = 0;
-    int slots_log2 = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 256, workgroups = 0;
+    int slots_log2 = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
+    int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0;
     size_t lds_bytes = 0;
     size_t spill_words = 0;
     uint32_t* d_spill = nullptr;
@@ -243,38 +244,40 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     coral_tuning t;
     std::memset(&t, 0, sizeof t);
     if (tuning) t = *tuning;
-    int threads = t.threads ? t.threads : 256;
-    if (threads != 128 && threads != 256 && threads != 512)
-        return fail(CORAL_ERR_ARG, "threads must be 128, 256 or 512");
     HIP_TRY(hipSetDevice(idx->device));
     HIP_TRY(hipStreamSynchronize(idx->stream));
 
     // todo / candidate buffers: room for the rows of 16 beam entries
     int tcap = std::max(512, ((idx->M + 3) & ~3));
     tcap = std::max(tcap, idx->R * 4);
-    int ccap = tcap;
+    const int ccap = tcap, ocap = 256;
+    int id_bits = 1;
+    while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
     int slots_log2 = t.visited_slots_log2;
     if (slots_log2 == 0) {
-        // degree-32 graphs visit about 30 nodes per beam entry; 48 slots per entry keep
-        // the load factor near one half; shrink only if LDS cannot hold the table
+        // a degree-32 graph over a million nodes sees about 75 first visits per beam
+        // entry; 112 cells per entry keep the load factor near 0.65
         slots_log2 = 12;
-        while ((1 << slots_log2) < 48 * L && slots_log2 < 15) ++slots_log2;
-        while (slots_log2 > 11 &&
-               coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap) + 64 > (size_t)kMaxLdsBytes)
+        while ((1 << slots_log2) < 112 * L && slots_log2 < 16) ++slots_log2;
+        while (slots_log2 > 12 &&
+               coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap, ocap) + 64 > (size_t)kMaxLdsBytes)
             --slots_log2;
     }
-    if (slots_log2 < 11 || slots_log2 > 15)
-        return fail(CORAL_ERR_ARG, "visited_slots_log2 must be in 11..15");
+    if (slots_log2 < 10 || slots_log2 > 16)
+        return fail(CORAL_ERR_ARG, "visited_slots_log2 must be in 10..16");
     const int slots = 1 << slots_log2;
-    if (idx->M + tcap + 1 >= slots)
-        return fail(CORAL_ERR_ARG, "visited table of %d slots too small for %d start ids", slots,
-                    idx->M);
-    int vis_limit = std::min(slots - tcap - 1, slots - slots / 8);
-    if (vis_limit < idx->M) vis_limit = idx->M;
-    const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap);
+    const int rem_bits = std::max(0, id_bits - slots_log2);
+    // a cell is 1 + ((d << rem_bits) | remainder) in 16 bits
+    int dmax = rem_bits >= 16 ? -1 : std::min(63, (65535 >> rem_bits) - 1);
+    const int vis_limit = dmax < 0 ? 0 : slots - slots / 4;
+    const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap, ocap);
     if (lds + 64 > (size_t)kMaxLdsBytes)
-        return fail(CORAL_ERR_ARG, "L=%d with a %d-slot visited table needs %zu bytes of LDS", L, slots,
+        return fail(CORAL_ERR_ARG, "L=%d with a %d-cell visited table needs %zu bytes of LDS", L, slots,
                     lds);
+    int threads = t.threads;
+    if (threads == 0) threads = lds + 64 > (size_t)kMaxLdsBytes / 2 ? 1024 : 512;
+    if (threads != 128 && threads != 256 && threads != 512 && threads != 1024)
+        return fail(CORAL_ERR_ARG, "threads must be 128, 256, 512 or 1024");
     int wg_per_cu = 0;
     HIP_TRY(coral::search_kernel_prepare(idx->dim, lds, threads, &wg_per_cu));
     if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
@@ -302,6 +305,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     HIP_TRY(hipStreamSynchronize(idx->stream));
     idx->Q = Q, idx->L = L, idx->slots_log2 = slots_log2, idx->vis_limit = vis_limit;
     idx->tcap = tcap, idx->ccap = ccap, idx->threads = threads, idx->workgroups = workgroups;
+    idx->id_bits = id_bits, idx->rem_bits = rem_bits, idx->dmax = dmax, idx->ocap = ocap;
     idx->lds_bytes = lds, idx->spill_words = spill_words;
     idx->prepared = true;
     return CORAL_OK;
@@ -334,6 +338,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     a.metric = idx->metric, a.policy = policy;
     a.slots_log2 = idx->slots_log2, a.vis_limit = idx->vis_limit;
     a.tcap = idx->tcap, a.ccap = idx->ccap;
+    a.id_bits = idx->id_bits, a.rem_bits = idx->rem_bits, a.dmax = idx->dmax, a.ocap = idx->ocap;
 
     hipEvent_t ev0, ev1;
     HIP_TRY(hipEventCreate(&ev0));

@@ -88,9 +88,9 @@ typedef struct {
 
 /* Optional launch tuning; zero-initialise for defaults. */
 typedef struct {
-    int32_t visited_slots_log2; /* LDS visited table size; 0 = chosen from L */
+    int32_t visited_slots_log2; /* LDS visited table: log2 of its 16-bit cells, 10..16; 0 = chosen from L */
     int32_t workgroups;         /* persistent workgroups; 0 = chosen from Q and the device */
-    int32_t threads;            /* threads per workgroup: 0 (=256), 128, 256 or 512 */
+    int32_t threads;            /* threads per workgroup: 128, 256, 512 or 1024; 0 = chosen from the LDS need */
     int32_t reserved[5];
 } coral_tuning;
 
