@@ -9,7 +9,8 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libcoral_search.so")
+# CORAL_SEARCH_LIB points at another build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("CORAL_SEARCH_LIB") or os.path.join(HERE, "lib", "libcoral_search.so")
 
 L2, IP = 0, 1
 POLICY_ROUNDS, POLICY_BEST_FIRST = 0, 1
@@ -30,7 +31,7 @@ class IndexDesc(C.Structure):
 
 
 class Stats(C.Structure):
-    _fields_ = [("time_s", C.c_double), ("hops", C.c_int64), ("expansions", C.c_int64),
+    _fields_ = [("time_s", C.c_double), ("kernel_s", C.c_double), ("hops", C.c_int64), ("expansions", C.c_int64),
                 ("dist_evals", C.c_int64), ("rounds", C.c_int64), ("spills", C.c_int64)]
 
     def as_dict(self):

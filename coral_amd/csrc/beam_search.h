@@ -21,6 +21,7 @@ struct SearchArgs {
     uint32_t* spill;           // [workgroups][spill_words] zeroed bitmaps
     int* next_qid;             // work counter, zero at launch
     int* spill_count;          // queries that left LDS, zero at launch
+    unsigned long long* phase_ticks;  // debug builds: 8 per-phase tick sums, else nullptr
     size_t spill_words;        // ceil(n/32)
     int64_t n;
     int32_t dim, R, M, Q, k, L;

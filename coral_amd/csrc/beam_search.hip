@@ -28,6 +28,28 @@
 
 namespace coral {
 
+// Optional per-phase cycle accounting (debug builds only; thread 0 of each workgroup).
+#ifdef CORAL_PHASE_TIMERS
+#define PHASE_DECL unsigned long long ph_t = wall_clock64(), ph_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define PHASE_MARK(i)                          \
+    do {                                       \
+        if (tid == 0) {                        \
+            unsigned long long n_ = wall_clock64(); \
+            ph_acc[i] += n_ - ph_t;            \
+            ph_t = n_;                         \
+        }                                      \
+    } while (0)
+#define PHASE_FLUSH()                                                             \
+    do {                                                                          \
+        if (tid == 0 && a.phase_ticks)                                            \
+            for (int i_ = 0; i_ < 8; ++i_) atomicAdd(&a.phase_ticks[i_], ph_acc[i_]); \
+    } while (0)
+#else
+#define PHASE_DECL
+#define PHASE_MARK(i)
+#define PHASE_FLUSH()
+#endif
+
 constexpr uint64_t kKeyMax = ~0ull;
 
 // float -> uint32 whose unsigned order is the float order
@@ -153,7 +175,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     uint32_t* olist = elist + Lp;
     float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_ne, s_first, s_outpos, s_nover;
+    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_first, s_outpos, s_nover;
 
     VisitedSet vs;
     vs.words = table, vs.olist = olist, vs.ocount = &s_nover;
@@ -173,10 +195,11 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         __syncthreads();
         const int qid = s_qid;
         if (qid >= a.Q) break;
+        PHASE_DECL;
 
         for (int i = tid; i < (slots >> 1); i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
-        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_ne = 0, s_nover = 0;
+        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0;
         __syncthreads();
 
         float4 qreg[CPL];
@@ -189,7 +212,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         WgState st;
         st.nb = 0, st.cur = 0, st.live = kKeyMax;
         float thr = 3.402823466e+38f;  // signed form of the farthest sentinel
-        int hops = 0, nd = 0, rounds = 0;
+        int hops = 0, nd = 0, ne = 0, rounds = 0;
         bool spill = false;
 
         // ---- distance phase: todo[0..T) -> cand[], counting passes of the frozen threshold
@@ -300,6 +323,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             __syncthreads();
         };
 
+        PHASE_MARK(0);
         // ---- seeds: every start id is visited and measured, none counts as a hop
         const int M = a.M;
         for (int i = tid; i < M; i += NT) {
@@ -310,6 +334,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         __syncthreads();
         distance_phase(M);
         merge();
+        PHASE_MARK(1);
         if (tid == 0) s_nvis = M, s_cntf = 0;
         nd = M;
         if (a.policy == 1) hops = M;
@@ -354,29 +379,30 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             }
             __syncthreads();
             const int nexp = s_nexp;
+            PHASE_MARK(2);
             if (nexp == 0) break;
 
-            const int ech = TCAP / R;  // beam entries whose rows fit the todo list
+            // The round's rows are taken in chunks of `ech` beam entries (what the todo
+            // list holds).  Requesting the next chunk's neighbour ids ahead of time was
+            // measured and lost to this plain form: with two workgroups per CU the other
+            // workgroup already covers the wait for the graph rows.
+            const int ech = TCAP / R;
+            ne += nexp;
             for (int e0 = 0; e0 < nexp; e0 += ech) {
-                const int ecount = min(ech, nexp - e0);
                 if (!spill && s_nvis > a.vis_limit) spill = true;
                 if (tid == 0) s_ntodo = 0;
                 __syncthreads();
-                const int total = ecount * R;
+                const int total = min(ech, nexp - e0) * R;
                 for (int f0 = 0; f0 < total; f0 += NT) {
                     const int f = f0 + tid;
                     int v = -1;
-                    bool head = false;
                     if (f < total) {
-                        const int e = f / R, j = f - e * R;
-                        v = a.nbrs[(size_t)elist[e0 + e] * R + j];
-                        head = j == 0;
+                        const int e = f / R;
+                        v = a.nbrs[(size_t)elist[e0 + e] * R + (f - e * R)];
                     }
                     bool isnew = false;
                     if (v >= 0) isnew = vs.test_and_set((uint32_t)v, spill) != 0;
-                    const uint64_t mh = __ballot(head);
                     const uint64_t m = __ballot(isnew);
-                    if (lane == 0 && mh) atomicAdd(&s_ne, __popcll(mh));
                     if (m) {
                         int pos = 0;
                         if (lane == 0) pos = atomicAdd(&s_ntodo, __popcll(m));
@@ -387,10 +413,13 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 __syncthreads();
                 const int T = s_ntodo;
                 nd += T;
+                PHASE_MARK(3);
                 if (s_ncand + T > CCAP) merge();  // merge() starts and ends with a barrier
+                PHASE_MARK(5);
                 if (tid == 0) s_nvis += T;
                 distance_phase(T);
                 __syncthreads();
+                PHASE_MARK(4);
             }
             ++rounds;
             const int cntf = s_cntf;
@@ -401,6 +430,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 hops += 1;
             }
             merge();
+            PHASE_MARK(5);
             if (tid == 0) s_cntf = 0;
             if (a.policy == 0 && nb0 + cntf > L) thr = key_s((st.cur ? beam1 : beam0)[L - 1]);
         }
@@ -451,7 +481,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             }
             if (tid == 0) {
                 int32_t* c = a.counters + (size_t)qid * 4;
-                c[0] = hops, c[1] = s_ne, c[2] = nd, c[3] = rounds;
+                c[0] = hops, c[1] = ne, c[2] = nd, c[3] = rounds;
                 if (s_nover > 0) atomicAdd(a.spill_count, 1);
             }
             // leave the global bitmap clean: word by word from the list, or all of it
@@ -462,6 +492,8 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 for (int i = tid; i < nover; i += NT) atomicExch(&vs.bitmap[olist[i] >> 5], 0u);
             }
             if (nover > 0) __threadfence();
+            PHASE_MARK(6);
+            PHASE_FLUSH();
         }
     }
 }

@@ -74,6 +74,7 @@ struct coral_index {
     size_t counters_alloc = 0;
     int* d_scalars = nullptr;  // [0] next_qid, [1] spill_count
     unsigned long long* d_hit = nullptr;
+    unsigned long long* d_phase = nullptr;  // debug builds only
     int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
     int last_Q = 0;
 };
@@ -183,6 +184,7 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_counters);
     (void)hipFree(idx->d_scalars);
     (void)hipFree(idx->d_hit);
+    (void)hipFree(idx->d_phase);
     if (idx->h_counters) (void)hipHostFree(idx->h_counters);
     if (idx->stream) (void)hipStreamDestroy(idx->stream);
     delete idx;
@@ -247,10 +249,11 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     HIP_TRY(hipSetDevice(idx->device));
     HIP_TRY(hipStreamSynchronize(idx->stream));
 
-    // todo / candidate buffers: room for the rows of 16 beam entries
-    int tcap = std::max(512, ((idx->M + 3) & ~3));
-    tcap = std::max(tcap, idx->R * 4);
-    const int ccap = tcap, ocap = 256;
+    // todo / candidate buffers: sized below, once the visited table is known
+    int min_cap = 256;
+    while (min_cap < idx->M || min_cap < idx->R * 4) min_cap <<= 1;
+    int tcap = min_cap;
+    const int ocap = 256;
     int id_bits = 1;
     while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
     int slots_log2 = t.visited_slots_log2;
@@ -260,7 +263,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         slots_log2 = 12;
         while ((1 << slots_log2) < 112 * L && slots_log2 < 16) ++slots_log2;
         while (slots_log2 > 12 &&
-               coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap, ocap) + 64 > (size_t)kMaxLdsBytes)
+               coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap) + 64 > (size_t)kMaxLdsBytes)
             --slots_log2;
     }
     if (slots_log2 < 10 || slots_log2 > 16)
@@ -270,14 +273,26 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // a cell is 1 + ((d << rem_bits) | remainder) in 16 bits
     int dmax = rem_bits >= 16 ? -1 : std::min(63, (65535 >> rem_bits) - 1);
     const int vis_limit = dmax < 0 ? 0 : slots - slots / 4;
-    const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, ccap, ocap);
-    if (lds + 64 > (size_t)kMaxLdsBytes)
+    // Larger chunks mean fewer latency-bound steps per round: take the largest todo /
+    // candidate capacity that does not lower the number of workgroups a CU can hold.
+    auto lds_for = [&](int cap) { return coral::search_lds_bytes(L, idx->dim, slots_log2, cap, cap, ocap) + 64; };
+    if (lds_for(min_cap) > (size_t)kMaxLdsBytes)
         return fail(CORAL_ERR_ARG, "L=%d with a %d-cell visited table needs %zu bytes of LDS", L, slots,
-                    lds);
+                    lds_for(min_cap));
+    const int wg_fit = (int)((size_t)kMaxLdsBytes / lds_for(min_cap));
+    // (capacities are powers of two: the candidate buffer is bitonic-sorted in place)
+    for (int cap : {1024, 512}) {
+        if (cap <= tcap) break;
+        if (lds_for(cap) <= (size_t)kMaxLdsBytes && (int)((size_t)kMaxLdsBytes / lds_for(cap)) >= std::min(wg_fit, 2)) {
+            tcap = cap;
+            break;
+        }
+    }
     int threads = t.threads;
-    if (threads == 0) threads = lds + 64 > (size_t)kMaxLdsBytes / 2 ? 1024 : 512;
+    if (threads == 0) threads = lds_for(tcap) > (size_t)kMaxLdsBytes / 2 ? 1024 : 512;
     if (threads != 128 && threads != 256 && threads != 512 && threads != 1024)
         return fail(CORAL_ERR_ARG, "threads must be 128, 256, 512 or 1024");
+    const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap);
     int wg_per_cu = 0;
     HIP_TRY(coral::search_kernel_prepare(idx->dim, lds, threads, &wg_per_cu));
     if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
@@ -304,7 +319,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     }
     HIP_TRY(hipStreamSynchronize(idx->stream));
     idx->Q = Q, idx->L = L, idx->slots_log2 = slots_log2, idx->vis_limit = vis_limit;
-    idx->tcap = tcap, idx->ccap = ccap, idx->threads = threads, idx->workgroups = workgroups;
+    idx->tcap = tcap, idx->ccap = tcap, idx->threads = threads, idx->workgroups = workgroups;
     idx->id_bits = id_bits, idx->rem_bits = rem_bits, idx->dmax = dmax, idx->ocap = ocap;
     idx->lds_bytes = lds, idx->spill_words = spill_words;
     idx->prepared = true;
@@ -340,29 +355,50 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     a.tcap = idx->tcap, a.ccap = idx->ccap;
     a.id_bits = idx->id_bits, a.rem_bits = idx->rem_bits, a.dmax = idx->dmax, a.ocap = idx->ocap;
 
-    hipEvent_t ev0, ev1;
+    hipEvent_t ev0, evk, ev1;
     HIP_TRY(hipEventCreate(&ev0));
+    HIP_TRY(hipEventCreate(&evk));
     HIP_TRY(hipEventCreate(&ev1));
     HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_scalars, 4, 0u, stream));
+#ifdef CORAL_PHASE_TIMERS
+    if (!idx->d_phase) HIP_TRY(hipMalloc(&idx->d_phase, 8 * sizeof(unsigned long long)));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_phase, 16, 0u, stream));
+    a.phase_ticks = idx->d_phase;
+#endif
     // timed region, same scope as the reference: kernel + counter read-back
     HIP_TRY(hipEventRecord(ev0, stream));
     const int wgs = std::min(idx->workgroups, (int)Q);
     HIP_TRY(coral::launch_search(a, wgs, idx->threads, idx->lds_bytes, stream));
+    HIP_TRY(hipEventRecord(evk, stream));
     HIP_TRY(hipMemcpyAsync(idx->h_counters, idx->d_counters, (size_t)Q * 4 * sizeof(int32_t),
                            hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipEventRecord(ev1, stream));
     HIP_TRY(hipEventSynchronize(ev1));
-    float ms = 0.f;
+    float ms = 0.f, ms_kernel = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
+    HIP_TRY(hipEventElapsedTime(&ms_kernel, ev0, evk));
     (void)hipEventDestroy(ev0);
+    (void)hipEventDestroy(evk);
     (void)hipEventDestroy(ev1);
     int scal[2] = {0, 0};
     HIP_TRY(hipMemcpyAsync(scal, idx->d_scalars, sizeof scal, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
+#ifdef CORAL_PHASE_TIMERS
+    {
+        unsigned long long t[8];
+        HIP_TRY(hipMemcpy(t, idx->d_phase, sizeof t, hipMemcpyDeviceToHost));
+        double sum = 0;
+        for (int i = 0; i < 7; ++i) sum += (double)t[i];
+        std::fprintf(stderr, "[phase %%] init %.1f seeds %.1f elist %.1f expand %.1f distance %.1f merge %.1f output %.1f\n",
+                     100 * t[0] / sum, 100 * t[1] / sum, 100 * t[2] / sum, 100 * t[3] / sum, 100 * t[4] / sum,
+                     100 * t[5] / sum, 100 * t[6] / sum);
+    }
+#endif
     idx->last_Q = Q;
     if (stats) {
         std::memset(stats, 0, sizeof *stats);
         stats->time_s = ms / 1000.0;
+        stats->kernel_s = ms_kernel / 1000.0;
         for (int q = 0; q < Q; ++q) {
             const int32_t* c = idx->h_counters + (size_t)q * 4;
             stats->hops += c[0], stats->expansions += c[1];

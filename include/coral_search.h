@@ -79,6 +79,7 @@ typedef struct {
  * per-query counters, measured with a HIP event pair on the search stream. */
 typedef struct {
     double time_s;
+    double kernel_s;     /* the search kernel alone (HIP event pair around the launch) */
     int64_t hops;        /* what Test_Result.hops holds for this policy */
     int64_t expansions;  /* graph rows read */
     int64_t dist_evals;  /* vector rows read (first visits + start ids) */
