@@ -24,8 +24,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch seen by the memory-side counters (rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE, scaled by what the same counters read for a plain copy kernel);
-# measured offline, see the kernel's summary under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {256: None, 512: None}
+# measured offline (profiles/beam_search_kernel_1Mx200_L*.md; FETCH_SIZE reads half the bytes of a
+# 1 GiB copy on this GPU, so its factor is 2.0; WRITE_SIZE's is 1.0).  None = not measured.
+MEASURED_TRAFFIC_BYTES = {256: 1.5782e+11, 512: 3.2219e+11}
 
 
 def algorithmic_bytes(expansions, dist_evals, Q, dim, k, R=32):
@@ -122,6 +123,13 @@ def main():
     if also:
         out["also"] = {k2: also[k2] for k2 in ("L", "qps", "recall", "kernel_ms", "gbps", "ms_per_step", "spills")}
         out["also"]["frac"] = also["gbps"] / HBM_PEAK_GBPS
+
+    # the IndexGPU::Search shape: host buffers in and out (device allocation, query upload,
+    # search, id download); reported beside the headline, never as the headline
+    idx.search(queries, k, head["L"], want_dists=False)
+    t = time.perf_counter()
+    idx.search(queries, k, head["L"], want_dists=False)
+    out["host_buffers_qps"] = Q / (time.perf_counter() - t)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w, gt, head["L"], k)
