@@ -40,7 +40,7 @@ class Stats(C.Structure):
 
 class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
-                ("reserved", C.c_int32 * 5)]
+                ("policy", C.c_int32), ("reserved", C.c_int32 * 4)]
 
 
 _lib = None
@@ -129,8 +129,8 @@ class Index:
             raise ValueError("mask must hold ceil(n/32) words")
         _check(lib().coral_index_set_deleted(self._h, _ptr(m)))
 
-    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0):
-        t = Tuning(visited_slots_log2, workgroups, threads)
+    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS):
+        t = Tuning(visited_slots_log2, workgroups, threads, policy)
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

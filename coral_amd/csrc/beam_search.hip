@@ -290,17 +290,39 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             while (P < nc) P <<= 1;
             for (int i = nc + tid; i < P; i += NT) cand[i] = kKeyMax;
             __syncthreads();
-            for (int k2 = 2; k2 <= P; k2 <<= 1) {
-                for (int j = k2 >> 1; j > 0; j >>= 1) {
-                    for (int t = tid; t < (P >> 1); t += NT) {
-                        const int i = 2 * t - (t & (j - 1));
-                        const int x = i + j;
-                        const bool asc = (i & k2) == 0;
-                        const uint64_t ka = cand[i], kb = cand[x];
-                        if ((ka > kb) == asc) cand[i] = kb, cand[x] = ka;
+            // Bitonic sort of cand[0..P).  Blocks of 128 keys belong to one wave each: every
+            // step whose partner distance stays inside a block needs no workgroup barrier
+            // (LDS operations of one wave complete in order), only the few steps that
+            // cross blocks do.
+            const int B = P < 128 ? P : 128, nblk = P / B;
+            auto exchange = [&](int i, int j, int k2) {
+                const int x = i + j;
+                const bool asc = (i & k2) == 0;
+                const uint64_t ka = cand[i], kb = cand[x];
+                if ((ka > kb) == asc) cand[i] = kb, cand[x] = ka;
+            };
+            auto wave_sync = [&]() {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            };
+            auto block_steps = [&](int k2, int jfrom) {  // steps j = jfrom .. 1 of stage k2, inside blocks
+                for (int blk = wave; blk < nblk; blk += NW) {
+                    for (int j = jfrom; j > 0; j >>= 1) {
+                        if (lane < (B >> 1)) exchange(blk * B + 2 * lane - (lane & (j - 1)), j, k2);
+                        wave_sync();
                     }
+                }
+            };
+            for (int k2 = 2; k2 <= B; k2 <<= 1) block_steps(k2, k2 >> 1);
+            __syncthreads();
+            for (int k2 = 2 * B; k2 <= P; k2 <<= 1) {
+                for (int j = k2 >> 1; j >= B; j >>= 1) {
+                    for (int t = tid; t < (P >> 1); t += NT) exchange(2 * t - (t & (j - 1)), j, k2);
                     __syncthreads();
                 }
+                block_steps(k2, B >> 1);
+                __syncthreads();
             }
             const uint64_t* src = st.cur ? beam1 : beam0;
             uint64_t* dst = st.cur ? beam0 : beam1;

@@ -65,7 +65,7 @@ struct coral_index {
     bool prepared = false;
     int Q = 0, L = 0;
     int slots_log2 = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
-    int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0;
+    int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0, prepared_policy = 0;
     size_t lds_bytes = 0;
     size_t spill_words = 0;
     uint32_t* d_spill = nullptr;
@@ -246,6 +246,9 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     coral_tuning t;
     std::memset(&t, 0, sizeof t);
     if (tuning) t = *tuning;
+    if (t.policy != CORAL_POLICY_ROUNDS && t.policy != CORAL_POLICY_BEST_FIRST)
+        return fail(CORAL_ERR_ARG, "unknown policy %d", t.policy);
+    const bool best_first = t.policy == CORAL_POLICY_BEST_FIRST;
     HIP_TRY(hipSetDevice(idx->device));
     HIP_TRY(hipStreamSynchronize(idx->stream));
 
@@ -260,8 +263,9 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     if (slots_log2 == 0) {
         // a degree-32 graph over a million nodes sees about 75 first visits per beam
         // entry; 112 cells per entry keep the load factor near 0.65
+        // (best-first: about 31 first visits per entry, 48 cells)
         slots_log2 = 12;
-        while ((1 << slots_log2) < 112 * L && slots_log2 < 16) ++slots_log2;
+        while ((1 << slots_log2) < (best_first ? 48 : 112) * L && slots_log2 < 16) ++slots_log2;
         while (slots_log2 > 12 &&
                coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap) + 64 > (size_t)kMaxLdsBytes)
             --slots_log2;
@@ -282,14 +286,14 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     const int wg_fit = (int)((size_t)kMaxLdsBytes / lds_for(min_cap));
     // (capacities are powers of two: the candidate buffer is bitonic-sorted in place)
     for (int cap : {1024, 512}) {
-        if (cap <= tcap) break;
+        if (cap <= tcap || best_first) break;  // best-first expands one row at a time
         if (lds_for(cap) <= (size_t)kMaxLdsBytes && (int)((size_t)kMaxLdsBytes / lds_for(cap)) >= std::min(wg_fit, 2)) {
             tcap = cap;
             break;
         }
     }
     int threads = t.threads;
-    if (threads == 0) threads = lds_for(tcap) > (size_t)kMaxLdsBytes / 2 ? 1024 : 512;
+    if (threads == 0) threads = best_first ? 256 : (lds_for(tcap) > (size_t)kMaxLdsBytes / 2 ? 1024 : 512);
     if (threads != 128 && threads != 256 && threads != 512 && threads != 1024)
         return fail(CORAL_ERR_ARG, "threads must be 128, 256, 512 or 1024");
     const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap);
@@ -321,6 +325,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     idx->Q = Q, idx->L = L, idx->slots_log2 = slots_log2, idx->vis_limit = vis_limit;
     idx->tcap = tcap, idx->ccap = tcap, idx->threads = threads, idx->workgroups = workgroups;
     idx->id_bits = id_bits, idx->rem_bits = rem_bits, idx->dmax = dmax, idx->ocap = ocap;
+    idx->prepared_policy = t.policy;
     idx->lds_bytes = lds, idx->spill_words = spill_words;
     idx->prepared = true;
     return CORAL_OK;
@@ -423,8 +428,11 @@ int coral_search(coral_index* idx, const float* h_queries, int32_t Q, int32_t k,
     if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
     if (k <= 0 || k > L) return fail(CORAL_ERR_ARG, "k=%d must be in 1..L=%d", k, L);
     HIP_TRY(hipSetDevice(idx->device));
-    if (!idx->prepared || idx->L != L || idx->Q < Q) {
-        if (int rc = coral_search_prepare(idx, Q, L, nullptr)) return rc;
+    if (!idx->prepared || idx->L != L || idx->Q < Q || idx->prepared_policy != policy) {
+        coral_tuning t;
+        std::memset(&t, 0, sizeof t);
+        t.policy = policy;
+        if (int rc = coral_search_prepare(idx, Q, L, &t)) return rc;
     }
     float* d_q = nullptr;
     int32_t* d_ids = nullptr;

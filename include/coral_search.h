@@ -92,7 +92,9 @@ typedef struct {
     int32_t visited_slots_log2; /* LDS visited table: log2 of its 16-bit cells, 10..16; 0 = chosen from L */
     int32_t workgroups;         /* persistent workgroups; 0 = chosen from Q and the device */
     int32_t threads;            /* threads per workgroup: 128, 256, 512 or 1024; 0 = chosen from the LDS need */
-    int32_t reserved[5];
+    int32_t policy;             /* the policy the scratch is sized for (CORAL_POLICY_*); best-first visits
+                                   fewer nodes per beam entry and works on one graph row at a time */
+    int32_t reserved[4];
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);

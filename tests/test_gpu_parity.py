@@ -71,7 +71,7 @@ def test_exact_against_same_order_oracle(orc, case):
     q = make_queries(150, dim, 300 + dim, metric)
     print("case", case, flush=True)
     idx = capi.Index(base, nbrs, starts, m)
-    idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads)
+    idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy)
     ids, dists, st = idx.search(q, k, L, policy=policy)
     cnt = idx.query_counters(q.shape[0])
     idx.close()
