@@ -51,6 +51,7 @@ namespace coral {
 #endif
 
 constexpr uint64_t kKeyMax = ~0ull;
+constexpr int kSmallMerge = 32;  // candidate counts merged by counting instead of sorting
 
 // float -> uint32 whose unsigned order is the float order
 __device__ __forceinline__ uint32_t ord32(float s) {
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     uint32_t* olist = elist + Lp;
     float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_first, s_outpos, s_nover;
+    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_cursor, s_outpos, s_nover;
 
     VisitedSet vs;
     vs.words = table, vs.olist = olist, vs.ocount = &s_nover;
@@ -199,7 +200,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
 
         for (int i = tid; i < (slots >> 1); i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
-        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0;
+        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0, s_cursor = 0;
         __syncthreads();
 
         float4 qreg[CPL];
@@ -286,6 +287,35 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             __syncthreads();
             const int nc = s_ncand;
             if (nc == 0) return;
+            if (nc <= kSmallMerge) {
+                // few candidates (every best-first step, the late rounds): no sort; a key's place
+                // is its own index plus the number of smaller keys in the other list, and the
+                // candidates are few enough to be counted by reading them all (broadcast reads)
+                const uint64_t* src = st.cur ? beam1 : beam0;
+                uint64_t* dst = st.cur ? beam0 : beam1;
+                const int nb = st.nb;
+                for (int i = tid; i < nb; i += NT) {
+                    const uint64_t key = src[i];
+                    int below = 0;
+                    for (int c = 0; c < nc; ++c) below += cand[c] < key;
+                    if (i + below < L) dst[i + below] = key;
+                }
+                for (int j = tid; j < nc; j += NT) {
+                    const uint64_t key = cand[j];
+                    int below = 0;
+                    for (int c = 0; c < nc; ++c) below += cand[c] < key;
+                    const int pos = below + lower_bound_u64(src, nb, key);
+                    if (pos < L) dst[pos] = key;
+                    if (below == 0 && pos < s_cursor) s_cursor = pos;
+                }
+                __syncthreads();
+                st.nb = min(L, nb + nc);
+                st.cur ^= 1;
+                st.live = st.nb == L ? dst[L - 1] : kKeyMax;
+                if (tid == 0) s_ncand = 0;
+                __syncthreads();
+                return;
+            }
             int P = 2;
             while (P < nc) P <<= 1;
             for (int i = nc + tid; i < P; i += NT) cand[i] = kKeyMax;
@@ -336,6 +366,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 const uint64_t key = cand[j];
                 const int pos = j + lower_bound_u64(src, nb, key);
                 if (pos < L) dst[pos] = key;
+                if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
             }
             __syncthreads();
             st.nb = min(L, nb + nc);
@@ -365,7 +396,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         for (;;) {
             uint64_t* beam = st.cur ? beam1 : beam0;
             const int nb0 = st.nb;
-            if (tid == 0) s_nexp = 0, s_first = 0x7fffffff;
+            if (tid == 0) s_nexp = 0;
             __syncthreads();
             if (a.policy == 0) {
                 for (int i0 = 0; i0 < nb0; i0 += NT) {
@@ -384,19 +415,30 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                         }
                     }
                 }
-            } else {
-                for (int i0 = 0; i0 < nb0; i0 += NT) {
-                    const int i = i0 + tid;
+            } else if (wave == 0) {
+                // best first: the closest entry not yet expanded.  s_cursor is a lower bound of
+                // its index (kept by the merge); wave 0 scans on from there 64 entries at a time
+                int c = s_cursor, found = nb0;
+                while (c < nb0) {
+                    const int i = c + lane;
                     const bool un = i < nb0 && (beam[i] & 1ull) == 0;
                     const uint64_t m = __ballot(un);
-                    if (m && lane == 0) atomicMin(&s_first, i0 + wave * 64 + (__ffsll((long long)m) - 1));
+                    if (m) {
+                        found = c + (__ffsll((long long)m) - 1);
+                        break;
+                    }
+                    c += 64;
                 }
-                __syncthreads();
-                if (tid == 0 && s_first < nb0) {
-                    const uint64_t key = beam[s_first];
-                    elist[0] = (uint32_t)key_id(key);
-                    beam[s_first] = key | 1ull;
-                    s_nexp = 1;
+                if (lane == 0) {
+                    if (found < nb0) {
+                        const uint64_t key = beam[found];
+                        elist[0] = (uint32_t)key_id(key);
+                        beam[found] = key | 1ull;
+                        s_nexp = 1;
+                        s_cursor = found + 1;
+                    } else {
+                        s_cursor = nb0;
+                    }
                 }
             }
             __syncthreads();

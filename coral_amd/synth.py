@@ -132,3 +132,41 @@ def medoid_start(base):
     mean = base.mean(axis=0, dtype=np.float64)
     d = ((base.astype(np.float64) - mean[None, :]) ** 2).sum(1)
     return int(np.argmin(d))
+
+
+def block_graph(base, R=32, block=4096, long_links=8, seed=7, device="cuda"):
+    """A cheap degree-R graph for very large bases where neither an exact kNN graph
+    nor the query-aware builder is affordable: consecutive ids form blocks; a node
+    links to its R - long_links nearest nodes inside its block and to long_links
+    pseudo-random nodes anywhere (SplitMix64 of (seed, id, j)), which keeps the graph
+    connected.  Rows are sorted block links first.  Test/benchmark data only."""
+    import torch
+    n = base.shape[0]
+    near = R - long_links
+    out = np.empty((n, R), dtype=np.int32)
+    for s in range(0, n, block * 64):
+        e = min(n, s + block * 64)
+        xb = torch.from_numpy(base[s:e]).to(device)
+        for b0 in range(0, e - s, block):
+            x = xb[b0:b0 + block]
+            m = x.shape[0]
+            sq = (x * x).sum(1)
+            d = sq[:, None] + sq[None, :] - 2.0 * (x @ x.T)
+            d.fill_diagonal_(float("inf"))
+            kk = min(near, m - 1)
+            idx = torch.topk(d, kk, dim=1, largest=False, sorted=True).indices + (s + b0)
+            out[s + b0:s + b0 + m, :kk] = idx.to(torch.int32).cpu().numpy()
+            if kk < near:
+                out[s + b0:s + b0 + m, kk:near] = -1
+    ids = np.arange(n, dtype=np.uint64)
+    for j in range(long_links):
+        r = (splitmix64(seed + j, ids) % np.uint64(n)).astype(np.int64)
+        r = np.where(r == np.arange(n), (r + 1) % n, r)
+        out[:, near + j] = r.astype(np.int32)
+    # a row's neighbours are its leading non-negative entries: compact rows that got -1 in the middle
+    if (out[:, :near] < 0).any():
+        for i in np.where((out[:, :near] < 0).any(axis=1))[0]:
+            row = out[i][out[i] >= 0]
+            out[i] = -1
+            out[i, :row.size] = row
+    return out

@@ -1,0 +1,152 @@
+"""The benchmark configurations other than the headline one, as parity cases:
+config 1 (100k x 128, exact 32-NN graph, k=10, L=64: the reference's CPU-runnable case),
+config 3 (inner product, 1M x 512, k=100, L=256), config 4 (10M x 200, batch sweep) and
+config 5 (100M x 200 with 10 % tombstones; skipped where memory is short).
+Graphs of configs 4 and 5 are cheap block graphs (coral_amd.synth.block_graph): these cases
+check parity and size handling, not recall."""
+import os
+import time
+
+import numpy as np
+import pytest
+
+from coral_amd import capi, synth, workloads
+
+pytestmark = pytest.mark.gpu
+WAVE64 = 3
+
+
+def check_basic(ids, dists, n, k, larger_is_closer=False):
+    assert ((ids >= 0) & (ids < n)).all()
+    d = np.diff(dists, axis=1)
+    assert (d <= 0).all() if larger_is_closer else (d >= 0).all()
+    assert all(len(set(r.tolist())) == k for r in ids[:: max(1, len(ids) // 64)])
+
+
+def test_config1_reference_cpu_case(orc):
+    w = workloads.config1()
+    base, q, nbrs, starts, k, L = w["base"], w["queries"], w["nbrs"], w["starts"], 10, 64
+    assert starts.size == 1 and (nbrs >= 0).all()
+    idx = capi.Index(base, nbrs, starts)
+    prob = orc.Problem(base, nbrs, starts)
+    gt, _ = orc.bruteforce(base, q, k)
+    # the rounds policy: exact against the same-order oracle, tolerance against the reference orders
+    ids, dists, st = idx.search(q, k, L)
+    cnt = idx.query_counters(q.shape[0])
+    oi, od, os_, _ = orc.search_B(prob, q, k, L, start_order=WAVE64, nbr_order=WAVE64)
+    assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(cnt, os_)
+    ri, rd, _, _ = orc.search_B(prob, q, k, L)
+    assert (np.abs(dists - rd)[ids == ri] <= 1e-5 * rd[ids == ri]).all()
+    assert (ids == ri).all(1).mean() >= 0.99
+    print("config1 rounds: %.0f QPS, recall@10 %.4f" % (q.shape[0] / st.time_s,
+                                                          orc.recall_hits(ids, gt, k) / gt.size), flush=True)
+    # the reference runs this configuration on its CPU path: best-first, M = 1, AVX-512 order
+    ids, dists, st = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)
+    cnt = idx.query_counters(q.shape[0])
+    oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
+    assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(cnt, os_)
+    ci, cd, cs, _ = orc.search_A(prob, q, k, L)  # the reference's own summation order
+    assert (np.abs(dists - cd)[ids == ci] <= 1e-5 * cd[ids == ci]).all()
+    assert (ids == ci).all(1).mean() >= 0.99
+    r_gpu = orc.recall_hits(ids, gt, k) / gt.size
+    r_cpu = orc.recall_hits(ci, gt, k) / gt.size
+    assert abs(r_gpu - r_cpu) <= 1e-3
+    print("config1 best-first: %.0f QPS, recall@10 %.4f (cpu order %.4f)" % (q.shape[0] / st.time_s, r_gpu, r_cpu),
+          flush=True)
+    idx.close()
+
+
+def test_config3_inner_product_1m_x_512(orc):
+    t0 = time.time()
+    w = workloads.config3()
+    base, q, nbrs, starts, k, L = w["base"], w["queries"], w["nbrs"], w["starts"], 100, 256
+    print("config3 prepared in %.0f s: %s" % (time.time() - t0, w["build"]), flush=True)
+    n = base.shape[0]
+    idx = capi.Index(base, nbrs, starts, capi.IP)
+    ids, dists, st = idx.search(q, k, L)
+    cnt = idx.query_counters(q.shape[0])
+    check_basic(ids, dists, n, k, larger_is_closer=True)
+    for qi in range(0, q.shape[0], 1001):  # returned value = raw inner product of the returned id
+        want = base[ids[qi]].astype(np.float64) @ q[qi].astype(np.float64)
+        assert np.allclose(dists[qi], want, rtol=1e-5, atol=1e-6)
+    sub = np.arange(0, q.shape[0], 211)
+    prob = orc.Problem(base, nbrs, starts)
+    oi, od, os_, _ = orc.search_B(prob, q[sub], k, L, metric=orc.IP, start_order=WAVE64, nbr_order=WAVE64)
+    assert np.array_equal(ids[sub], oi) and dists[sub].tobytes() == od.tobytes() and np.array_equal(cnt[sub], os_)
+    ri, rd, _, _ = orc.search_B(prob, q[sub], k, L, metric=orc.IP)
+    same = ids[sub] == ri
+    assert (np.abs(dists[sub] - rd)[same] <= 1e-5 * np.abs(rd[same])).all()
+    gt = workloads.ground_truth(base, q[sub], k, "ip")
+    r_gpu = orc.recall_hits(ids[sub], gt, k) / gt.size
+    r_ref = orc.recall_hits(ri, gt, k) / gt.size
+    assert abs(r_gpu - r_ref) <= 1e-3
+    B = st.expansions * 128 + st.dist_evals * 2048 + q.shape[0] * (2048 + k * 8)
+    print("config3: %.0f QPS, %.0f GB/s algorithmic, recall@100 %.4f, %.0f distance evaluations/query" %
+          (q.shape[0] / st.kernel_s, B / st.kernel_s / 1e9, r_gpu, st.dist_evals / q.shape[0]), flush=True)
+    idx.close()
+
+
+def big_case(orc, n, dim, Qs, L, k, tomb_seed=None):
+    t0 = time.time()
+    base = workloads.gaussian_base(4001 if n <= 10 ** 7 else 5001, n, dim)
+    print("generated %d x %d in %.0f s" % (n, dim, time.time() - t0), flush=True)
+    nbrs = synth.block_graph(base, 32)
+    print("block graph at %.0f s" % (time.time() - t0), flush=True)
+    starts = (np.arange(16, dtype=np.int64) * (n // 16) + 5).astype(np.int32)
+    q = synth.shifted_queries(max(Qs), dim, 2002, 2003, 2004)
+    idx = capi.Index(base, nbrs, starts)
+    mask = None
+    if tomb_seed is not None:
+        mask = synth.tombstone_mask(n, tomb_seed, 10)
+        idx.set_deleted(mask)
+    print("index resident at %.0f s" % (time.time() - t0), flush=True)
+    results = {}
+    for Q in Qs:
+        ids, dists, st = idx.search(q[:Q], k, L, have_delete=mask is not None)
+        results[Q] = (ids, dists, idx.query_counters(Q))
+        check_basic(ids, dists, n, k)
+        B = st.expansions * 128 + st.dist_evals * dim * 4 + Q * (dim * 4 + k * 8)
+        print("n=%d Q=%d: %.0f QPS, %.0f GB/s algorithmic, %d spills" %
+              (n, Q, Q / st.kernel_s, B / st.kernel_s / 1e9, st.spills), flush=True)
+    # a query's answer does not depend on the batch it travels in
+    small = min(Qs)
+    for Q in Qs:
+        assert np.array_equal(results[Q][0][:small], results[small][0])
+        assert results[Q][1][:small].tobytes() == results[small][1].tobytes()
+    ids, dists, cnt = results[small]
+    sub = np.arange(0, small, max(1, small // 48))
+    prob = orc.Problem(base, nbrs, starts, mask)
+    oi, od, os_, _ = orc.search_B(prob, q[sub], k, L, start_order=WAVE64, nbr_order=WAVE64)
+    assert np.array_equal(ids[sub], oi) and dists[sub].tobytes() == od.tobytes() and np.array_equal(cnt[sub], os_)
+    if mask is not None:
+        dead = (mask[ids >> 5] >> (ids & 31).astype(np.uint32)) & 1
+        assert not dead.any()
+    idx.close()
+
+
+def test_config4_10m_batch_sweep(orc):
+    big_case(orc, 10 ** 7, 200, (1000, 10000, 100000), 256, 100)
+
+
+def _mem_available_gib():
+    try:
+        for line in open("/proc/meminfo"):
+            if line.startswith("MemAvailable:"):
+                return int(line.split()[1]) / (1 << 20)
+    except OSError:
+        pass
+    return 0.0
+
+
+def test_config5_100m_tombstones(orc):
+    """80 GB of vectors + 12.8 GB of graph rows resident in HBM, 10 % of the ids tombstoned.
+    About a minute on an MI355X box; skipped where host or device memory cannot hold it."""
+    import torch
+    if os.environ.get("CORAL_SKIP_100M") == "1":
+        pytest.skip("CORAL_SKIP_100M=1")
+    if _mem_available_gib() < 130:
+        pytest.skip("needs about 100 GB of host memory")
+    free, _ = torch.cuda.mem_get_info()
+    if free < 120 * (1 << 30):
+        pytest.skip("needs about 105 GB of device memory")
+    big_case(orc, 10 ** 8, 200, (1000, 100000), 256, 100, tomb_seed=5002)
