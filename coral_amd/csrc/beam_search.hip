@@ -20,7 +20,7 @@
 // Distance summation order (mirrored bit for bit by the test oracle): lane l of a
 // group of G lanes accumulates float4 chunks l, l+G, ... with four fused
 // multiply-adds per chunk in x,y,z,w order; partials are combined by a butterfly
-// p[l] += p[l^off], off = G/2..1.
+// p[l] += p[l^off], off = 1, 2, 4, ..., G/2.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -132,6 +132,12 @@ struct VisitedSet {
         return 1;
     }
 };
+
+// the value of x in the lane a DPP control selects (all rows and banks enabled)
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
 
 // number of set bits of m below the calling lane
 __device__ __forceinline__ int prefix_popc(uint64_t m) {
@@ -255,16 +261,25 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     }
                     acc[u] = s;
                 }
+                // Cross-lane butterfly p[l] += p[l ^ off], off = 1, 2, 4, ..., G/2.  Inside a row of
+                // 16 lanes it runs on DPP (register speed): after off = 1, 2 a quad holds one value,
+                // so l ^ 7 (row_half_mirror) stands for l ^ 4 and l ^ 15 (row_mirror) for l ^ 8 with
+                // bit-identical results.  Across rows each lane only needs the row it will file, so it
+                // first picks that row's partial and the last one or two levels cost one exchange each.
 #pragma unroll
-                for (int off = G / 2; off > 0; off >>= 1) {
-#pragma unroll
-                    for (int u = 0; u < U; ++u) acc[u] = acc[u] + __shfl_xor(acc[u], off, 64);
+                for (int u = 0; u < U; ++u) {
+                    acc[u] = acc[u] + dpp_mov<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
+                    acc[u] = acc[u] + dpp_mov<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
+                    acc[u] = acc[u] + dpp_mov<0x141>(acc[u]);  // row_half_mirror
+                    acc[u] = acc[u] + dpp_mov<0x140>(acc[u]);  // row_mirror
                 }
                 float mine = acc[0];
                 int myid = vid[0];
 #pragma unroll
                 for (int u = 1; u < U; ++u)
-                    if (gl == u) mine = acc[u], myid = vid[u];
+                    if ((lane & (U - 1)) == u) mine = acc[u], myid = vid[u];
+                if (G >= 32) mine = mine + __shfl_xor(mine, 16, 64);
+                if (G >= 64) mine = mine + __shfl_xor(mine, 32, 64);
                 const bool valid = gl < U && myid >= 0;
                 const float s = a.metric == 0 ? mine : 0.0f - mine;
                 const bool pf = valid && (s < thr);

@@ -202,7 +202,7 @@ static int have_avx512(void) {
  * (G = 16, 32 or 64, the smallest that covers dim/4 chunks, capped at 64) owns
  * the row; lane l accumulates chunks l, l+G, ... with four fused multiply-adds
  * per chunk in x,y,z,w order; the G partials are then combined by a butterfly,
- * p[l] += p[l ^ off] for off = G/2 .. 1. */
+ * p[l] += p[l ^ off] for off = 1, 2, 4, .. G/2 (every lane ends with the same value). */
 static int wave64_group(int dim) {
     int chunks = dim / 4;
     if (chunks <= 16) return 16;
@@ -227,8 +227,11 @@ static float dist_wave64(const float* q, const float* b, int dim, int metric) {
         }
         p[l] = acc;
     }
-    for (int off = G / 2; off > 0; off >>= 1)
-        for (int l = 0; l < off; ++l) p[l] = p[l] + p[l + off];
+    for (int off = 1; off < G; off <<= 1) {
+        float t[64];
+        for (int l = 0; l < G; ++l) t[l] = p[l] + p[l ^ off];
+        for (int l = 0; l < G; ++l) p[l] = t[l];
+    }
     return p[0];
 }
 
