@@ -226,14 +226,19 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         auto distance_phase = [&](int T) {
             int cntf = 0;
             for (int base = wave * RPI; base < T; base += NW * RPI) {
+                // all ids of this iteration first (one LDS wait), then all row requests back to back
                 int vid[U];
+                const int r0 = base + grp * U;
+#pragma unroll
+                for (int u = 0; u < U; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (r0 + u >= T) vid[u] = -1;
                 float4 v[U][CPL];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const int r = base + grp * U + u;
-                    vid[u] = r < T ? (int)todo[r] : -1;
-                    const float4* row =
-                        reinterpret_cast<const float4*>(a.vec + (size_t)(vid[u] < 0 ? 0 : vid[u]) * dim);
+                    const float4* row = reinterpret_cast<const float4*>(
+                        a.vec + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * (uint32_t)dim);
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) {
                         const int c = gl + G * t;
@@ -462,9 +467,9 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             if (nexp == 0) break;
 
             // The round's rows are taken in chunks of `ech` beam entries (what the todo
-            // list holds).  Requesting the next chunk's neighbour ids ahead of time was
-            // measured and lost to this plain form: with two workgroups per CU the other
-            // workgroup already covers the wait for the graph rows.
+            // list holds).  Requesting graph rows ahead of time (the next chunk's, or for
+            // best-first the likely next entry's) was measured twice and lost to this plain
+            // form: the other workgroup on the CU already covers that wait.
             const int ech = TCAP / R;
             ne += nexp;
             for (int e0 = 0; e0 < nexp; e0 += ech) {
