@@ -561,7 +561,12 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             __syncthreads();
             for (int i = s_outpos + tid; i < a.k; i += NT) {
                 ids_out[i] = -1;
-                if (dists_out) dists_out[i] = a.metric == 0 ? 3.402823466e+38f : -3.402823466e+38f;
+                // unfilled slots: the farthest sentinel (rounds: +-FLT_MAX as the CUDA kernel pads its
+                // beam, src/search_gpu.cu:408; best-first: +-infinity, src/search_in_cpu.cpp:33-35)
+                if (dists_out) {
+                    const float far = a.policy == 1 ? __int_as_float(0x7f800000) : 3.402823466e+38f;
+                    dists_out[i] = a.metric == 0 ? far : -far;
+                }
             }
             if (tid == 0) {
                 int32_t* c = a.counters + (size_t)qid * 4;

@@ -10,7 +10,9 @@
 // does not register; it is accepted and ignored.
 // Extensions: --policy {rounds,best_first}, --index_dir <dir> (overrides the
 // derived ../indexes/<dataset>_<dist>_<R>_<thres>_<CE> path), --index_prefix
-// and --evaluation_prefix (default ../indexes/ and ../evaluation/).
+// and --evaluation_prefix (default ../indexes/ and ../evaluation/),
+// --device_recall 1 (recall through IndexGPU::Search_and_Verify, the loop of
+// the reference's tests/test_update.cpp:196-197, instead of the host count).
 #include <sys/stat.h>
 
 #include <algorithm>
@@ -63,6 +65,7 @@ const Option kOptions[] = {
     {"index_dir", false, false, "", "index directory (overrides the derived name)"},
     {"index_prefix", false, false, "../indexes/", "directory holding index directories"},
     {"evaluation_prefix", false, false, "../evaluation/", "directory receiving the CSV"},
+    {"device_recall", false, false, "0", "1: count hits on the device (IndexGPU::Search_and_Verify)"},
 };
 
 void usage() {
@@ -238,6 +241,7 @@ int main(int argc, char** argv) {
             index.LoadRoarGraph(std::string("../data/") + dataset + "/indexes/para-t2i-test-5");
         else if (index_type == "cdmg")
             index.LoadRoarGraph(std::string("../data/") + dataset + "/indexes/cdmg.index");
+        const bool device_recall = str("device_recall") == "1";
         const std::string policy = str("policy");
         if (policy == "best_first")
             index.SetPolicy(CORAL_POLICY_BEST_FIRST);
@@ -264,10 +268,21 @@ int main(int argc, char** argv) {
                 std::cout << "L must greater or equal than k" << std::endl;
                 return 1;
             }
-            Test_Result tr = index_type.empty() ? index.Search(query_data.data(), (int)q_pts, L, res.data())
-                                                : index.Search(query_data.data(), (int)q_pts, L, res.data(), 1);
+            float recall;
+            Test_Result tr;
+            if (device_recall) {
+                // the device count assumes gt rows k apart (src/index_gpu.cpp:96-98)
+                std::vector<int> gt_k((size_t)q_pts * k);
+                for (int64_t qi = 0; qi < q_pts; ++qi)
+                    std::copy_n(gt_ids.data() + (size_t)qi * gt_dim, k, gt_k.data() + (size_t)qi * k);
+                tr = index.Search_and_Verify(query_data.data(), gt_k.data(), (int)q_pts, L);
+                recall = tr.calc_recall((int)q_pts * k) / 100.0f;
+            } else {
+                tr = index_type.empty() ? index.Search(query_data.data(), (int)q_pts, L, res.data())
+                                        : index.Search(query_data.data(), (int)q_pts, L, res.data(), 1);
+                recall = ComputeRecall((int)q_pts, k, gt_dim, res.data(), gt_ids.data());
+            }
             const float time = tr.get_time(), qps = (float)q_pts / time;
-            const float recall = ComputeRecall((int)q_pts, k, gt_dim, res.data(), gt_ids.data());
             const float avg_hops = tr.avg_hops((int)q_pts);
             std::cout << L << "\t\t" << qps << "\t\t" << time << "\t\t" << recall << "\t\t" << avg_hops << std::endl;
             evaluation_out << L << "," << qps << "," << time << "," << recall << "," << avg_hops << std::endl;

@@ -19,7 +19,9 @@
  *     leading non-negative entries (the deg and nbrs[0..deg) fields of the
  *     reference's 400-byte Slot, include/disk_graph.h:30-52, and nothing else).
  *   - results are ordered closest first; unfilled slots hold id -1 and the
- *     farthest sentinel (FLT_MAX for L2, -FLT_MAX for IP).
+ *     farthest value of the policy's reference path: +-FLT_MAX (L2 / IP) for
+ *     CORAL_POLICY_ROUNDS (src/search_gpu.cu:408), +-infinity for
+ *     CORAL_POLICY_BEST_FIRST (src/search_in_cpu.cpp:33-35).
  *   - not thread-safe per index, like the reference (src/search.cu:404-408).
  */
 #ifndef CORAL_SEARCH_H

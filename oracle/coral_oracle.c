@@ -385,7 +385,7 @@ ORACLE_API int oracle_search_A(const oracle_index* idx, const float* queries, in
     const int dmetric = (order == ORDER_CPU_AVX512) ? ORACLE_L2 : metric;
     for (size_t i = 0; i < (size_t)Q * k; ++i) ids[i] = -1;
     if (dists)
-        for (size_t i = 0; i < (size_t)Q * k; ++i) dists[i] = INFINITY;
+        for (size_t i = 0; i < (size_t)Q * k; ++i) dists[i] = dmetric == ORACLE_IP ? -INFINITY : INFINITY;
 #ifdef _OPENMP
     int nt = nthreads > 0 ? nthreads : omp_get_max_threads();
 #else

@@ -155,7 +155,7 @@ def test_short_components_pad_with_minus_one(orc):
     for policy in (0, 1):
         ids, dists, _ = idx.search(q, 10, 16, policy=policy)
         assert (ids[:, 6:] == -1).all() and (np.sort(ids[:, :6], axis=1) == np.arange(6)).all()
-        assert (dists[:, 6:] == np.float32(3.402823466e38)).all()
+        assert (dists[:, 6:] == (np.float32(3.402823466e38) if policy == 0 else np.float32(np.inf))).all()
         prob = orc.Problem(base, nbrs, np.array([1], np.int32))
         oi = (orc.search_B(prob, q, 10, 16, start_order=WAVE64, nbr_order=WAVE64) if policy == 0
               else orc.search_A(prob, q, 10, 16, order=WAVE64))[0]
@@ -255,7 +255,27 @@ def test_cli_end_to_end(orc, tmp_path):
     r = subprocess.run(args[:-7] + ["--L", "8", "--config_file", str(work / "config.json")], cwd=work / "cwd",
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 1 and "L must greater or equal than k" in r.stdout
-    # best-first policy and the RoarGraph loader share the driver
+    # recall counted on the device by IndexGPU::Search_and_Verify gives the same table
+    r = subprocess.run(args + ["--device_recall", "1"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    for L in (32, 64):
+        a = [l for l in lines if l.startswith("%d\t" % L)][0].split()
+        b = [l for l in r.stdout.splitlines() if l.startswith("%d\t" % L)][0].split()
+        assert abs(float(a[3]) - float(b[3])) < 1e-6 and a[4] == b[4]
+    # --index_type roar replaces the graph by a RoarGraph file and searches from its entry point
+    # (tests/test_search_pipeline.cpp:247-252: ../data/<dataset>/indexes/roar.index)
+    os.makedirs(work / "data" / "syn" / "indexes")
+    roar = ragged(synth.exact_knn_graph(base, 32, device="cuda"), 9, keep_min=4)
+    formats.roargraph_write(work / "data" / "syn" / "indexes" / "roar.index", roar, 123)
+    r = subprocess.run(args + ["--index_type", "roar"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert (work / "evaluation" / "search" / "roar_syn_l2_32.csv").exists()
+    rprob = orc.Problem(base, roar, np.array([123], np.int32))
+    oi, _, os_, _ = orc.search_B(rprob, q, k, 64, start_order=WAVE64, nbr_order=WAVE64)
+    row = [l for l in r.stdout.splitlines() if l.startswith("64\t")][0].split()
+    assert abs(float(row[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
+    assert abs(float(row[4]) - os_[:, 0].sum() / Q) < 1e-2
+    # best-first policy through the same driver
     r = subprocess.run(args + ["--policy", "best_first"], cwd=work / "cwd", capture_output=True, text=True,
                        timeout=120)
     assert r.returncode == 0
@@ -263,3 +283,44 @@ def test_cli_end_to_end(orc, tmp_path):
     row = [l for l in r.stdout.splitlines() if l.startswith("32\t")][0].split()
     assert abs(float(row[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
     assert abs(float(row[4]) - os_[:, 0].sum() / Q) < 1e-2
+
+
+def test_randomised_shapes(orc):
+    """Forty seeded random combinations of n, dim, R, L, k, M, metric, policy, workgroup size and
+    visited-table size on random ragged graphs (uniform random neighbours, some empty rows):
+    everything integer-exact against the same-order oracle."""
+    rng = np.random.RandomState(2024)
+    for trial in range(40):
+        dim = int(rng.choice([4, 8, 20, 64, 68, 128, 132, 200, 256, 260, 512, 516, 1024]))
+        n = int(rng.randint(50, 6000))
+        R = int(rng.choice([1, 2, 5, 8, 16, 31, 32]))
+        L = int(rng.randint(1, 200))
+        k = int(rng.randint(1, L + 1))
+        M = int(rng.randint(1, min(L, n, 40) + 1))
+        metric = int(rng.randint(0, 2))
+        policy = int(rng.randint(0, 2))
+        threads = int(rng.choice([0, 128, 256, 512, 1024]))
+        slots = int(rng.choice([0, 0, 10, 11, 13]))
+        base = synth.gaussian_matrix(9000 + trial, n, dim)
+        if metric == 1:
+            base = synth.normalize_rows(base)
+        nbrs = ragged(rng.randint(0, n, (n, R)).astype(np.int32), trial)
+        nbrs[rng.randint(0, n, max(1, n // 50))] = -1
+        starts = rng.choice(n, M, replace=False).astype(np.int32)
+        q = make_queries(int(rng.randint(1, 40)), dim, 7000 + trial, "ip" if metric else "l2")
+        case = dict(trial=trial, n=n, dim=dim, R=R, L=L, k=k, M=M, metric=metric, policy=policy, threads=threads,
+                    slots=slots, Q=q.shape[0])
+        print("random case", case, flush=True)
+        idx = capi.Index(base, nbrs, starts, metric)
+        idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy)
+        ids, dists, st = idx.search(q, k, L, policy=policy)
+        cnt = idx.query_counters(q.shape[0])
+        idx.close()
+        prob = orc.Problem(base, nbrs, starts)
+        if policy == 0:
+            oi, od, os_, _ = orc.search_B(prob, q, k, L, metric=metric, start_order=WAVE64, nbr_order=WAVE64)
+        else:
+            oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=metric, order=WAVE64)
+        assert np.array_equal(ids, oi), case
+        assert dists.tobytes() == od.tobytes(), case
+        assert np.array_equal(cnt, os_), case
