@@ -62,6 +62,10 @@ SIGNATURES = {
                                C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(Stats)]),
     "coral_search_verify": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                       C.POINTER(C.c_int64)]),
+    "coral_bruteforce_knn_gpu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
+                                           C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]),
+    "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
+                                       C.c_void_p, C.POINTER(C.c_double)]),
 }
 
 
@@ -156,6 +160,23 @@ class Index:
         out = np.empty((Q, 4), dtype=np.int32)
         _check(lib().coral_search_query_counters(self._h, _ptr(out), Q))
         return out
+
+    def bruteforce(self, queries, k, have_delete=False, want_dists=True):
+        """Exact kNN of host queries among the index's vectors: (ids, dists, seconds)."""
+        q = np.ascontiguousarray(queries, dtype=np.float32)
+        Q = q.shape[0]
+        ids = np.empty((Q, k), dtype=np.int32)
+        dists = np.empty((Q, k), dtype=np.float32) if want_dists else None
+        t = C.c_double()
+        _check(lib().coral_bruteforce_knn(self._h, _ptr(q), Q, k, int(have_delete), _ptr(ids), _ptr(dists),
+                                          C.byref(t)))
+        return ids, dists, t.value
+
+    def bruteforce_device(self, d_queries, d_ids, d_dists, Q, k, have_delete=False, stream=None):
+        t = C.c_double()
+        _check(lib().coral_bruteforce_knn_gpu(self._h, d_queries, Q, k, int(have_delete), d_ids, d_dists, stream,
+                                              C.byref(t)))
+        return t.value
 
     def verify(self, d_ids_res, d_ids_gt, Q, k):
         hits = C.c_int64()

@@ -1,0 +1,296 @@
+// bruteforce.hip -- exact k-nearest-neighbour search by brute force on gfx950.
+//
+// Stands where the reference uses faiss: the ground-truth tool (tests/comp_gt.cpp:119-176,
+// GpuIndexFlatL2/IP) and the builder's exact k_b-NN of auxiliary queries
+// (src/knn.cu:174-193).  Output order and file layout are the gt file's
+// (uint32 nq, uint32 k, int32 ids[nq*k], include/efanna2e/util.h:81-103).
+//
+// Three kernels:
+//   distance_tile_kernel  a 128 x 128 tile of (query, base) pairs per workgroup, 8 x 8 pairs per
+//                         thread, operands staged through LDS.  Every pair is accumulated by ONE
+//                         thread walking the dimensions in order with one fused multiply-add per
+//                         dimension -- the arithmetic of the reference's l2_distance / ip_distance
+//                         (include/utils.cuh:254-275, 307-323) -- so the distances, and hence the
+//                         ids, are reproducible bit for bit on a CPU.
+//   row_select_kernel     per query row: exact k-th smallest by an 8-bit radix select over the
+//                         order-preserving bit pattern, then ordered compaction (ties by id) and
+//                         a bitonic sort of the k winners.
+//   merge_segments_kernel per query: the k best of the per-segment winners (large bases are
+//                         processed in segments so the distance buffer stays bounded).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "bruteforce.h"
+
+namespace coral {
+
+namespace {
+
+__device__ __forceinline__ uint32_t bf_ord32(float s) {
+    const uint32_t u = __float_as_uint(s);
+    return u ^ ((uint32_t)((int32_t)u >> 31) | 0x80000000u);
+}
+__device__ __forceinline__ float bf_unord32(uint32_t o) {
+    const uint32_t u = (o & 0x80000000u) ? (o ^ 0x80000000u) : ~o;
+    return __uint_as_float(u);
+}
+
+constexpr int TQ = 128, TB = 128, KC = 8;  // tile of queries x base points, dimensions per LDS stage
+
+}  // namespace
+
+// D[q][b] = signed distance (smaller is closer): sum (q-b)^2 for L2, 0 - sum q*b for IP;
+// +inf for tombstoned base ids.  grid = (ceil(nb/TB), ceil(nq/TQ)), 256 threads.
+__global__ __launch_bounds__(256) void distance_tile_kernel(const float* __restrict__ queries,
+                                                           const float* __restrict__ base, int nq,
+                                                           int64_t nb, int dim, int metric,
+                                                           const uint32_t* __restrict__ deleted,
+                                                           int64_t base_id0, float* __restrict__ D,
+                                                           int64_t ldD) {
+    __shared__ float sq[KC][TQ + 4];
+    __shared__ float sb[KC][TB + 4];
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;  // thread (ty, tx) owns queries ty*8.. and base tx*8..
+    const int64_t b0 = (int64_t)blockIdx.x * TB;
+    const int q0 = blockIdx.y * TQ;
+    float acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
+
+    // staging: 128 rows x 8 dims per operand = 256 float4; thread t loads row t/2, dims (t&1)*4..
+    const int lrow = tid >> 1, lk = (tid & 1) * 4;
+    for (int k0 = 0; k0 < dim; k0 += KC) {
+        float4 vq = make_float4(0, 0, 0, 0), vb = make_float4(0, 0, 0, 0);
+        if (k0 + lk < dim) {
+            if (q0 + lrow < nq)
+                vq = *reinterpret_cast<const float4*>(queries + (size_t)(q0 + lrow) * dim + k0 + lk);
+            if (b0 + lrow < nb)
+                vb = *reinterpret_cast<const float4*>(base + (size_t)(b0 + lrow) * dim + k0 + lk);
+        }
+        __syncthreads();
+        sq[lk + 0][lrow] = vq.x, sq[lk + 1][lrow] = vq.y, sq[lk + 2][lrow] = vq.z, sq[lk + 3][lrow] = vq.w;
+        sb[lk + 0][lrow] = vb.x, sb[lk + 1][lrow] = vb.y, sb[lk + 2][lrow] = vb.z, sb[lk + 3][lrow] = vb.w;
+        __syncthreads();
+        const int kend = min(KC, dim - k0);
+        for (int kk = 0; kk < kend; ++kk) {
+            float a[8], b[8];
+            const float4 a0 = *reinterpret_cast<const float4*>(&sq[kk][ty * 8]);
+            const float4 a1 = *reinterpret_cast<const float4*>(&sq[kk][ty * 8 + 4]);
+            const float4 c0 = *reinterpret_cast<const float4*>(&sb[kk][tx * 8]);
+            const float4 c1 = *reinterpret_cast<const float4*>(&sb[kk][tx * 8 + 4]);
+            a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
+            b[0] = c0.x, b[1] = c0.y, b[2] = c0.z, b[3] = c0.w, b[4] = c1.x, b[5] = c1.y, b[6] = c1.z, b[7] = c1.w;
+            if (metric == 0) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float t = a[i] - b[j];
+                        acc[i][j] = __fmaf_rn(t, t, acc[i][j]);
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
+            }
+        }
+    }
+    const float inf = __int_as_float(0x7f800000);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int q = q0 + ty * 8 + i;
+        if (q >= nq) continue;
+        float out[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t b = b0 + tx * 8 + j;
+            float s = metric == 0 ? acc[i][j] : 0.0f - acc[i][j];
+            if (b < nb && deleted) {
+                const int64_t id = base_id0 + b;
+                if ((deleted[id >> 5] >> (id & 31)) & 1u) s = inf;
+            }
+            out[j] = s;
+        }
+        float* dst = D + (size_t)(q - q0 + (int64_t)blockIdx.y * TQ) * ldD + b0 + tx * 8;
+        if (b0 + tx * 8 + 7 < nb && (((uintptr_t)dst) & 15) == 0) {
+            *reinterpret_cast<float4*>(dst) = make_float4(out[0], out[1], out[2], out[3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(out[4], out[5], out[6], out[7]);
+        } else {
+            for (int j = 0; j < 8; ++j)
+                if (b0 + tx * 8 + j < nb) dst[j] = out[j];
+        }
+    }
+}
+
+// One workgroup per row of n floats: the k smallest under (value, index), sorted, as
+// keys ord32(value) << 32 | (id0 + index).  Fewer than k finite entries: padded with ~0.
+// Entries equal to +inf (tombstones) never win over finite ones and are dropped at the end.
+__global__ __launch_bounds__(256) void row_select_kernel(const float* __restrict__ D, int64_t ldD,
+                                                         int64_t n, int k, int64_t id0,
+                                                         unsigned long long* __restrict__ out,
+                                                         int64_t out_stride) {
+    extern __shared__ unsigned long long skeys[];  // pow2 >= k keys
+    __shared__ unsigned int hist[256];
+    __shared__ unsigned int s_prefix, s_need, s_count, s_base;
+    const int tid = threadIdx.x;
+    const float* row = D + (size_t)blockIdx.x * ldD;
+    const int kk = (int)min((int64_t)k, n);
+
+    // radix select: after the loop s_prefix is the bit pattern of the kk-th smallest value and
+    // s_need how many entries equal to it belong to the answer
+    if (tid == 0) s_prefix = 0u, s_need = (unsigned)kk;
+    __syncthreads();
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        hist[tid] = 0u;
+        __syncthreads();
+        const uint32_t prefix = s_prefix;
+        const uint32_t himask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+        for (int64_t i = tid; i < n; i += 256) {
+            const uint32_t o = bf_ord32(row[i]);
+            if ((o & himask) == prefix) atomicAdd(&hist[(o >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            unsigned need = s_need, run = 0;
+            int d = 0;
+            for (; d < 256; ++d) {
+                if (run + hist[d] >= need) break;
+                run += hist[d];
+            }
+            s_prefix = prefix | ((uint32_t)d << shift);
+            s_need = need - run;
+        }
+        __syncthreads();
+    }
+    const uint32_t vk = s_prefix;
+    const unsigned need_eq = s_need;  // entries == vk to take, lowest indices first
+    // ordered compaction: everything below vk, and the first need_eq entries equal to vk
+    if (tid == 0) s_count = 0u, s_base = 0u;
+    __syncthreads();
+    const int lane = tid & 63, wave = tid >> 6;
+    __shared__ unsigned int w_eq[4];
+    for (int64_t i0 = 0; i0 < n; i0 += 256) {
+        const int64_t i = i0 + tid;
+        uint32_t o = 0xffffffffu;
+        bool lt = false, eq = false;
+        if (i < n) {
+            o = bf_ord32(row[i]);
+            lt = o < vk, eq = o == vk;
+        }
+        const unsigned long long meq = __ballot(eq);
+        if (lane == 0) w_eq[wave] = (unsigned)__popcll(meq);
+        __syncthreads();
+        unsigned eq_before = 0, eq_total = 0;
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) eq_before += w_eq[w];
+            eq_total += w_eq[w];
+        }
+        const unsigned long long below = (1ull << lane) - 1ull;
+        const unsigned eq_rank = s_base + eq_before + (unsigned)__popcll(meq & below);  // among equals, by index
+        const bool take = lt || (eq && eq_rank < need_eq);
+        // position: entries taken so far + taken before me in this tile
+        const unsigned long long mtake = __ballot(take);
+        __shared__ unsigned int w_take[4];
+        if (lane == 0) w_take[wave] = (unsigned)__popcll(mtake);
+        __syncthreads();
+        unsigned take_before = 0, take_total = 0;
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) take_before += w_take[w];
+            take_total += w_take[w];
+        }
+        if (take) {
+            const unsigned pos = s_count + take_before + (unsigned)__popcll(mtake & below);
+            skeys[pos] = ((unsigned long long)o << 32) | (unsigned long long)(uint32_t)(id0 + i);
+        }
+        __syncthreads();
+        if (tid == 0) s_count += take_total, s_base += eq_total;
+        __syncthreads();
+    }
+    // sort the kk winners
+    int P = 2;
+    while (P < kk) P <<= 1;
+    for (int i = kk + tid; i < P; i += 256) skeys[i] = ~0ull;
+    __syncthreads();
+    for (int k2 = 2; k2 <= P; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1) {
+            for (int t = tid; t < (P >> 1); t += 256) {
+                const int i = 2 * t - (t & (j - 1)), x = i + j;
+                const bool asc = (i & k2) == 0;
+                const unsigned long long ka = skeys[i], kb = skeys[x];
+                if ((ka > kb) == asc) skeys[i] = kb, skeys[x] = ka;
+            }
+            __syncthreads();
+        }
+    unsigned long long* dst = out + (size_t)blockIdx.x * out_stride;
+    for (int i = tid; i < k; i += 256) {
+        unsigned long long key = i < kk ? skeys[i] : ~0ull;
+        if ((uint32_t)(key >> 32) == bf_ord32(__int_as_float(0x7f800000))) key = ~0ull;  // tombstoned
+        dst[i] = key;
+    }
+}
+
+// per query: the k smallest of nseg*k sorted-per-segment keys -> ids and values
+__global__ __launch_bounds__(256) void merge_segments_kernel(const unsigned long long* __restrict__ part,
+                                                             int nseg, int k, int metric,
+                                                             int32_t* __restrict__ ids,
+                                                             float* __restrict__ dists) {
+    extern __shared__ unsigned long long skeys[];
+    const int tid = threadIdx.x, total = nseg * k;
+    const unsigned long long* src = part + (size_t)blockIdx.x * total;
+    int P = 2;
+    while (P < total) P <<= 1;
+    for (int i = tid; i < P; i += 256) skeys[i] = i < total ? src[i] : ~0ull;
+    __syncthreads();
+    for (int k2 = 2; k2 <= P; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1) {
+            for (int t = tid; t < (P >> 1); t += 256) {
+                const int i = 2 * t - (t & (j - 1)), x = i + j;
+                const bool asc = (i & k2) == 0;
+                const unsigned long long ka = skeys[i], kb = skeys[x];
+                if ((ka > kb) == asc) skeys[i] = kb, skeys[x] = ka;
+            }
+            __syncthreads();
+        }
+    for (int i = tid; i < k; i += 256) {
+        const unsigned long long key = skeys[i];
+        const bool none = key == ~0ull;
+        ids[(size_t)blockIdx.x * k + i] = none ? -1 : (int32_t)(uint32_t)key;
+        if (dists) {
+            const float s = bf_unord32((uint32_t)(key >> 32));
+            const float far = 3.402823466e+38f;
+            dists[(size_t)blockIdx.x * k + i] = none ? (metric == 0 ? far : -far) : (metric == 0 ? s : 0.0f - s);
+        }
+    }
+}
+
+hipError_t launch_distance_tile(const float* queries, const float* base, int nq, int64_t nb, int dim,
+                                int metric, const uint32_t* deleted, int64_t base_id0, float* D,
+                                int64_t ldD, hipStream_t stream) {
+    dim3 grid((unsigned)((nb + TB - 1) / TB), (unsigned)((nq + TQ - 1) / TQ));
+    hipLaunchKernelGGL(distance_tile_kernel, grid, dim3(256), 0, stream, queries, base, nq, nb, dim, metric,
+                       deleted, base_id0, D, ldD);
+    return hipGetLastError();
+}
+
+hipError_t launch_row_select(const float* D, int64_t ldD, int nq, int64_t n, int k, int64_t id0,
+                             unsigned long long* out, int64_t out_stride, hipStream_t stream) {
+    int P = 2;
+    while (P < k) P <<= 1;
+    hipLaunchKernelGGL(row_select_kernel, dim3(nq), dim3(256), (size_t)P * 8, stream, D, ldD, n, k, id0, out,
+                       out_stride);
+    return hipGetLastError();
+}
+
+hipError_t launch_merge_segments(const unsigned long long* part, int nq, int nseg, int k, int metric,
+                                 int32_t* ids, float* dists, hipStream_t stream) {
+    int P = 2;
+    while (P < nseg * k) P <<= 1;
+    hipLaunchKernelGGL(merge_segments_kernel, dim3(nq), dim3(256), (size_t)P * 8, stream, part, nseg, k, metric,
+                       ids, dists);
+    return hipGetLastError();
+}
+
+}  // namespace coral

@@ -16,6 +16,7 @@
 
 #include "beam_search.h"
 #include "error.h"
+#include "index_internal.h"
 
 namespace {
 thread_local std::string g_err;
@@ -36,48 +37,10 @@ int fail(int code, const char* fmt, ...) {
 namespace {
 using coral::fail;
 
-#define HIP_TRY(expr)                                                                       \
-    do {                                                                                    \
-        hipError_t e_ = (expr);                                                             \
-        if (e_ != hipSuccess)                                                               \
-            return fail(e_ == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE,    \
-                        "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__,    \
-                        __LINE__);                                                          \
-    } while (0)
-
 constexpr int kMaxL = 2048;
 constexpr int kMaxLdsBytes = 160 * 1024;
 
 }  // namespace
-
-struct coral_index {
-    int device = 0;
-    int64_t n = 0;
-    int dim = 0, R = 0, M = 0, metric = 0;
-    float* d_vec = nullptr;
-    int32_t* d_nbrs = nullptr;
-    int32_t* d_start = nullptr;
-    uint32_t* d_deleted = nullptr;
-    hipStream_t stream = nullptr;
-    int num_cu = 0;
-
-    // state of search_prepare
-    bool prepared = false;
-    int Q = 0, L = 0;
-    int slots_log2 = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
-    int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0, prepared_policy = 0;
-    size_t lds_bytes = 0;
-    size_t spill_words = 0;
-    uint32_t* d_spill = nullptr;
-    size_t spill_alloc_words = 0;
-    int32_t* d_counters = nullptr;
-    size_t counters_alloc = 0;
-    int* d_scalars = nullptr;  // [0] next_qid, [1] spill_count
-    unsigned long long* d_hit = nullptr;
-    unsigned long long* d_phase = nullptr;  // debug builds only
-    int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
-    int last_Q = 0;
-};
 
 extern "C" {
 

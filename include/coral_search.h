@@ -149,6 +149,18 @@ CORAL_API int coral_search(coral_index* idx, const float* h_queries, int32_t Q, 
 CORAL_API int coral_search_verify(coral_index* idx, const int32_t* d_ids_res, const int32_t* d_ids_gt,
                         int32_t Q, int32_t k, int64_t* hits);
 
+/* Exact k nearest neighbours of Q queries among the index's vectors by brute force:
+ * what the reference gets from faiss for ground truth (tests/comp_gt.cpp:119-176) and for
+ * the builder's k_b-NN (src/knn.cu:174-193).  Ordered by (distance, id); every distance is
+ * accumulated in dimension order by fused multiply-adds, the arithmetic of
+ * include/utils.cuh:254-275 / :307-323.  have_delete leaves tombstoned ids out.  Unfilled
+ * slots: id -1, +-FLT_MAX.  The *_gpu form takes device pointers (d_dists may be NULL). */
+CORAL_API int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q, int32_t k,
+                                       int32_t have_delete, int32_t* d_ids, float* d_dists, void* stream,
+                                       double* time_s);
+CORAL_API int coral_bruteforce_knn(coral_index* idx, const float* h_queries, int32_t Q, int32_t k,
+                                   int32_t have_delete, int32_t* h_ids, float* h_dists, double* time_s);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,6 +49,9 @@ def lib():
         _lib.oracle_bruteforce.restype = None
         _lib.oracle_bruteforce.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_int,
                                            C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        _lib.oracle_bruteforce_order.restype = None
+        _lib.oracle_bruteforce_order.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_int,
+                                                 C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         _lib.oracle_search_A.restype = C.c_int
         _lib.oracle_search_A.argtypes = [C.POINTER(OracleIndex), C.c_void_p, C.c_int, C.c_int, C.c_int,
                                          C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -157,13 +160,14 @@ def ref_search_in_cpu(prob, queries, k, L, M=None, nthreads=0):
     return ids, dists, stats, t.value
 
 
-def bruteforce(base, queries, k, metric=L2, deleted=None):
+def bruteforce(base, queries, k, metric=L2, deleted=None, order=-1):
+    """Exact kNN under (distance, id); order -1 = fp64 closed form, else an fp32 summation order."""
     base, q = _f32(base), _f32(queries)
     ids = np.empty((q.shape[0], k), np.int32)
     dists = np.empty((q.shape[0], k), np.float32)
     d = None if deleted is None else np.ascontiguousarray(deleted, dtype=np.uint32)
-    lib().oracle_bruteforce(_p(base), base.shape[0], base.shape[1], _p(q), q.shape[0], k, metric, _p(d),
-                            _p(ids), _p(dists))
+    lib().oracle_bruteforce_order(_p(base), base.shape[0], base.shape[1], _p(q), q.shape[0], k, metric, order,
+                                  _p(d), _p(ids), _p(dists))
     return ids, dists
 
 

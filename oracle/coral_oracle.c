@@ -623,8 +623,45 @@ ORACLE_API int64_t oracle_recall_hits(int q_num, int k, int gt_dim, const int32_
     return total;
 }
 
-/* Exact brute-force kNN under (distance,id), fp64 accumulation then rounded to
- * fp32: the closed form every approximate result is scored against. */
+/* Exact brute-force kNN under (distance,id).  order < 0: fp64 accumulation then rounded to
+ * fp32 (the closed form every approximate result is scored against); order >= 0: fp32 in that
+ * summation order (ORDER_GPU_SEQ is what the brute-force HIP kernel computes). */
+ORACLE_API void oracle_bruteforce_order(const float* base, int64_t n, int dim, const float* queries,
+                                        int Q, int k, int metric, int order, const uint32_t* deleted,
+                                        int32_t* ids, float* dists) {
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int qi = 0; qi < Q; ++qi) {
+        bent* all = (bent*)malloc((size_t)n * sizeof(bent));
+        int64_t m = 0;
+        const float* q = queries + (size_t)qi * dim;
+        for (int64_t i = 0; i < n; ++i) {
+            if (is_deleted(deleted, (int32_t)i)) continue;
+            const float* b = base + (size_t)i * dim;
+            float s;
+            if (order < 0) {
+                double acc = 0.0;
+                for (int d = 0; d < dim; ++d)
+                    acc += metric == ORACLE_L2 ? ((double)q[d] - b[d]) * ((double)q[d] - b[d])
+                                               : -(double)q[d] * b[d];
+                s = (float)acc;
+            } else {
+                const float d = dist_any(q, b, dim, metric, order);
+                s = metric == ORACLE_IP ? 0.0f - d : d;
+            }
+            all[m].id = (int32_t)i, all[m].s = s, all[m].expanded = 0;
+            ++m;
+        }
+        qsort(all, (size_t)m, sizeof(bent), bent_cmp);
+        for (int j = 0; j < k; ++j) {
+            ids[(size_t)qi * k + j] = j < m ? all[j].id : -1;
+            if (dists)
+                dists[(size_t)qi * k + j] =
+                    j < m ? (metric == ORACLE_IP ? 0.0f - all[j].s : all[j].s) : farthest(metric);
+        }
+        free(all);
+    }
+}
+
 ORACLE_API void oracle_bruteforce(const float* base, int64_t n, int dim, const float* queries,
                                   int Q, int k, int metric, const uint32_t* deleted, int32_t* ids,
                                   float* dists) {

@@ -25,3 +25,17 @@ def ref(orc):
     if r is None:
         pytest.skip("oracle/_ref is not built (the reference tree is absent)")
     return r
+
+
+@pytest.fixture(scope="session", autouse=True)
+def _torch_runtime_first():
+    """Tests use torch as plumbing (graph construction, device buffers) next to the library.
+    PyTorch wheels carry their own HIP runtime; initialising it before libcoral_search.so
+    touches the device keeps both on one runtime instance whatever order the tests run in."""
+    try:
+        import torch
+        if torch.cuda.is_available():
+            torch.cuda.init()
+    except ImportError:
+        pass
+    yield
