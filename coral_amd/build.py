@@ -26,7 +26,7 @@ HOST = ["-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include"]
 
 LIB_SOURCES = ["beam_search.hip", "bruteforce.hip", "coral_search.cpp", "bruteforce_api.cpp", "formats.cpp",
                "index_gpu.cpp"]
-CLI_SOURCES = ["test_search_pipeline.cpp"]
+CLI_SOURCES = ["test_search_pipeline.cpp", "comp_gt.cpp"]
 
 
 def _run(cmd):
@@ -55,7 +55,8 @@ def build(verbose=True):
     for src in CLI_SOURCES:
         path = os.path.join(CSRC, src)
         if os.path.exists(path):
-            _run([HIPCC] + COMMON + HOST + [path, "-o", CLI, "-L" + LIBDIR, "-lcoral_search", "-Wl,-rpath,$ORIGIN"])
+            exe = os.path.join(LIBDIR, os.path.splitext(src)[0])
+            _run([HIPCC] + COMMON + HOST + [path, "-o", exe, "-L" + LIBDIR, "-lcoral_search", "-Wl,-rpath,$ORIGIN"])
     return LIB
 
 

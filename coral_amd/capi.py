@@ -96,13 +96,18 @@ class Index:
     """An HBM-resident index (vectors + compact graph rows + start ids)."""
 
     def __init__(self, base, nbrs, start_ids, metric=L2, device=0):
+        """nbrs=None makes a vectors-only index (brute force only)."""
         base = np.ascontiguousarray(base, dtype=np.float32)
-        nbrs = np.ascontiguousarray(nbrs, dtype=np.int32)
-        start_ids = np.ascontiguousarray(start_ids, dtype=np.int32)
-        if base.ndim != 2 or nbrs.ndim != 2 or nbrs.shape[0] != base.shape[0]:
-            raise ValueError("base must be [n,dim] and nbrs [n,R]")
-        d = IndexDesc(_ptr(base), _ptr(nbrs), base.shape[0], base.shape[1], nbrs.shape[1], _ptr(start_ids),
-                      start_ids.size, metric, device)
+        if nbrs is None:
+            nbrs, start_ids = np.empty((base.shape[0], 0), np.int32), np.empty(0, np.int32)
+            d = IndexDesc(_ptr(base), None, base.shape[0], base.shape[1], 0, None, 0, metric, device)
+        else:
+            nbrs = np.ascontiguousarray(nbrs, dtype=np.int32)
+            start_ids = np.ascontiguousarray(start_ids, dtype=np.int32)
+            if base.ndim != 2 or nbrs.ndim != 2 or nbrs.shape[0] != base.shape[0]:
+                raise ValueError("base must be [n,dim] and nbrs [n,R]")
+            d = IndexDesc(_ptr(base), _ptr(nbrs), base.shape[0], base.shape[1], nbrs.shape[1], _ptr(start_ids),
+                          start_ids.size, metric, device)
         h = C.c_void_p()
         _check(lib().coral_index_create(C.byref(d), C.byref(h)))
         self._h = h

@@ -84,14 +84,17 @@ static int validate_graph(const int32_t* nbrs, int64_t n, int R, const int32_t* 
 int coral_index_create(const coral_index_desc* d, coral_index** out) {
     if (!d || !out) return fail(CORAL_ERR_ARG, "null argument");
     *out = nullptr;
-    if (!d->base || !d->nbrs) return fail(CORAL_ERR_ARG, "null base or nbrs");
+    if (!d->base) return fail(CORAL_ERR_ARG, "null base");
+    const bool vectors_only = d->nbrs == nullptr;  // enough for coral_bruteforce_knn*
     if (d->n <= 0 || d->n > 0x7fffffffLL) return fail(CORAL_ERR_ARG, "n out of range");
     if (d->dim <= 0 || d->dim % 4 != 0 || d->dim > 2048)
         return fail(CORAL_ERR_ARG, "dim must be a positive multiple of 4, at most 2048 (got %d)",
                     d->dim);
-    if (d->R <= 0 || d->R > 32) return fail(CORAL_ERR_ARG, "R must be in 1..32 (got %d)", d->R);
     if (d->metric != CORAL_L2 && d->metric != CORAL_IP) return fail(CORAL_ERR_ARG, "bad metric");
-    if (int rc = validate_graph(d->nbrs, d->n, d->R, d->start_ids, d->n_start)) return rc;
+    if (!vectors_only) {
+        if (d->R <= 0 || d->R > 32) return fail(CORAL_ERR_ARG, "R must be in 1..32 (got %d)", d->R);
+        if (int rc = validate_graph(d->nbrs, d->n, d->R, d->start_ids, d->n_start)) return rc;
+    }
 
     int ndev = 0;
     hipError_t e = hipGetDeviceCount(&ndev);
@@ -102,8 +105,8 @@ int coral_index_create(const coral_index_desc* d, coral_index** out) {
 
     coral_index* idx = new (std::nothrow) coral_index();
     if (!idx) return fail(CORAL_ERR_MEMORY, "host allocation failed");
-    idx->device = d->device, idx->n = d->n, idx->dim = d->dim, idx->R = d->R;
-    idx->M = d->n_start, idx->metric = d->metric;
+    idx->device = d->device, idx->n = d->n, idx->dim = d->dim, idx->R = vectors_only ? 0 : d->R;
+    idx->M = vectors_only ? 0 : d->n_start, idx->metric = d->metric;
     hipDeviceProp_t prop;
     auto cleanup = [&](int rc) {
         coral_index_destroy(idx);
@@ -120,16 +123,20 @@ int coral_index_create(const coral_index_desc* d, coral_index** out) {
     idx->num_cu = prop.multiProcessorCount;
     HIP_TRY_C(hipStreamCreate(&idx->stream));
     const size_t vec_bytes = (size_t)d->n * d->dim * sizeof(float);
-    const size_t nbr_bytes = (size_t)d->n * d->R * sizeof(int32_t);
+    const size_t nbr_bytes = vectors_only ? 0 : (size_t)d->n * d->R * sizeof(int32_t);
     HIP_TRY_C(hipMalloc(&idx->d_vec, vec_bytes));
-    HIP_TRY_C(hipMalloc(&idx->d_nbrs, nbr_bytes));
-    HIP_TRY_C(hipMalloc(&idx->d_start, (size_t)d->n_start * sizeof(int32_t)));
+    if (!vectors_only) {
+        HIP_TRY_C(hipMalloc(&idx->d_nbrs, nbr_bytes));
+        HIP_TRY_C(hipMalloc(&idx->d_start, (size_t)d->n_start * sizeof(int32_t)));
+    }
     HIP_TRY_C(hipMalloc(&idx->d_scalars, 4 * sizeof(int)));
     HIP_TRY_C(hipMalloc(&idx->d_hit, sizeof(unsigned long long)));
     HIP_TRY_C(hipMemcpy(idx->d_vec, d->base, vec_bytes, hipMemcpyHostToDevice));
-    HIP_TRY_C(hipMemcpy(idx->d_nbrs, d->nbrs, nbr_bytes, hipMemcpyHostToDevice));
-    HIP_TRY_C(hipMemcpy(idx->d_start, d->start_ids, (size_t)d->n_start * sizeof(int32_t),
-                        hipMemcpyHostToDevice));
+    if (!vectors_only) {
+        HIP_TRY_C(hipMemcpy(idx->d_nbrs, d->nbrs, nbr_bytes, hipMemcpyHostToDevice));
+        HIP_TRY_C(hipMemcpy(idx->d_start, d->start_ids, (size_t)d->n_start * sizeof(int32_t),
+                            hipMemcpyHostToDevice));
+    }
 #undef HIP_TRY_C
     *out = idx;
     return CORAL_OK;
@@ -156,6 +163,7 @@ void coral_index_destroy(coral_index* idx) {
 int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const int32_t* start_ids,
                           int32_t n_start) {
     if (!idx || !nbrs) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
     if (int rc = validate_graph(nbrs, idx->n, idx->R, start_ids, n_start)) return rc;
     HIP_TRY(hipSetDevice(idx->device));
     HIP_TRY(hipStreamSynchronize(idx->stream));
@@ -202,6 +210,7 @@ int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* 
 
 int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tuning* tuning) {
     if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
     if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
     if (L <= 0 || L > kMaxL) return fail(CORAL_ERR_ARG, "L must be in 1..%d (got %d)", kMaxL, L);
     if (idx->M > L)

@@ -66,7 +66,7 @@ typedef struct coral_index coral_index;
  * of coral_index_create only (the data is copied into HBM). */
 typedef struct {
     const float* base;        /* [n][dim] fp32 row major; dim % 4 == 0 */
-    const int32_t* nbrs;      /* [n][R] compact rows, -1 padded */
+    const int32_t* nbrs;      /* [n][R] compact rows, -1 padded; NULL = vectors only (brute force) */
     int64_t n;
     int32_t dim;
     int32_t R;                /* row width, <= 32 (MAX_DEGREE, include/uni.h:60) */

@@ -10,6 +10,39 @@ pytestmark = pytest.mark.gpu
 SEQ = 0  # ORDER_GPU_SEQ
 
 
+def test_comp_gt_tool_and_vectors_only_index(orc, tmp_path):
+    """The ground-truth driver: fbin in, gt file out (layout of tests/comp_gt.cpp:142-175)."""
+    import os
+    import subprocess
+    from coral_amd import formats
+    n, dim, Q, k = 6000, 100, 50, 20
+    base = synth.gaussian_matrix(5, n, dim)
+    q = synth.shifted_queries(Q, dim, 6, 7, 8)
+    formats.fbin_write(tmp_path / "base.fbin", base)
+    formats.fbin_write(tmp_path / "query.fbin", q)
+    tool = os.path.join(os.path.dirname(capi.LIB_PATH), "comp_gt")
+    for dist, m in (("l2", capi.L2), ("ip", capi.IP)):
+        r = subprocess.run([tool, "--base_data_path", str(tmp_path / "base.fbin"), "--query_data_path",
+                            str(tmp_path / "query.fbin"), "--gt_save_file", str(tmp_path / "gt.bin"), "--k", str(k),
+                            "--nq", "40", "--dist", dist], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stderr
+        gt = formats.gt_read(tmp_path / "gt.bin")
+        assert gt.shape == (40, k)
+        b2, q2 = (formats.normalize_l2(base), formats.normalize_l2(q)) if dist == "ip" else (base, q)
+        oi, _ = orc.bruteforce(b2, q2[:40], k, m, order=SEQ)
+        assert np.array_equal(gt, oi)
+    r = subprocess.run([tool, "--dist", "l2"], capture_output=True, text=True)
+    assert r.returncode == 255 and "required but missing" in r.stderr
+    # a vectors-only index serves brute force and refuses graph search
+    idx = capi.Index(base, None, None)
+    ids, _, _ = idx.bruteforce(q, k)
+    assert np.array_equal(ids, orc.bruteforce(base, q, k, order=SEQ)[0])
+    with pytest.raises(capi.CoralError) as e:
+        idx.search(q, 5, 16)
+    assert e.value.code == capi.ERR_STATE
+    idx.close()
+
+
 def ring(n, R=2):
     g = np.full((n, R), -1, np.int32)
     g[:, 0] = (np.arange(n) + 1) % n
