@@ -148,7 +148,22 @@ __global__ __launch_bounds__(256) void row_select_kernel(const float* __restrict
         __syncthreads();
         const uint32_t prefix = s_prefix;
         const uint32_t himask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-        for (int64_t i = tid; i < n; i += 256) {
+        // rows start 16-byte aligned (ldD is a multiple of 4): float4 loads, two per thread in flight
+        const int64_t n4 = n >> 2;
+        const float4* row4 = reinterpret_cast<const float4*>(row);
+        for (int64_t i = tid; i < n4; i += 512) {
+            const float4 v0 = row4[i];
+            const bool two = i + 256 < n4;
+            const float4 v1 = two ? row4[i + 256] : v0;
+            const float e[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (j >= 4 && !two) break;
+                const uint32_t o = bf_ord32(e[j]);
+                if ((o & himask) == prefix) atomicAdd(&hist[(o >> shift) & 255u], 1u);
+            }
+        }
+        for (int64_t i = (n4 << 2) + tid; i < n; i += 256) {
             const uint32_t o = bf_ord32(row[i]);
             if ((o & himask) == prefix) atomicAdd(&hist[(o >> shift) & 255u], 1u);
         }
@@ -173,6 +188,16 @@ __global__ __launch_bounds__(256) void row_select_kernel(const float* __restrict
     const int lane = tid & 63, wave = tid >> 6;
     __shared__ unsigned int w_eq[4];
     for (int64_t i0 = 0; i0 < n; i0 += 256) {
+        // almost every stretch of the row holds no winner: look at 1024 entries at a time with
+        // float4 loads and step over the stretches without any
+        if ((i0 & 1023) == 0 && i0 + 1024 <= n) {
+            const float4 v = reinterpret_cast<const float4*>(row + i0)[tid];
+            const bool hit = bf_ord32(v.x) <= vk || bf_ord32(v.y) <= vk || bf_ord32(v.z) <= vk || bf_ord32(v.w) <= vk;
+            if (!__syncthreads_or(hit)) {
+                i0 += 768;  // the loop adds the last 256
+                continue;
+            }
+        }
         const int64_t i = i0 + tid;
         uint32_t o = 0xffffffffu;
         bool lt = false, eq = false;
