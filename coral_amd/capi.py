@@ -52,6 +52,8 @@ SIGNATURES = {
     "coral_index_destroy": (None, [C.c_void_p]),
     "coral_index_set_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
     "coral_index_set_deleted": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "coral_index_mark_deleted": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
+    "coral_index_get_deleted": (C.c_int, [C.c_void_p, C.c_void_p]),
     "coral_index_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32),
                                    C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "coral_search_prepare": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(Tuning)]),
@@ -64,6 +66,7 @@ SIGNATURES = {
                                       C.POINTER(C.c_int64)]),
     "coral_bruteforce_knn_gpu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                            C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]),
+    "coral_start_ids_fps": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                        C.c_void_p, C.POINTER(C.c_double)]),
 }
@@ -138,6 +141,16 @@ class Index:
             raise ValueError("mask must hold ceil(n/32) words")
         _check(lib().coral_index_set_deleted(self._h, _ptr(m)))
 
+    def mark_deleted(self, ids):
+        """Tombstone the given ids on the device (GPUFuncs::del_node_mark); earlier tombstones stay."""
+        ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+        _check(lib().coral_index_mark_deleted(self._h, _ptr(ids) if ids.size else None, ids.size))
+
+    def get_deleted(self):
+        m = np.empty((self.n + 31) // 32, np.uint32)
+        _check(lib().coral_index_get_deleted(self._h, _ptr(m)))
+        return m
+
     def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS):
         t = Tuning(visited_slots_log2, workgroups, threads, policy)
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
@@ -182,6 +195,12 @@ class Index:
         _check(lib().coral_bruteforce_knn_gpu(self._h, d_queries, Q, k, int(have_delete), d_ids, d_dists, stream,
                                               C.byref(t)))
         return t.value
+
+    def start_ids_fps(self, first_id, M):
+        """M entry points by farthest-point sampling in hop distance, starting from first_id."""
+        out = np.empty(M, dtype=np.int32)
+        _check(lib().coral_start_ids_fps(self._h, int(first_id), M, _ptr(out)))
+        return out
 
     def verify(self, d_ids_res, d_ids_gt, Q, k):
         hits = C.c_int64()

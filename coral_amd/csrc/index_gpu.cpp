@@ -151,6 +151,12 @@ void IndexGPU::LoadRoarGraph(std::string filename) {
     if (coral_index_set_graph(index_, nbrs_.data(), start_ids_.data(), 1)) raise("LoadRoarGraph");
 }
 
+void IndexGPU::Delete(const std::vector<int> del_ids) {
+    if (!index_) throw std::runtime_error("Delete before RunPrepare");
+    if (coral_index_mark_deleted(index_, del_ids.data(), (int32_t)del_ids.size())) raise("Delete");
+    have_delete_ = true;
+}
+
 void IndexGPU::SetDeleted(const uint32_t* mask_words) {
     if (!index_) throw std::runtime_error("SetDeleted before RunPrepare");
     if (coral_index_set_deleted(index_, mask_words)) raise("SetDeleted");

@@ -117,6 +117,13 @@ CORAL_API int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const
  * host_mask holds ceil(n/32) words, or NULL to clear. */
 CORAL_API int coral_index_set_deleted(coral_index* idx, const uint32_t* host_mask);
 
+/* GPUFuncs::del_node_mark (src/update.cu:406-412, 660-672): ORs the bits of count host ids into the mask
+ * (allocated and cleared on first use).  Ids outside [0, n) are skipped and reported as CORAL_ERR_GRAPH
+ * after the valid ones were marked; the reference does not check.  coral_index_get_deleted copies the
+ * mask back, ceil(n/32) words. */
+CORAL_API int coral_index_mark_deleted(coral_index* idx, const int32_t* h_ids, int32_t count);
+CORAL_API int coral_index_get_deleted(coral_index* idx, uint32_t* host_mask);
+
 CORAL_API int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* R,
                      int32_t* n_start, int32_t* metric);
 
@@ -160,6 +167,12 @@ CORAL_API int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries,
                                        double* time_s);
 CORAL_API int coral_bruteforce_knn(coral_index* idx, const float* h_queries, int32_t Q, int32_t k,
                                    int32_t have_delete, int32_t* h_ids, float* h_dists, double* time_s);
+
+/* Entry points by farthest-point sampling in hop distance, Graph::FPS (src/start.cu:74-145): out_ids[0] =
+ * first_id; each further id is the node whose smallest hop count from the ids chosen so far is largest
+ * (lowest id on ties; nodes unreachable from them are never chosen).  The reference draws first_id from
+ * std::random_device among nodes with a non-empty row; here the caller names it.  Writes M ids. */
+CORAL_API int coral_start_ids_fps(coral_index* idx, int32_t first_id, int32_t M, int32_t* out_ids);
 
 #ifdef __cplusplus
 }

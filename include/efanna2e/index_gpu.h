@@ -97,6 +97,9 @@ class CORAL_API IndexGPU {
     Test_Result Search_and_Verify(const float* queries, const int* gts, int num, int beam_capacity = 0);
     // src/graph.cu:709-743
     void LoadRoarGraph(std::string filename);
+    // src/index_gpu.cpp:138-206 with upd_type 0: the ids are tombstoned on the device (del_node_mark,
+    // src/update.cu:660-672) and later searches leave them out of their results; the graph is not repaired
+    void Delete(const std::vector<int> del_ids);
 
     // --- beyond the reference ---
     void SetPolicy(int coral_policy) { policy_ = coral_policy; }

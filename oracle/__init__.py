@@ -171,6 +171,15 @@ def bruteforce(base, queries, k, metric=L2, deleted=None, order=-1):
     return ids, dists
 
 
+def fps(nbrs, first, M):
+    nbrs = _i32(nbrs)
+    out = np.empty(M, np.int32)
+    fn = lib().oracle_fps
+    fn.restype, fn.argtypes = None, [C.c_void_p, C.c_int64, C.c_int, C.c_int32, C.c_int, C.c_void_p]
+    fn(_p(nbrs), nbrs.shape[0], nbrs.shape[1], int(first), M, _p(out))
+    return out
+
+
 def recall_hits(res, gt, k):
     res, gt = _i32(res), _i32(gt)
     return int(lib().oracle_recall_hits(res.shape[0], k, gt.shape[1], _p(res), _p(gt)))

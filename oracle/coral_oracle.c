@@ -690,6 +690,45 @@ ORACLE_API void oracle_bruteforce(const float* base, int64_t n, int dim, const f
     }
 }
 
+/* Graph::FPS, src/start.cu:74-145 with bfs :53-72 and update_min_hop_kernel :20-30: out[0] = first;
+ * then repeatedly BFS from the id chosen last, min_hops = per-node minimum over the searches
+ * (INT_MAX before the first, -1 for nodes no search has reached), next id = arg-max of min_hops with
+ * the lowest index on ties. */
+ORACLE_API void oracle_fps(const int32_t* nbrs, int64_t n, int R, int32_t first, int M, int32_t* out) {
+    int32_t* hops = (int32_t*)malloc((size_t)n * 4);
+    int32_t* minh = (int32_t*)malloc((size_t)n * 4);
+    int32_t* queue = (int32_t*)malloc((size_t)n * 4);
+    for (int64_t i = 0; i < n; ++i) minh[i] = INT32_MAX;
+    int32_t start = first;
+    int count = 0;
+    out[count++] = start;
+    while (count < M) {
+        for (int64_t i = 0; i < n; ++i) hops[i] = -1;
+        int64_t head = 0, tail = 0;
+        hops[start] = 0;
+        queue[tail++] = start;
+        while (head < tail) {
+            const int32_t u = queue[head++];
+            const int32_t* row = nbrs + (size_t)u * R;
+            for (int j = 0; j < R && row[j] >= 0; ++j)
+                if (hops[row[j]] < 0) hops[row[j]] = hops[u] + 1, queue[tail++] = row[j];
+        }
+        for (int64_t i = 0; i < n; ++i) {
+            if (hops[i] >= 0) {
+                if (hops[i] < minh[i] || minh[i] < 0) minh[i] = hops[i];
+            } else if (minh[i] == INT32_MAX) {
+                minh[i] = -1;
+            }
+        }
+        int64_t best = 0;
+        for (int64_t i = 1; i < n; ++i)
+            if (minh[i] > minh[best]) best = i;
+        start = (int32_t)best;
+        out[count++] = start;
+    }
+    free(hops), free(minh), free(queue);
+}
+
 ORACLE_API int oracle_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

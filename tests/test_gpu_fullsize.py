@@ -57,4 +57,9 @@ def test_full_size_properties(orc):
     gt = torch.topk(d, k, dim=1, largest=False).indices.to(torch.int32)
     hits = idx.verify(torch.from_numpy(ids[sub]).cuda().data_ptr(), gt.data_ptr(), len(sub), k)
     assert hits == orc.recall_hits(ids[sub], gt.cpu().numpy(), k)
+    # entry points by hop-distance farthest-point sampling: the 16 ids the oracle picks on this graph
+    print("farthest-point sampling of 16 start ids", flush=True)
+    fps = idx.start_ids_fps(int(starts[0]), 16)
+    assert fps.tolist() == orc.fps(nbrs, int(starts[0]), 16).tolist()
+    assert len(set(fps.tolist())) == 16
     idx.close()
