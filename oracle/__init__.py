@@ -180,6 +180,50 @@ def fps(nbrs, first, M):
     return out
 
 
+class GraphState:
+    """Rows under construction: nbrs [n][R] (-1 padded), dists [n][R], deg [n]; updated in place."""
+
+    def __init__(self, n, R):
+        self.nbrs = np.full((n, R), -1, np.int32)
+        self.dists = np.zeros((n, R), np.float32)
+        self.deg = np.zeros(n, np.int32)
+
+    def copy(self):
+        g = GraphState(0, self.nbrs.shape[1])
+        g.nbrs, g.dists, g.deg = self.nbrs.copy(), self.dists.copy(), self.deg.copy()
+        return g
+
+
+def nap_batch(base, state, knn, metric=L2, need_discard=True):
+    """One batch of the query-aware construction on `state`; returns [written, occlusion evals, member pairs]."""
+    base, knn = _f32(base), _i32(knn)
+    stats = np.zeros(3, np.int64)
+    fn = lib().oracle_nap_batch
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_int, C.c_int, C.c_int, C.c_void_p]
+    rc = fn(_p(base), base.shape[0], base.shape[1], metric, state.nbrs.shape[1], _p(state.nbrs), _p(state.dists),
+            _p(state.deg), _p(knn), knn.shape[0], knn.shape[1], int(bool(need_discard)), _p(stats))
+    if rc:
+        raise MemoryError("oracle_nap_batch")
+    return stats
+
+
+def enhance_batch(base, state, iso_ids, knn_ids, knn_dists, metric=L2):
+    """One batch of the connectivity enhancement; returns [reverse edges, rejected claims, distance evals]."""
+    base, iso_ids, knn_ids, knn_dists = _f32(base), _i32(iso_ids), _i32(knn_ids), _f32(knn_dists)
+    stats = np.zeros(3, np.int64)
+    fn = lib().oracle_enhance_batch
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+    rc = fn(_p(base), base.shape[0], base.shape[1], metric, state.nbrs.shape[1], _p(state.nbrs), _p(state.dists),
+            _p(state.deg), _p(iso_ids), _p(knn_ids), _p(knn_dists), iso_ids.size, knn_ids.shape[1], _p(stats))
+    if rc:
+        raise MemoryError("oracle_enhance_batch")
+    return stats
+
+
 def recall_hits(res, gt, k):
     res, gt = _i32(res), _i32(gt)
     return int(lib().oracle_recall_hits(res.shape[0], k, gt.shape[1], _p(res), _p(gt)))

@@ -729,6 +729,245 @@ ORACLE_API void oracle_fps(const int32_t* nbrs, int64_t n, int R, int32_t first,
     free(hops), free(minh), free(queue);
 }
 
+/* ------------------------------------------------------------ graph builder
+ *
+ * One batch of the query-aware construction, GPUFuncs::gpu_neibor_aware (src/upd_gpu.cu:260-303):
+ * every auxiliary query contributes its k_b nearest base ids (a "cluster"); every member of a cluster is a
+ * pivot whose candidate list holds the other members (only pairs where at least one side has no neighbours
+ * yet, src/upd_gpu.cu:53-73) and its own current neighbours (:48-52), sorted by distance to the pivot
+ * (:275-278), thinned by the occlusion rule (candidate_ignore_kernel, :203-247) and written back with the
+ * nearest discarded ones as filler (update_new_nbrs_kernel, :88-164).  Distances are the sequential fp32
+ * chain of include/utils.cuh:254-275 / :307-323.
+ *
+ * Two things the reference leaves to chance are fixed here, each to one of its possible outcomes:
+ *   - the sort (cub::DeviceSegmentedSort::SortPairs, src/utils.cu:219-262) is not stable; here ties keep
+ *     column order (members in cluster order, then current neighbours in row order);
+ *   - a base id that occurs in several clusters of a batch is written by whichever pivot thread wins
+ *     atomicTestAndSetBit (src/upd_gpu.cu:101); here the lowest pivot index wins.
+ * All pivots read the rows as they were before the batch (the kernels that read run before the one that writes).
+ *
+ * Parity status: nothing executable exists for these functions (the reference builder needs CUDA and faiss);
+ * they are pinned by code reading, by hand-computed cases, by an independent pure-Python restatement on small
+ * inputs and by the invariants of the occlusion rule (tests/test_oracle_builder.py).
+ */
+enum { ST_INITIAL = 0, ST_RETAINED = 1, ST_DISCARDED = 2, ST_REPEATED = 3, ST_INVALID = 4 };
+typedef struct {
+    int32_t id;
+    int32_t col;
+    int32_t status;
+    float dist;
+} cand_t;
+
+/* stable insertion sort by distance, closest first; invalid entries (farthest value) keep to the end */
+static void cand_sort(cand_t* c, int m, int metric) {
+    for (int i = 1; i < m; ++i) {
+        cand_t x = c[i];
+        int j = i - 1;
+        while (j >= 0 && closer(c[j].dist, x.dist, metric)) c[j + 1] = c[j], --j;
+        c[j + 1] = x;
+    }
+}
+
+/* candidate_ignore_kernel, src/upd_gpu.cu:203-247 (the same loop as src/enhance.cu:334-380) */
+static void cand_ignore(const float* base, int dim, int metric, cand_t* c, int m, int R, int64_t* dist_evals) {
+    int nbr_num = 0;
+    for (int i = 0; i < m && nbr_num < R; ++i) {
+        if (c[i].status == ST_INVALID) break;
+        if (c[i].status == ST_INITIAL) {
+            c[i].status = ST_RETAINED;
+            ++nbr_num;
+            const float* vi = base + (size_t)c[i].id * dim;
+            for (int j = i + 1; j < m; ++j) {
+                if (c[j].status == ST_INVALID) break;
+                if (c[j].id == c[i].id)
+                    c[j].status = ST_REPEATED;
+                else if (c[j].status == ST_INITIAL) {
+                    if (dist_evals) ++*dist_evals;
+                    if (closer(c[j].dist, dist_gpu_seq(vi, base + (size_t)c[j].id * dim, dim, metric), metric))
+                        c[j].status = ST_DISCARDED;
+                }
+            }
+        } else if (c[i].status == ST_DISCARDED) {
+            for (int j = i + 1; j < m; ++j) {
+                if (c[j].status == ST_INVALID) break;
+                if (c[j].id == c[i].id) c[j].status = ST_REPEATED;
+            }
+        }
+    }
+}
+
+/* update_new_nbrs_kernel, src/upd_gpu.cu:102-156 (and update_iso_nbrs_kernel, src/enhance.cu:528-568, which
+ * always fills): writes at most R entries, returns the new degree */
+static int cand_emit(const cand_t* c, int m, int R, int need_discard, int32_t* out_ids, float* out_dists) {
+    int retained = 0, n = 0;
+    for (int i = 0; i < m; ++i) {
+        if (c[i].status == ST_RETAINED) ++retained;
+        else if (c[i].status == ST_INVALID) break;
+    }
+    int discarded_need = need_discard ? R - retained : 0;
+    for (int j = 0; j < m && n < R; ++j) {
+        if (c[j].status == ST_RETAINED) {
+            out_ids[n] = c[j].id, out_dists[n] = c[j].dist, ++n;
+        } else if (c[j].status == ST_DISCARDED) {
+            if (discarded_need-- > 0) out_ids[n] = c[j].id, out_dists[n] = c[j].dist, ++n;
+        } else if (c[j].status == ST_INVALID)
+            break;
+    }
+    return n;
+}
+
+/* nbrs [n][R] (-1 padded), dists [n][R], deg [n] are updated in place.  knn [batch][kb] holds distinct base
+ * ids per row.  stats (optional): [0] pivots written, [1] distance evaluations of the occlusion rule,
+ * [2] member-pair distances. */
+ORACLE_API int oracle_nap_batch(const float* base, int64_t n, int dim, int metric, int R, int32_t* nbrs,
+                                float* dists, int32_t* deg, const int32_t* knn, int batch, int kb,
+                                int need_discard, int64_t* stats) {
+    const int C = kb + R;
+    const int64_t P = (int64_t)batch * kb;
+    int32_t* owner = (int32_t*)malloc((size_t)n * sizeof(int32_t));
+    int32_t* new_ids = (int32_t*)malloc((size_t)P * R * sizeof(int32_t));
+    float* new_d = (float*)malloc((size_t)P * R * sizeof(float));
+    int32_t* new_deg = (int32_t*)malloc((size_t)P * sizeof(int32_t));
+    if (!owner || !new_ids || !new_d || !new_deg) return -1;
+    for (int64_t i = 0; i < n; ++i) owner[i] = -1;
+    for (int64_t p = 0; p < P; ++p)
+        if (owner[knn[p]] < 0) owner[knn[p]] = (int32_t)p;
+    int64_t written = 0, evals = 0, pairs = 0;
+#pragma omp parallel for schedule(dynamic, 1) reduction(+ : written, evals, pairs)
+    for (int b = 0; b < batch; ++b) {
+        const int32_t* ids = knn + (size_t)b * kb;
+        float* G = (float*)malloc((size_t)kb * kb * sizeof(float));
+        cand_t* c = (cand_t*)malloc((size_t)C * sizeof(cand_t));
+        /* member-pair distances, only where at least one side is still without neighbours */
+        for (int r = 0; r < kb; ++r)
+            for (int q = r + 1; q < kb; ++q) {
+                if (deg[ids[r]] > 0 && deg[ids[q]] > 0) continue;
+                G[r * kb + q] = G[q * kb + r] =
+                    dist_gpu_seq(base + (size_t)ids[r] * dim, base + (size_t)ids[q] * dim, dim, metric);
+                ++pairs;
+            }
+        for (int r = 0; r < kb; ++r) {
+            const int64_t p = (int64_t)b * kb + r;
+            const int32_t pid = ids[r];
+            new_deg[p] = -1;
+            if (owner[pid] != p) continue;
+            const int rdeg = deg[pid];
+            int m = 0;
+            for (int q = 0; q < C; ++q) {
+                cand_t e = {-1, q, ST_INVALID, farthest(metric)};
+                if (q < kb) {
+                    if (q != r && ids[q] != pid && !(rdeg > 0 && deg[ids[q]] > 0))
+                        e.id = ids[q], e.status = ST_INITIAL, e.dist = G[r * kb + q];
+                } else if (q - kb < rdeg) {
+                    e.id = nbrs[(size_t)pid * R + (q - kb)], e.status = ST_INITIAL;
+                    e.dist = dists[(size_t)pid * R + (q - kb)];
+                }
+                c[m++] = e;
+            }
+            cand_sort(c, m, metric);
+            cand_ignore(base, dim, metric, c, m, R, &evals);
+            new_deg[p] = cand_emit(c, m, R, need_discard, new_ids + (size_t)p * R, new_d + (size_t)p * R);
+            ++written;
+        }
+        free(G), free(c);
+    }
+    for (int64_t p = 0; p < P; ++p) {
+        if (new_deg[p] < 0) continue;
+        const int32_t pid = knn[p];
+        for (int j = 0; j < R; ++j) {
+            nbrs[(size_t)pid * R + j] = j < new_deg[p] ? new_ids[(size_t)p * R + j] : -1;
+            dists[(size_t)pid * R + j] = j < new_deg[p] ? new_d[(size_t)p * R + j] : 0.0f;
+        }
+        deg[pid] = new_deg[p];
+    }
+    if (stats) stats[0] = written, stats[1] = evals, stats[2] = pairs;
+    free(owner), free(new_ids), free(new_d), free(new_deg);
+    return 0;
+}
+
+/* One batch of the connectivity enhancement, GPUFuncs::enhance_neibor_aware_gpu (src/enhance.cu:660-689):
+ * iso_ids [batch] are nodes without neighbours, knn_ids / knn_dists [batch][kn] what the beam search found for
+ * their vectors (closest first; an id of -1 ends a list).
+ *   1. build_candidate_kernel (src/enhance.cu:131-208): every found node that no earlier (node, position) of this
+ *      batch has claimed (atomicTestAndSetBit in the reference; here the lowest node index, then the lowest
+ *      position, wins) takes the isolated node into its own distance-sorted row: insertion position by distance;
+ *      a full row accepts only when no closer neighbour occludes the newcomer and then evicts its farthest
+ *      neighbour that the newcomer occludes (else its last); a row with room accepts always.
+ *   2. the isolated node's own row: its found list through the occlusion rule, filled with discarded ones
+ *      (src/enhance.cu:334-380, 519-575).
+ * stats (optional): [0] reverse edges inserted, [1] claims rejected by a full row, [2] distance evaluations. */
+ORACLE_API int oracle_enhance_batch(const float* base, int64_t n, int dim, int metric, int R, int32_t* nbrs,
+                                    float* dists, int32_t* deg, const int32_t* iso_ids, const int32_t* knn_ids,
+                                    const float* knn_dists, int batch, int kn, int64_t* stats) {
+    uint8_t* claimed = (uint8_t*)calloc((size_t)n, 1);
+    cand_t* c = (cand_t*)malloc((size_t)kn * sizeof(cand_t));
+    if (!claimed || !c) return -1;
+    int64_t inserted = 0, rejected = 0, evals = 0;
+    for (int b = 0; b < batch; ++b) {
+        const int32_t iso = iso_ids[b];
+        const float* iv = base + (size_t)iso * dim;
+        for (int i = 0; i < kn; ++i) {
+            const int32_t v = knn_ids[(size_t)b * kn + i];
+            if (v < 0) break;
+            const float vd = knn_dists[(size_t)b * kn + i];
+            if (claimed[v]) continue;
+            claimed[v] = 1;
+            int32_t* row = nbrs + (size_t)v * R;
+            float* rd = dists + (size_t)v * R;
+            const int d = deg[v];
+            int pos = 0, valid = 1, out_pos;
+            for (; pos < d; ++pos) {
+                if (!closer(vd, rd[pos], metric)) break;
+                if (valid) {
+                    ++evals;
+                    if (closer(vd, dist_gpu_seq(iv, base + (size_t)row[pos] * dim, dim, metric), metric)) valid = 0;
+                }
+            }
+            if (d == R) {
+                if (!valid || pos >= d) {
+                    ++rejected;
+                    continue;
+                }
+                for (out_pos = d - 1; out_pos >= pos; --out_pos) {
+                    ++evals;
+                    if (closer(rd[out_pos], dist_gpu_seq(iv, base + (size_t)row[out_pos] * dim, dim, metric), metric))
+                        break;
+                }
+                if (out_pos < pos) out_pos = d - 1;
+            } else {
+                out_pos = d;
+                deg[v] = d + 1;
+            }
+            for (int j = out_pos; j > pos; --j) row[j] = row[j - 1], rd[j] = rd[j - 1];
+            row[pos] = iso, rd[pos] = vd;
+            ++inserted;
+        }
+    }
+    for (int b = 0; b < batch; ++b) {
+        const int32_t iso = iso_ids[b];
+        int m = 0;
+        for (int i = 0; i < kn; ++i) {
+            const int32_t v = knn_ids[(size_t)b * kn + i];
+            if (v < 0) break;
+            cand_t e = {v, i, ST_INITIAL, knn_dists[(size_t)b * kn + i]};
+            c[m++] = e;
+        }
+        cand_sort(c, m, metric);
+        cand_ignore(base, dim, metric, c, m, R, &evals);
+        int32_t ids[64];
+        float ds[64];
+        const int nd = cand_emit(c, m, R, 1, ids, ds);
+        for (int j = 0; j < R; ++j) {
+            nbrs[(size_t)iso * R + j] = j < nd ? ids[j] : -1;
+            dists[(size_t)iso * R + j] = j < nd ? ds[j] : 0.0f;
+        }
+        deg[iso] = nd;
+    }
+    if (stats) stats[0] = inserted, stats[1] = rejected, stats[2] = evals;
+    free(claimed), free(c);
+    return 0;
+}
+
 ORACLE_API int oracle_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();
