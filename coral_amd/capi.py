@@ -43,6 +43,33 @@ class Tuning(C.Structure):
                 ("policy", C.c_int32), ("reserved", C.c_int32 * 4)]
 
 
+class BuildParams(C.Structure):
+    _fields_ = [("R", C.c_int32), ("k_b", C.c_int32), ("batch", C.c_int32), ("need_discard", C.c_int32),
+                ("connect_enhance", C.c_int32), ("enhance_search_batch", C.c_int32), ("enhance_nap_batch", C.c_int32),
+                ("enhance_L", C.c_int32), ("n_start", C.c_int32), ("first_start_id", C.c_int32),
+                ("reserved", C.c_int32 * 6)]
+
+
+class BuildStats(C.Structure):
+    _fields_ = [("knn_s", C.c_double), ("nap_s", C.c_double), ("enhance_s", C.c_double), ("total_s", C.c_double),
+                ("batches", C.c_int64), ("isolated", C.c_int64), ("reverse_edges", C.c_int64),
+                ("reverse_rejected", C.c_int64), ("edges", C.c_int64)]
+
+    def as_dict(self):
+        return {f: getattr(self, f) for f, _ in self._fields_}
+
+
+def build_params(**kw):
+    """The reference's defaults (config.json, CLI), overridden by keyword."""
+    p = BuildParams()
+    _check(lib().coral_build_params_default(C.byref(p)))
+    for k, v in kw.items():
+        if not hasattr(p, k):
+            raise TypeError("no build parameter %r" % k)
+        setattr(p, k, v)
+    return p
+
+
 _lib = None
 
 # name -> (restype, argtypes); also the list of symbols the header declares
@@ -66,6 +93,15 @@ SIGNATURES = {
                                       C.POINTER(C.c_int64)]),
     "coral_bruteforce_knn_gpu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                            C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]),
+    "coral_build_params_default": (C.c_int, [C.c_void_p]),
+    "coral_build_begin": (C.c_int, [C.c_void_p, C.c_int32]),
+    "coral_build_end": (C.c_int, [C.c_void_p]),
+    "coral_build_nap_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32]),
+    "coral_build_enhance_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                            C.c_void_p, C.c_void_p]),
+    "coral_build_connect_enhance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "coral_build_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
+    "coral_index_get_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_start_ids_fps": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                        C.c_void_p, C.POINTER(C.c_double)]),
@@ -201,6 +237,51 @@ class Index:
         out = np.empty(M, dtype=np.int32)
         _check(lib().coral_start_ids_fps(self._h, int(first_id), M, _ptr(out)))
         return out
+
+    # ---- graph construction
+    def build_begin(self, R):
+        _check(lib().coral_build_begin(self._h, R))
+        self.R = R
+
+    def build_end(self):
+        _check(lib().coral_build_end(self._h))
+
+    def build_nap_batch(self, d_knn_ids, batch, k_b, need_discard=True):
+        """d_knn_ids: device pointer (int) to int32 [batch][k_b]."""
+        _check(lib().coral_build_nap_batch(self._h, d_knn_ids, batch, k_b, int(bool(need_discard))))
+
+    def build_enhance_batch(self, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn):
+        ins, rej = C.c_int64(), C.c_int64()
+        _check(lib().coral_build_enhance_batch(self._h, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn, C.byref(ins),
+                                               C.byref(rej)))
+        return ins.value, rej.value
+
+    def build_connect_enhance(self, params):
+        st = BuildStats()
+        _check(lib().coral_build_connect_enhance(self._h, C.byref(params), C.byref(st)))
+        self.n_start = params.n_start
+        return st
+
+    def build_graph(self, aux, params):
+        """IndexGPU::BuildGPU: the whole construction from host auxiliary queries [A][dim]."""
+        aux = np.ascontiguousarray(aux, dtype=np.float32)
+        st = BuildStats()
+        _check(lib().coral_build_graph(self._h, _ptr(aux), aux.shape[0], C.byref(params), C.byref(st)))
+        self.R, self.n_start = params.R, params.n_start
+        return st
+
+    def get_graph(self, with_build_state=False):
+        """(nbrs, start_ids) or, during a build, (nbrs, dists, deg, start_ids)."""
+        nbrs = np.empty((self.n, self.R), np.int32)
+        starts = np.empty(self.n_start, np.int32)
+        if not with_build_state:
+            _check(lib().coral_index_get_graph(self._h, _ptr(nbrs), None, None, _ptr(starts) if starts.size else None))
+            return nbrs, starts
+        dists = np.empty((self.n, self.R), np.float32)
+        deg = np.empty(self.n, np.int32)
+        _check(lib().coral_index_get_graph(self._h, _ptr(nbrs), _ptr(dists), _ptr(deg),
+                                           _ptr(starts) if starts.size else None))
+        return nbrs, dists, deg, starts
 
     def verify(self, d_ids_res, d_ids_gt, Q, k):
         hits = C.c_int64()

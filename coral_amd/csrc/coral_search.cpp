@@ -155,6 +155,7 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_scalars);
     (void)hipFree(idx->d_hit);
     (void)hipFree(idx->d_phase);
+    coral::free_build_state(idx);
     if (idx->h_counters) (void)hipHostFree(idx->h_counters);
     if (idx->stream) (void)hipStreamDestroy(idx->stream);
     delete idx;

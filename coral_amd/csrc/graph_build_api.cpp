@@ -1,0 +1,319 @@
+// graph_build_api.cpp -- coral_build_*: the query-aware graph construction behind the C ABI.
+//   coral_build_graph            IndexGPU::BuildGPU            src/index_gpu.cpp:308-383 (KNNTask :385-499, GraphTask :501-580)
+//   coral_build_nap_batch        GPUFuncs::graph_update        src/upd_disk.cu:218-224 -> gpu_neibor_aware, src/upd_gpu.cu:260-303
+//   coral_build_connect_enhance  GPUFuncs::gpu_connect_enhance src/enhance.cu:728-861 (enhance_mode 0, isolated nodes)
+//   coral_build_enhance_batch    GPUFuncs::enhance_neibor_aware_gpu src/enhance.cu:660-689
+#include <algorithm>
+#include <chrono>
+#include <climits>
+#include <vector>
+
+#include "beam_search.h"
+#include "graph_build.h"
+#include "index_internal.h"
+
+using coral::fail;
+
+namespace coral {
+void free_build_state(coral_index* idx) {
+    (void)hipFree(idx->d_nbr_dists), (void)hipFree(idx->d_deg), (void)hipFree(idx->d_owner);
+    (void)hipFree(idx->d_new_ids), (void)hipFree(idx->d_new_dists), (void)hipFree(idx->d_new_deg);
+    (void)hipFree(idx->d_len), (void)hipFree(idx->d_build_stats);
+    idx->d_nbr_dists = nullptr, idx->d_deg = nullptr, idx->d_owner = nullptr;
+    idx->d_new_ids = nullptr, idx->d_new_dists = nullptr, idx->d_new_deg = nullptr;
+    idx->d_len = nullptr, idx->d_build_stats = nullptr;
+    idx->stage_rows = 0, idx->len_alloc = 0;
+    idx->building = false;
+}
+}  // namespace coral
+
+namespace {
+
+double now_s() {
+    return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+int set_start_ids(coral_index* idx, const int32_t* ids, int M) {
+    if (M != idx->M) {
+        int32_t* p = nullptr;
+        HIP_TRY(hipMalloc(&p, (size_t)M * sizeof(int32_t)));
+        (void)hipFree(idx->d_start);
+        idx->d_start = p;
+        idx->M = M;
+        idx->prepared = false;
+    }
+    HIP_TRY(hipMemcpyAsync(idx->d_start, ids, (size_t)M * sizeof(int32_t), hipMemcpyHostToDevice, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    return CORAL_OK;
+}
+
+// ids outside [0, n) would be followed into memory that is not there: count them before any kernel uses them
+int check_ids(coral_index* idx, const int32_t* d_ids, int64_t count, bool minus_one_ok, const char* what) {
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)(idx->d_build_stats + 2), 2, 0u, idx->stream));
+    HIP_TRY(coral::launch_count_bad_ids(d_ids, count, idx->n, minus_one_ok ? 1 : 0, idx->d_build_stats + 2, idx->stream));
+    unsigned long long bad = 0;
+    HIP_TRY(hipMemcpyAsync(&bad, idx->d_build_stats + 2, sizeof(bad), hipMemcpyDeviceToHost, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    if (bad) return fail(CORAL_ERR_GRAPH, "%llu of %lld %s are outside [0,%lld)", bad, (long long)count, what, (long long)idx->n);
+    return CORAL_OK;
+}
+
+int ensure_stage(coral_index* idx, size_t rows) {
+    if (rows <= idx->stage_rows) return CORAL_OK;
+    (void)hipFree(idx->d_new_ids), (void)hipFree(idx->d_new_dists), (void)hipFree(idx->d_new_deg);
+    idx->d_new_ids = nullptr, idx->d_new_dists = nullptr, idx->d_new_deg = nullptr, idx->stage_rows = 0;
+    HIP_TRY(hipMalloc(&idx->d_new_ids, rows * idx->R * sizeof(int32_t)));
+    HIP_TRY(hipMalloc(&idx->d_new_dists, rows * idx->R * sizeof(float)));
+    HIP_TRY(hipMalloc(&idx->d_new_deg, rows * sizeof(int32_t)));
+    idx->stage_rows = rows;
+    return CORAL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int coral_build_params_default(coral_build_params* p) {
+    if (!p) return fail(CORAL_ERR_ARG, "null argument");
+    *p = coral_build_params{};
+    p->R = 32, p->k_b = 100, p->batch = 1024, p->need_discard = 1, p->connect_enhance = 1;
+    p->enhance_search_batch = 524288, p->enhance_nap_batch = 4096, p->enhance_L = 256;
+    p->n_start = 16, p->first_start_id = -1;
+    return CORAL_OK;
+}
+
+int coral_build_begin(coral_index* idx, int32_t R) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    if (R <= 0 || R > coral::kBuildMaxR) return fail(CORAL_ERR_ARG, "R must be in 1..%d (got %d)", coral::kBuildMaxR, R);
+    if (idx->d_nbrs && idx->R != R)
+        return fail(CORAL_ERR_ARG, "the index already holds rows of width %d (asked for %d)", idx->R, R);
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    coral::free_build_state(idx);
+    const size_t n = (size_t)idx->n;
+    if (!idx->d_nbrs) {
+        HIP_TRY(hipMalloc(&idx->d_nbrs, n * R * sizeof(int32_t)));
+        idx->R = R;
+    }
+    idx->prepared = false;
+    HIP_TRY(hipMalloc(&idx->d_nbr_dists, n * R * sizeof(float)));
+    HIP_TRY(hipMalloc(&idx->d_deg, n * sizeof(int32_t)));
+    HIP_TRY(hipMalloc(&idx->d_owner, n * sizeof(int32_t)));
+    HIP_TRY(hipMalloc(&idx->d_build_stats, 4 * sizeof(unsigned long long)));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_nbrs, n * R, 0xffffffffu, idx->stream));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_nbr_dists, n * R, 0u, idx->stream));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_deg, n, 0u, idx->stream));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_owner, n, (uint32_t)INT_MAX, idx->stream));
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_build_stats, 8, 0u, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    idx->building = true;
+    return CORAL_OK;
+}
+
+int coral_build_end(coral_index* idx) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    coral::free_build_state(idx);
+    return CORAL_OK;
+}
+
+int coral_build_nap_batch(coral_index* idx, const int32_t* d_knn_ids, int32_t batch, int32_t k_b, int32_t need_discard) {
+    if (!idx || !d_knn_ids) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->building) return fail(CORAL_ERR_STATE, "coral_build_begin has not been called");
+    if (batch <= 0) return fail(CORAL_ERR_ARG, "batch must be positive");
+    if (k_b < 2 || k_b > coral::kBuildMaxKb)
+        return fail(CORAL_ERR_ARG, "k_b must be in 2..%d (got %d)", coral::kBuildMaxKb, k_b);
+    if ((int64_t)batch * k_b > INT_MAX / 2) return fail(CORAL_ERR_ARG, "batch * k_b too large");
+    HIP_TRY(hipSetDevice(idx->device));
+    if (int rc = ensure_stage(idx, (size_t)batch * k_b)) return rc;
+    if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * k_b, false, "cluster ids")) return rc;
+    HIP_TRY(coral::launch_nap_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists, idx->d_deg,
+                                    idx->d_owner, d_knn_ids, batch, k_b, need_discard, idx->d_new_ids, idx->d_new_dists,
+                                    idx->d_new_deg, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    return CORAL_OK;
+}
+
+int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_ids, const int32_t* d_knn_ids,
+                              const float* d_knn_dists, int32_t batch, int32_t kn, int64_t* reverse_edges,
+                              int64_t* reverse_rejected) {
+    if (!idx || !d_iso_ids || !d_knn_ids || !d_knn_dists) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->building) return fail(CORAL_ERR_STATE, "coral_build_begin has not been called");
+    if (batch <= 0) return fail(CORAL_ERR_ARG, "batch must be positive");
+    if (kn < 1 || kn > coral::kBuildMaxKb + coral::kBuildMaxR)
+        return fail(CORAL_ERR_ARG, "found-list length must be in 1..%d (got %d)", coral::kBuildMaxKb + coral::kBuildMaxR, kn);
+    if ((int64_t)batch * kn > INT_MAX / 2) return fail(CORAL_ERR_ARG, "batch * list length too large");
+    HIP_TRY(hipSetDevice(idx->device));
+    if ((size_t)batch > idx->len_alloc) {
+        (void)hipFree(idx->d_len);
+        idx->d_len = nullptr, idx->len_alloc = 0;
+        HIP_TRY(hipMalloc(&idx->d_len, (size_t)batch * sizeof(int32_t)));
+        idx->len_alloc = (size_t)batch;
+    }
+    if (int rc = check_ids(idx, d_iso_ids, batch, false, "isolated ids")) return rc;
+    if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * kn, true, "found ids")) return rc;
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_build_stats, 4, 0u, idx->stream));
+    HIP_TRY(coral::launch_enhance_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists,
+                                        idx->d_deg, idx->d_owner, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn, idx->d_len,
+                                        idx->d_build_stats, idx->stream));
+    unsigned long long st[2] = {0, 0};
+    HIP_TRY(hipMemcpyAsync(st, idx->d_build_stats, sizeof(st), hipMemcpyDeviceToHost, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    if (reverse_edges) *reverse_edges = (int64_t)st[0];
+    if (reverse_rejected) *reverse_rejected = (int64_t)st[1];
+    return CORAL_OK;
+}
+
+int coral_build_connect_enhance(coral_index* idx, const coral_build_params* prm, coral_build_stats* stats) {
+    if (!idx || !prm) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->building) return fail(CORAL_ERR_STATE, "coral_build_begin has not been called");
+    if (prm->k_b < 1 || prm->k_b > prm->enhance_L) return fail(CORAL_ERR_ARG, "k_b must be in 1..enhance_L");
+    if (prm->n_start < 1 || prm->enhance_search_batch < 1 || prm->enhance_nap_batch < 1)
+        return fail(CORAL_ERR_ARG, "n_start and the enhancement batch sizes must be positive");
+    HIP_TRY(hipSetDevice(idx->device));
+    hipStream_t st = idx->stream;
+    const int64_t n = idx->n;
+    const int dim = idx->dim, kb = prm->k_b;
+    // load_isolated_nodes (src/enhance.cu:577-611): ids without neighbours, ascending
+    std::vector<int32_t> deg((size_t)n);
+    HIP_TRY(hipMemcpyAsync(deg.data(), idx->d_deg, (size_t)n * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    std::vector<int32_t> iso;
+    int32_t first = prm->first_start_id;
+    for (int64_t i = 0; i < n; ++i) {
+        if (deg[i] == 0)
+            iso.push_back((int32_t)i);
+        else if (first < 0)
+            first = (int32_t)i;
+    }
+    if (stats) stats->isolated = (int64_t)iso.size();
+    if (first < 0 || first >= n) return fail(CORAL_ERR_STATE, "no node has neighbours yet: nothing to search from");
+    if (deg[first] == 0) return fail(CORAL_ERR_ARG, "first_start_id %d has no neighbours", first);
+    std::vector<int32_t> starts((size_t)prm->n_start);
+    if (iso.empty()) {
+        if (int rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data())) return rc;
+        return set_start_ids(idx, starts.data(), prm->n_start);
+    }
+    const int64_t iso_num = (int64_t)iso.size();
+    const int64_t sb = std::min<int64_t>(prm->enhance_search_batch, iso_num);
+    int32_t *d_iso = nullptr, *d_res = nullptr;
+    float *d_iso_vec = nullptr, *d_res_d = nullptr;
+    auto release = [&]() { (void)hipFree(d_iso), (void)hipFree(d_res), (void)hipFree(d_iso_vec), (void)hipFree(d_res_d); };
+    int rc = CORAL_OK;
+    auto ok = [&](hipError_t e, const char* what) {
+        if (e == hipSuccess) return true;
+        rc = fail(e == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE, "%s failed: %s", what, hipGetErrorString(e));
+        return false;
+    };
+    if (ok(hipMalloc(&d_iso, (size_t)iso_num * sizeof(int32_t)), "hipMalloc") &&
+        ok(hipMalloc(&d_iso_vec, (size_t)sb * dim * sizeof(float)), "hipMalloc") &&
+        ok(hipMalloc(&d_res, (size_t)sb * kb * sizeof(int32_t)), "hipMalloc") &&
+        ok(hipMalloc(&d_res_d, (size_t)sb * kb * sizeof(float)), "hipMalloc"))
+        ok(hipMemcpy(d_iso, iso.data(), (size_t)iso_num * sizeof(int32_t), hipMemcpyHostToDevice), "hipMemcpy");
+    for (int64_t i = 0; rc == CORAL_OK && i < iso_num; i += sb) {
+        const int batch = (int)std::min<int64_t>(sb, iso_num - i);
+        // src/enhance.cu:793-795: fresh entry points on the graph as it is now, then one search over the batch
+        if ((rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data()))) break;
+        if ((rc = set_start_ids(idx, starts.data(), prm->n_start))) break;
+        if (!ok(coral::launch_gather_rows(idx->d_vec, dim, d_iso + i, batch, d_iso_vec, st), "gather")) break;
+        coral_tuning tun{};
+        tun.policy = CORAL_POLICY_ROUNDS;
+        if ((rc = coral_search_prepare(idx, batch, prm->enhance_L, &tun))) break;
+        if ((rc = coral_search_gpu(idx, d_iso_vec, d_res, d_res_d, batch, kb, CORAL_POLICY_ROUNDS, 0, nullptr, nullptr)))
+            break;
+        for (int64_t j = 0; j < batch; j += prm->enhance_nap_batch) {
+            const int b1 = (int)std::min<int64_t>(prm->enhance_nap_batch, batch - j);
+            int64_t ins = 0, rej = 0;
+            if ((rc = coral_build_enhance_batch(idx, d_iso + i + j, d_res + (size_t)j * kb, d_res_d + (size_t)j * kb, b1, kb,
+                                                &ins, &rej)))
+                break;
+            if (stats) stats->reverse_edges += ins, stats->reverse_rejected += rej;
+        }
+    }
+    release();
+    return rc;
+}
+
+int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const coral_build_params* prm,
+                      coral_build_stats* stats) {
+    if (!idx || !h_aux || !prm) return fail(CORAL_ERR_ARG, "null argument");
+    if (A <= 0) return fail(CORAL_ERR_ARG, "no auxiliary queries");
+    if (prm->batch <= 0) return fail(CORAL_ERR_ARG, "batch must be positive");
+    if (prm->k_b > idx->n) return fail(CORAL_ERR_ARG, "k_b exceeds the number of base vectors");
+    coral_build_stats local{};
+    coral_build_stats* S = stats ? stats : &local;
+    *S = coral_build_stats{};
+    const double t0 = now_s();
+    if (int rc = coral_build_begin(idx, prm->R)) return rc;
+    HIP_TRY(hipSetDevice(idx->device));
+    const int dim = idx->dim, kb = prm->k_b;
+    // the exact k_b-NN of a chunk of auxiliary queries at a time (KNNTask), then its batches in order (GraphTask)
+    const int64_t chunk = std::min<int64_t>(A, (int64_t)prm->batch * 8);
+    float* d_aux = nullptr;
+    int32_t* d_knn = nullptr;
+    int rc = CORAL_OK;
+    if (hipMalloc(&d_aux, (size_t)chunk * dim * sizeof(float)) != hipSuccess ||
+        hipMalloc(&d_knn, (size_t)chunk * kb * sizeof(int32_t)) != hipSuccess)
+        rc = fail(CORAL_ERR_MEMORY, "device allocation for the auxiliary queries failed");
+    for (int64_t a0 = 0; rc == CORAL_OK && a0 < A; a0 += chunk) {
+        const int64_t cq = std::min(chunk, A - a0);
+        if (hipMemcpy(d_aux, h_aux + (size_t)a0 * dim, (size_t)cq * dim * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+            rc = fail(CORAL_ERR_DEVICE, "upload of auxiliary queries failed");
+            break;
+        }
+        double t = 0.0;
+        if ((rc = coral_bruteforce_knn_gpu(idx, d_aux, (int32_t)cq, kb, 0, d_knn, nullptr, nullptr, &t))) break;
+        S->knn_s += t;
+        const double t1 = now_s();
+        for (int64_t b0 = 0; b0 < cq; b0 += prm->batch) {
+            const int b = (int)std::min<int64_t>(prm->batch, cq - b0);
+            if ((rc = coral_build_nap_batch(idx, d_knn + (size_t)b0 * kb, b, kb, prm->need_discard))) break;
+            ++S->batches;
+        }
+        S->nap_s += now_s() - t1;
+    }
+    (void)hipFree(d_aux), (void)hipFree(d_knn);
+    if (rc) return rc;
+    const double t2 = now_s();
+    if (prm->connect_enhance) {
+        if ((rc = coral_build_connect_enhance(idx, prm, S))) return rc;
+    } else {
+        std::vector<int32_t> deg((size_t)idx->n), starts((size_t)prm->n_start);
+        HIP_TRY(hipMemcpy(deg.data(), idx->d_deg, (size_t)idx->n * sizeof(int32_t), hipMemcpyDeviceToHost));
+        int32_t first = prm->first_start_id;
+        int64_t isolated = 0;
+        for (int64_t i = 0; i < idx->n; ++i) {
+            isolated += deg[i] == 0;
+            if (first < 0 && deg[i] > 0) first = (int32_t)i;
+        }
+        S->isolated = isolated;
+        if (first < 0) return fail(CORAL_ERR_STATE, "no node has neighbours");
+        if ((rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data()))) return rc;
+        if ((rc = set_start_ids(idx, starts.data(), prm->n_start))) return rc;
+    }
+    S->enhance_s = now_s() - t2;
+    std::vector<int32_t> deg((size_t)idx->n);
+    HIP_TRY(hipMemcpy(deg.data(), idx->d_deg, (size_t)idx->n * sizeof(int32_t), hipMemcpyDeviceToHost));
+    for (int32_t d : deg) S->edges += d;
+    S->total_s = now_s() - t0;
+    return CORAL_OK;
+}
+
+int coral_index_get_graph(coral_index* idx, int32_t* h_nbrs, float* h_dists, int32_t* h_deg, int32_t* h_start_ids) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given or built)");
+    if ((h_dists || h_deg) && !idx->building)
+        return fail(CORAL_ERR_STATE, "distances and degrees exist only between coral_build_begin and coral_build_end");
+    HIP_TRY(hipSetDevice(idx->device));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    const size_t cells = (size_t)idx->n * idx->R;
+    if (h_nbrs) HIP_TRY(hipMemcpy(h_nbrs, idx->d_nbrs, cells * sizeof(int32_t), hipMemcpyDeviceToHost));
+    if (h_dists) HIP_TRY(hipMemcpy(h_dists, idx->d_nbr_dists, cells * sizeof(float), hipMemcpyDeviceToHost));
+    if (h_deg) HIP_TRY(hipMemcpy(h_deg, idx->d_deg, (size_t)idx->n * sizeof(int32_t), hipMemcpyDeviceToHost));
+    if (h_start_ids && idx->M > 0)
+        HIP_TRY(hipMemcpy(h_start_ids, idx->d_start, (size_t)idx->M * sizeof(int32_t), hipMemcpyDeviceToHost));
+    return CORAL_OK;
+}
+
+}  // extern "C"

@@ -44,5 +44,23 @@ struct coral_index {
     unsigned long long* d_phase = nullptr;  // debug builds only
     int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
     int last_Q = 0;
+
+    // graph construction (coral_build_*): per-neighbour distances, degrees, the per-batch claim table
+    // (INT_MAX when idle) and the staging rows of one batch
+    bool building = false;
+    float* d_nbr_dists = nullptr;  // [n][R]
+    int32_t* d_deg = nullptr;      // [n]
+    int32_t* d_owner = nullptr;    // [n]
+    int32_t* d_new_ids = nullptr;
+    float* d_new_dists = nullptr;
+    int32_t* d_new_deg = nullptr;
+    size_t stage_rows = 0;
+    int32_t* d_len = nullptr;  // found-list lengths of one enhancement batch
+    size_t len_alloc = 0;
+    unsigned long long* d_build_stats = nullptr;  // [0] reverse edges inserted, [1] turned away, [2] ids out of range
 };
+
+namespace coral {
+void free_build_state(coral_index* idx);
+}
 

@@ -174,6 +174,81 @@ CORAL_API int coral_bruteforce_knn(coral_index* idx, const float* h_queries, int
  * std::random_device among nodes with a non-empty row; here the caller names it.  Writes M ids. */
 CORAL_API int coral_start_ids_fps(coral_index* idx, int32_t first_id, int32_t M, int32_t* out_ids);
 
+/* ---- Graph construction from auxiliary queries (IndexGPU::BuildGPU, src/index_gpu.cpp:308-383) ----
+ * Rows under construction live in the index itself, so a search may run at any point of a build (the
+ * connectivity enhancement does).  Two outcomes that the reference leaves to thread timing are fixed here:
+ * equal distances keep the order in which the candidates were listed (cluster order, then the current row),
+ * and a node that several clusters (or several isolated nodes) of one batch claim goes to the first of them. */
+typedef struct {
+    int32_t R;                    /* row width, <= 32: --M_pjbp, tests/test_build_pipeline.cpp:82 */
+    int32_t k_b;                  /* nearest base points per auxiliary query, 2..128: config.json "k" */
+    int32_t batch;                /* auxiliary queries per update: config.json "batch" (1024) */
+    int32_t need_discard;         /* fill rows with the nearest ruled-out candidates: config.json "need_discard" */
+    int32_t connect_enhance;      /* --CE: 0 = leave untouched nodes isolated, 1 = attach them afterwards */
+    int32_t enhance_search_batch; /* config.json "enhance_search_batch" (524288) */
+    int32_t enhance_nap_batch;    /* config.json "enhance_nap_batch" (4096) */
+    int32_t enhance_L;            /* beam capacity of the enhancement search: 256, src/enhance.cu:783 */
+    int32_t n_start;              /* entry points: config.json "search_start_nodes_num" (16) */
+    int32_t first_start_id;       /* first id of the farthest-point sampling (the reference draws it from
+                                     std::random_device, src/start.cu:77-86); -1 = lowest id that has neighbours */
+    int32_t reserved[6];
+} coral_build_params;
+
+typedef struct {
+    double knn_s;      /* exact k_b-NN of the auxiliary queries */
+    double nap_s;      /* batch updates */
+    double enhance_s;  /* connectivity enhancement, entry points included */
+    double total_s;
+    int64_t batches;
+    int64_t isolated;          /* nodes without neighbours after the batch updates */
+    int64_t reverse_edges;     /* isolated nodes inserted into rows of the nodes found for them */
+    int64_t reverse_rejected;  /* ... turned away by a full row */
+    int64_t edges;             /* sum of degrees at the end */
+} coral_build_stats;
+
+/* the values of the reference's config.json and CLI defaults */
+CORAL_API int coral_build_params_default(coral_build_params* p);
+
+/* Graph ctor in construction mode: every row empty.  On a vectors-only index this creates the rows. */
+CORAL_API int coral_build_begin(coral_index* idx, int32_t R);
+/* frees the per-neighbour distances and the staging; the rows and start ids stay */
+CORAL_API int coral_build_end(coral_index* idx);
+
+/* GPUFuncs::graph_update -> gpu_neibor_aware (src/upd_disk.cu:218-224, src/upd_gpu.cu:260-303): one batch of
+ * clusters, d_knn_ids int32 [batch][k_b] on the device, distinct ids per row.  Every member becomes a pivot:
+ * candidates = the other members (pairs where both sides already have neighbours are left out) + its current row;
+ * sorted by distance; occlusion rule; write-back (with need_discard, filled up to R with the nearest ruled-out). */
+CORAL_API int coral_build_nap_batch(coral_index* idx, const int32_t* d_knn_ids, int32_t batch, int32_t k_b,
+                                    int32_t need_discard);
+
+/* GPUFuncs::enhance_neibor_aware_gpu (src/enhance.cu:660-689): d_iso_ids [batch] nodes without neighbours,
+ * d_knn_ids / d_knn_dists [batch][kn] what the search found for their vectors (closest first, -1 ends a list).
+ * Each found node takes the first isolated node that lists it into its own row (src/enhance.cu:161-207); each
+ * isolated node gets its row from its list through the occlusion rule, filled (src/enhance.cu:334-380, 519-575). */
+CORAL_API int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_ids, const int32_t* d_knn_ids,
+                                        const float* d_knn_dists, int32_t batch, int32_t kn, int64_t* reverse_edges,
+                                        int64_t* reverse_rejected);
+
+/* GPUFuncs::gpu_connect_enhance, isolated nodes (src/enhance.cu:728-803, enhance_mode 0): per search batch, entry
+ * points by coral_start_ids_fps on the graph as it is, one CORAL_POLICY_ROUNDS search (k = k_b, L = enhance_L) for
+ * the isolated nodes' own vectors, then coral_build_enhance_batch per enhance_nap_batch.  The entry points of the
+ * last search batch stay the index's start ids, as in the reference.  Its second phase (top_hit_num most-hit nodes,
+ * src/enhance.cu:819-856) is not built: it is off by the code's default (src/index_gpu.cpp:78) and reads past its
+ * id array whenever top_hit_num exceeds n. */
+CORAL_API int coral_build_connect_enhance(coral_index* idx, const coral_build_params* params, coral_build_stats* stats);
+
+/* IndexGPU::BuildGPU: begin; exact k_b-NN of the A auxiliary queries (host, [A][dim]; what the reference asks faiss
+ * for, src/knn.cu:174-193) in order, `batch` at a time through coral_build_nap_batch; then the enhancement (or, with
+ * connect_enhance 0, just the entry points).  The index can be searched afterwards; call coral_build_end to drop the
+ * construction state. */
+CORAL_API int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const coral_build_params* params,
+                                coral_build_stats* stats);
+
+/* Download rows [n][R] (-1 padded) and start ids [n_start]; during a build also the per-neighbour distances
+ * [n][R] and degrees [n] (the dists and deg fields of the reference's Slot).  Any pointer may be NULL. */
+CORAL_API int coral_index_get_graph(coral_index* idx, int32_t* h_nbrs, float* h_dists, int32_t* h_deg,
+                                    int32_t* h_start_ids);
+
 #ifdef __cplusplus
 }
 #endif

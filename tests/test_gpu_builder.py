@@ -1,0 +1,169 @@
+"""Graph construction on the device (src/upd_gpu.cu:12-303, src/enhance.cu:131-208, 334-575, 660-803,
+src/index_gpu.cpp:308-580) against the oracle's restatement: rows, per-neighbour distances, degrees and start ids
+must be identical, batch by batch and for the whole pipeline."""
+import numpy as np
+import pytest
+
+from coral_amd import capi, synth
+from util import make_queries
+
+pytestmark = pytest.mark.gpu
+WAVE64 = 3  # the search kernel's summation order
+SEQ = 0  # one thread walks the row: the brute-force kernels and the builder
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_same_state(idx, st):
+    nbrs, dists, deg, _ = idx.get_graph(with_build_state=True)
+    assert np.array_equal(deg, st.deg)
+    assert np.array_equal(nbrs, st.nbrs)
+    assert dists.tobytes() == st.dists.tobytes()
+
+
+def base_of(n, dim, seed, metric):
+    base = synth.gaussian_matrix(seed, n, dim)
+    return synth.normalize_rows(base) if metric == capi.IP else base
+
+
+@pytest.mark.parametrize("n,dim,R,kb,batch,metric,need_discard,seed", [
+    (3000, 32, 8, 10, 64, capi.L2, 1, 0),
+    (3000, 32, 8, 10, 64, capi.L2, 0, 1),
+    (4000, 64, 32, 100, 24, capi.L2, 1, 2),
+    (4000, 64, 32, 100, 24, capi.IP, 1, 3),
+    (2000, 200, 16, 33, 40, capi.L2, 1, 4),
+    (2000, 8, 5, 128, 9, capi.IP, 0, 5),
+    (500, 4, 3, 2, 300, capi.L2, 1, 6),
+])
+def test_nap_batches_equal_the_oracle(orc, n, dim, R, kb, batch, metric, need_discard, seed):
+    rng = np.random.RandomState(seed)
+    base = base_of(n, dim, 50 + seed, metric)
+    if seed == 6:
+        base = np.round(base)  # ties and duplicate points
+    idx = capi.Index(base, None, None, metric=metric)
+    idx.build_begin(R)
+    st = orc.GraphState(n, R)
+    for it in range(5):
+        if it % 2 == 0:  # clusters of true neighbours: the exact kb-NN of shifted queries
+            q = make_queries(batch, dim, 900 + 10 * seed + it, "ip" if metric == capi.IP else "l2")
+            knn, _ = orc.bruteforce(base, q, kb, metric, order=SEQ)
+        else:  # arbitrary clusters, many ids shared between the clusters of the batch
+            pool = rng.choice(n, min(n, 4 * kb + 50), replace=False)
+            knn = np.stack([rng.choice(pool, kb, replace=False) for _ in range(batch)]).astype(np.int32)
+        t_knn = dev(knn)
+        idx.build_nap_batch(t_knn.data_ptr(), knn.shape[0], kb, need_discard)
+        orc.nap_batch(base, st, knn, metric=metric, need_discard=need_discard)
+        assert_same_state(idx, st)
+    idx.close()
+
+
+@pytest.mark.parametrize("metric,R,kn,seed", [(capi.L2, 8, 20, 0), (capi.IP, 32, 100, 1), (capi.L2, 5, 9, 2)])
+def test_enhance_batches_equal_the_oracle(orc, metric, R, kn, seed):
+    rng = np.random.RandomState(seed)
+    n, dim, linked_n = 3000, 32, 2400
+    base = base_of(n, dim, 70 + seed, metric)
+    idx = capi.Index(base, None, None, metric=metric)
+    idx.build_begin(R)
+    st = orc.GraphState(n, R)
+    for it in range(4):  # a graph over the first linked_n nodes, rows of every fill level
+        knn = np.stack([rng.choice(linked_n, 12, replace=False) for _ in range(150)]).astype(np.int32)
+        t_knn = dev(knn)
+        idx.build_nap_batch(t_knn.data_ptr(), 150, 12, it % 2)
+        orc.nap_batch(base, st, knn, metric=metric, need_discard=it % 2)
+    linked = np.where(st.deg > 0)[0].astype(np.int32)
+    sub = base[linked]
+    for lo in (linked_n, linked_n + 300):
+        iso = np.arange(lo, lo + 300, dtype=np.int32)
+        ids, dd = orc.bruteforce(sub, base[iso], kn, metric, order=SEQ)  # the nearest linked nodes stand in for the search
+        ids = linked[ids]
+        ids[5, kn // 2:] = -1  # a short list
+        t_iso, t_ids, t_dd = dev(iso), dev(ids), dev(dd)  # named: the device buffers must outlive the call
+        ins, rej = idx.build_enhance_batch(t_iso.data_ptr(), t_ids.data_ptr(), t_dd.data_ptr(), iso.size, kn)
+        stats = orc.enhance_batch(base, st, iso, ids, dd, metric=metric)
+        assert (ins, rej) == (stats[0], stats[1])
+        assert_same_state(idx, st)
+        linked = np.where(st.deg > 0)[0].astype(np.int32)
+        sub = base[linked]
+    assert (st.deg[linked_n:linked_n + 600] > 0).all()
+    idx.close()
+
+
+def oracle_pipeline(orc, base, aux, metric, p):
+    """IndexGPU::BuildGPU composed from the oracle's pieces, in the order coral_build_graph documents."""
+    n = base.shape[0]
+    st = orc.GraphState(n, p.R)
+    for a0 in range(0, aux.shape[0], p.batch):
+        knn, _ = orc.bruteforce(base, aux[a0:a0 + p.batch], p.k_b, metric, order=SEQ)
+        orc.nap_batch(base, st, knn, metric=metric, need_discard=p.need_discard)
+    iso = np.where(st.deg == 0)[0].astype(np.int32)
+    first = int(np.where(st.deg > 0)[0][0]) if p.first_start_id < 0 else p.first_start_id
+    starts = None
+    if p.connect_enhance:
+        for i in range(0, iso.size, p.enhance_search_batch):
+            part = iso[i:i + p.enhance_search_batch]
+            starts = orc.fps(st.nbrs, first, p.n_start)
+            prob = orc.Problem(base, st.nbrs.copy(), starts)
+            ids, dd, _, _ = orc.search_B(prob, base[part], p.k_b, p.enhance_L, metric=metric, start_order=WAVE64,
+                                         nbr_order=WAVE64)
+            for j in range(0, part.size, p.enhance_nap_batch):
+                sl = slice(j, j + p.enhance_nap_batch)
+                orc.enhance_batch(base, st, part[sl], ids[sl], dd[sl], metric=metric)
+    if starts is None:
+        starts = orc.fps(st.nbrs, first, p.n_start)
+    return st, starts, iso.size
+
+
+@pytest.mark.parametrize("metric,ce,seed", [(capi.L2, 1, 0), (capi.IP, 1, 1), (capi.L2, 0, 2)])
+def test_whole_construction_equals_the_oracle_pipeline(orc, metric, ce, seed):
+    n, dim, A = 12000, 48, 900
+    base = base_of(n, dim, 300 + seed, metric)
+    aux = make_queries(A, dim, 400 + seed, "ip" if metric == capi.IP else "l2")
+    p = capi.build_params(R=16, k_b=24, batch=128, connect_enhance=ce, enhance_search_batch=5000,
+                          enhance_nap_batch=700, enhance_L=64, n_start=8)
+    idx = capi.Index(base, None, None, metric=metric)
+    stats = idx.build_graph(aux, p)
+    nbrs, dists, deg, starts = idx.get_graph(with_build_state=True)
+    st, want_starts, iso_n = oracle_pipeline(orc, base, aux, metric, p)
+    assert stats.isolated == iso_n and iso_n > 1000
+    assert stats.batches == (A + p.batch - 1) // p.batch
+    assert np.array_equal(deg, st.deg) and np.array_equal(nbrs, st.nbrs) and dists.tobytes() == st.dists.tobytes()
+    assert starts.tolist() == want_starts.tolist()
+    assert stats.edges == int(st.deg.sum())
+    if ce:
+        assert (deg > 0).all()
+    # the built index answers searches like an index created from the downloaded rows
+    idx.build_end()
+    q = make_queries(50, dim, 77, "ip" if metric == capi.IP else "l2")
+    ids, dd, _ = idx.search(q, 10, 64)
+    idx.close()
+    idx2 = capi.Index(base, nbrs, starts, metric=metric)
+    ids2, dd2, _ = idx2.search(q, 10, 64)
+    idx2.close()
+    assert np.array_equal(ids, ids2) and dd.tobytes() == dd2.tobytes()
+
+
+def test_builder_argument_errors():
+    base = synth.gaussian_matrix(1, 100, 8)
+    idx = capi.Index(base, None, None)
+    knn = dev(np.arange(20, dtype=np.int32).reshape(2, 10))
+    with pytest.raises(capi.CoralError):  # not begun
+        idx.build_nap_batch(knn.data_ptr(), 2, 10)
+    with pytest.raises(capi.CoralError):
+        idx.build_begin(33)
+    idx.build_begin(4)
+    bad = dev(np.array([[1, 2, 100]], np.int32))  # id == n
+    with pytest.raises(capi.CoralError) as e:
+        idx.build_nap_batch(bad.data_ptr(), 1, 3)
+    assert e.value.code == 2
+    with pytest.raises(capi.CoralError):
+        idx.build_nap_batch(knn.data_ptr(), 2, 129)
+    idx.build_nap_batch(knn.data_ptr(), 2, 10)
+    nbrs, dists, deg, _ = idx.get_graph(with_build_state=True)
+    assert (deg[:20] > 0).all() and (deg[20:] == 0).all()
+    idx.build_end()
+    with pytest.raises(capi.CoralError):
+        idx.get_graph(with_build_state=True)
+    idx.close()
