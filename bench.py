@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # and WRITE_SIZE, scaled by what the same counters read for a plain copy kernel);
 # measured offline (profiles/beam_search_kernel_1Mx200_L*.md; FETCH_SIZE reads half the bytes of a
 # 1 GiB copy on this GPU, so its factor is 2.0; WRITE_SIZE's is 1.0).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {256: 1.5798e+11, 512: 3.2649e+11}
+MEASURED_TRAFFIC_BYTES = {256: 1.3825e+11, 512: 2.6955e+11}
 
 
 def algorithmic_bytes(expansions, dist_evals, Q, dim, k, R=32):

@@ -125,8 +125,10 @@ def test_bruteforce_ground_truth_at_full_size(orc):
     sub = np.arange(0, Q, 313)
     oi, od = orc.bruteforce(base, q[sub], k, order=SEQ)
     assert np.array_equal(ids[sub], oi) and dists[sub].tobytes() == od.tobytes()
-    # agrees with the matmul-based ground truth used by the benchmark up to near-ties
-    gt = workloads.ground_truth(base, q[sub], k)
+    # agrees with a matmul-based top-k (|b|^2 - 2 q.b, another arithmetic altogether) up to near-ties
+    tb, tq = torch.from_numpy(base).cuda(), torch.from_numpy(q[sub]).cuda()
+    gt = torch.topk((tb * tb).sum(1)[None, :] - 2.0 * (tq @ tb.T), k, dim=1, largest=False).indices.cpu().numpy()
+    del tb, tq
     agree = np.mean([len(set(a.tolist()) & set(b.tolist())) for a, b in zip(ids[sub], gt)]) / k
     assert agree > 0.999
     # device-pointer entry, and the gt-file layout on disk
