@@ -79,6 +79,9 @@ void IndexGPU::load_config(const std::string& config_file) {
     if (json_number(text, "test_beam_capacity", &v)) pc.test_beam_capacity = (int)v;
     if (json_number(text, "search_start_nodes_num", &v)) pc.search_start_nodes_num = (int)v;
     if (json_number(text, "search_in_cpu", &v)) pc.search_in_cpu = (int)v;
+    if (json_number(text, "need_discard", &v)) pc.need_discard = (int)v;
+    if (json_number(text, "enhance_nap_batch", &v)) pc.enhance_nap_batch = (int)v;
+    if (json_number(text, "enhance_search_batch", &v)) pc.enhance_search_batch = (int)v;
 }
 
 void IndexGPU::LoadSearchNeededData(const char* base_file, const char* sampled_query_file, DIST_METRIC m) {
@@ -141,6 +144,48 @@ void IndexGPU::RunPrepare(Parameters& parameters, Mode mode, size_t n_bp, float*
     if (index_) coral_index_destroy(index_);
     index_ = nullptr;
     if (coral_index_create(&d, &index_)) raise("create index");
+}
+
+void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data, Parameters& parameters) {
+    SetParameters(parameters);
+    load_config(parameters.Get<std::string>("config_file", std::string("default")));
+    const int CE = parameters.Get<int>("CE");
+    if (CE != 0 && CE != 1) throw std::runtime_error("BuildGPU: CE must be 0 or 1 (2, enhancement only, is not provided)");
+    max_degree_ = parameters.Get<int>("max_degree");
+    k_ = parameters.Get<int>("k");
+    metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
+    graph_dir_ = parameters.Get<std::string>("graph_file");
+    if (!bp_data || !sq_data || n_bp == 0 || n_sq == 0) throw std::runtime_error("BuildGPU: empty input");
+    if (bp_data != h_base_) {  // keep a copy, like RunPrepare does with caller-owned vectors
+        std::free(h_base_);
+        h_base_ = nullptr;
+        if (posix_memalign((void**)&h_base_, 32, n_bp * dimension_ * sizeof(float)) != 0)
+            throw std::runtime_error("out of host memory for the base vectors");
+        std::memcpy(h_base_, bp_data, n_bp * dimension_ * sizeof(float));
+    }
+    nd_ = n_bp;
+    coral_index_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.base = h_base_, d.n = (int64_t)nd_, d.dim = (int32_t)dimension_;
+    d.metric = metric_ == DIST_METRIC::L2_ ? CORAL_L2 : CORAL_IP, d.device = 0;
+    if (index_) coral_index_destroy(index_);
+    index_ = nullptr;
+    if (coral_index_create(&d, &index_)) raise("create index");
+    coral_build_params p;
+    coral_build_params_default(&p);
+    p.R = max_degree_, p.k_b = k_, p.batch = PC.batch, p.need_discard = PC.need_discard, p.connect_enhance = CE;
+    p.enhance_search_batch = PC.enhance_search_batch, p.enhance_nap_batch = PC.enhance_nap_batch;
+    p.n_start = PC.search_start_nodes_num;
+    if (coral_build_graph(index_, sq_data, (int64_t)n_sq, &p, &last_build)) raise("BuildGPU");
+    // Graph::save_build (include/graph.cuh:481-484): start ids, then every row with its distances
+    nbrs_.assign(nd_ * (size_t)max_degree_, -1);
+    std::vector<float> dists(nd_ * (size_t)max_degree_);
+    start_ids_.assign((size_t)p.n_start, 0);
+    if (coral_index_get_graph(index_, nbrs_.data(), dists.data(), nullptr, start_ids_.data())) raise("download graph");
+    if (coral_build_end(index_)) raise("BuildGPU");
+    if (coral_graph_dir_write(graph_dir_.c_str(), (int64_t)nd_, max_degree_, nbrs_.data(), dists.data()))
+        raise("save graph");
+    if (coral_start_ids_write(graph_dir_.c_str(), start_ids_.data(), (int32_t)start_ids_.size())) raise("save start ids");
 }
 
 void IndexGPU::LoadRoarGraph(std::string filename) {

@@ -13,8 +13,6 @@
 // and --evaluation_prefix (default ../indexes/ and ../evaluation/),
 // --device_recall 1 (recall through IndexGPU::Search_and_Verify, the loop of
 // the reference's tests/test_update.cpp:196-197, instead of the host count).
-#include <sys/stat.h>
-
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -26,6 +24,7 @@
 #include <string>
 #include <vector>
 
+#include "cli_options.h"
 #include "coral_formats.h"
 #include "efanna2e/index_gpu.h"
 
@@ -33,15 +32,7 @@ using namespace efanna2e;
 
 namespace {
 
-struct Option {
-    const char* name;
-    bool required;
-    bool multitoken;
-    const char* fallback;  // nullptr: no default
-    const char* help;
-};
-
-const Option kOptions[] = {
+const cli::Option kOptions[] = {
     {"data_type", true, false, nullptr, "data type <int8/uint8/float>"},
     {"dist", true, false, nullptr, "distance function <l2/ip>"},
     {"base_data_path", true, false, nullptr, "Input data file in bin format"},
@@ -68,79 +59,6 @@ const Option kOptions[] = {
     {"device_recall", false, false, "0", "1: count hits on the device (IndexGPU::Search_and_Verify)"},
 };
 
-void usage() {
-    std::cout << "Arguments:\n  -h [ --help ]  Print information on arguments\n";
-    for (const Option& o : kOptions)
-        std::cout << "  --" << o.name << (o.fallback ? std::string(" arg (=") + o.fallback + ")" : " arg") << "  "
-                  << o.help << "\n";
-}
-
-const Option* find_option(const std::string& name) {
-    for (const Option& o : kOptions)
-        if (name == o.name) return &o;
-    return nullptr;
-}
-
-// returns false (after printing what is wrong) on a malformed command line
-bool parse(int argc, char** argv, std::map<std::string, std::vector<std::string>>& out, bool* help) {
-    *help = false;
-    for (int i = 1; i < argc; ++i) {
-        std::string a = argv[i];
-        if (a == "-h" || a == "--help") {
-            *help = true;
-            return true;
-        }
-        std::string name, value;
-        bool has_value = false;
-        if (a == "-T") {
-            name = "num_threads";
-        } else if (a.rfind("--", 0) == 0) {
-            const size_t eq = a.find('=');
-            name = a.substr(2, eq == std::string::npos ? std::string::npos : eq - 2);
-            if (eq != std::string::npos) value = a.substr(eq + 1), has_value = true;
-        } else {
-            std::cerr << "too many positional options have been specified on the command line\n";
-            return false;
-        }
-        const Option* o = find_option(name);
-        if (!o) {
-            std::cerr << "unrecognised option '" << a << "'\n";
-            return false;
-        }
-        std::vector<std::string>& vals = out[name];
-        if (has_value) {
-            vals.push_back(value);
-        } else if (o->multitoken) {
-            while (i + 1 < argc && !(argv[i + 1][0] == '-' && !std::isdigit((unsigned char)argv[i + 1][1])))
-                vals.push_back(argv[++i]);
-            if (vals.empty()) {
-                std::cerr << "the required argument for option '--" << name << "' is missing\n";
-                return false;
-            }
-        } else {
-            if (i + 1 >= argc) {
-                std::cerr << "the required argument for option '--" << name << "' is missing\n";
-                return false;
-            }
-            vals.assign(1, argv[++i]);
-        }
-    }
-    for (const Option& o : kOptions) {
-        if (out.count(o.name)) continue;
-        if (o.required) {
-            std::cerr << "the option '--" << o.name << "' is required but missing\n";
-            return false;
-        }
-        if (o.fallback) out[o.name].assign(1, o.fallback);
-    }
-    return true;
-}
-
-void make_dirs(const std::string& path) {
-    for (size_t p = 1; p <= path.size(); ++p)
-        if (p == path.size() || path[p] == '/') mkdir(path.substr(0, p).c_str(), 0755);
-}
-
 // tests/test_search_pipeline.cpp:25-39
 float ComputeRecall(int q_num, int k, int gt_dim, int* res, int* gt) {
     return (float)coral_recall_hits(q_num, k, gt_dim, res, gt) / (float)((size_t)k * q_num);
@@ -151,9 +69,10 @@ float ComputeRecall(int q_num, int k, int gt_dim, int* res, int* gt) {
 int main(int argc, char** argv) {
     std::map<std::string, std::vector<std::string>> opt;
     bool help = false;
-    if (!parse(argc, argv, opt, &help)) return -1;
+    const size_t n_options = sizeof kOptions / sizeof kOptions[0];
+    if (!cli::parse(kOptions, n_options, argc, argv, opt, &help)) return -1;
     if (help) {
-        usage();
+        cli::usage(kOptions, n_options);
         return 0;
     }
     auto str = [&](const char* n) { return opt[n].empty() ? std::string() : opt[n][0]; };
@@ -252,7 +171,7 @@ int main(int argc, char** argv) {
 
         std::cout << "k: " << k << std::endl;
         std::vector<int> res((size_t)q_pts * k, 0);
-        make_dirs(eval_dir);
+        cli::make_dirs(eval_dir);
         std::ofstream evaluation_out(evaluation_save_file, std::ios::out);
         if (!evaluation_out.is_open()) {
             std::cout << "Unable to open evaluation file: " << evaluation_save_file << std::endl;

@@ -33,7 +33,7 @@ enum Metric { L2 = 0, INNER_PRODUCT = 1, FAST_L2 = 2, PQ = 3, COSINE = 4 };  // 
 enum Mode { CONS, SEARCH, UPD, CE };                                          // include/uni.h:147
 enum GraphType { GPU, CPU, DISK };                                            // include/uni.h:149
 
-// The keys of config.json that search reads (src/index_gpu.cpp:40-87); defaults
+// The keys of config.json that search and construction read (src/index_gpu.cpp:40-87); defaults
 // are the reference's (include/uni.h:97-132).
 struct ProConfig {
     int dim = 200;
@@ -44,6 +44,10 @@ struct ProConfig {
     int test_beam_capacity = 512;
     int search_start_nodes_num = 16;
     int search_in_cpu = 0;
+    // read by the builder
+    int need_discard = 1;
+    int enhance_nap_batch = 4096;
+    int enhance_search_batch = 524288;
 };
 CORAL_API ProConfig& GetProConfig();
 #define PC (::efanna2e::GetProConfig())
@@ -97,6 +101,13 @@ class CORAL_API IndexGPU {
     Test_Result Search_and_Verify(const float* queries, const int* gts, int num, int beam_capacity = 0);
     // src/graph.cu:709-743
     void LoadRoarGraph(std::string filename);
+    // src/index_gpu.cpp:308-383: builds the graph over the n_bp base vectors from the n_sq auxiliary ("sampled")
+    // queries and writes the index directory parameters["graph_file"] (graph.part*.idx/.data, graph.search_start_ids,
+    // graph.batch_id).  Reads config_file, CE (0 or 1; 2, "only CE", is not provided), max_degree, k (the cluster
+    // size), dist, graph_file.  Both arrays hold rows of GetDimension() floats.  The built index stays loaded, so
+    // Search works right after.  The timings and counts of the run are in last_build.
+    void BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data, Parameters& parameters);
+    coral_build_stats last_build{};
     // src/index_gpu.cpp:138-206 with upd_type 0: the ids are tombstoned on the device (del_node_mark,
     // src/update.cu:660-672) and later searches leave them out of their results; the graph is not repaired
     void Delete(const std::vector<int> del_ids);

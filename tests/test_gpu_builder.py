@@ -167,3 +167,60 @@ def test_builder_argument_errors():
     with pytest.raises(capi.CoralError):
         idx.get_graph(with_build_state=True)
     idx.close()
+
+
+def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tmp_path):
+    """test_build_pipeline -> graph.part0.idx/.data + graph.search_start_ids -> test_search_pipeline."""
+    import os
+    import subprocess
+    from coral_amd import formats
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    n, dim, A, Q, k = 15000, 48, 1100, 100, 10
+    base = base_of(n, dim, 500, capi.L2)
+    aux = make_queries(A, dim, 600)
+    q = make_queries(Q, dim, 700)
+    work = tmp_path / "run"
+    os.makedirs(work / "cwd")
+    formats.fbin_write(work / "base.fbin", base)
+    formats.fbin_write(work / "aux.fbin", aux)
+    formats.fbin_write(work / "query.fbin", q)
+    gt, _ = orc.bruteforce(base, q, k)
+    formats.gt_write(work / "gt.bin", gt)
+    (work / "config.json").write_text('{"batch": 256, "enhance_nap_batch": 1000, "search_start_nodes_num": 8}')
+    cli = os.path.join(root, "coral_amd", "lib", "test_build_pipeline")
+    args = [cli, "--data_type", "float", "--dist", "l2", "--dataset", "syn", "--base_data_path", str(work / "base.fbin"),
+            "--sampled_query_data_path", str(work / "aux.fbin"), "--M_pjbp", "16", "--k", "24", "--CE", "1",
+            "--query_thres", "1.0", "--config_file", str(work / "config.json"), "-T", "8"]
+    r = subprocess.run(args, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr + r.stdout
+    index_dir = work / "indexes" / "syn_l2_16_1.0_1"  # ../indexes/<dataset>_<dist>_<R>_<thres>_<CE>
+    assert "Save index to ../indexes/syn_l2_16_1.0_1" in r.stdout
+    nbrs, dists = formats.graph_dir_read(index_dir, n, 16, want_dists=True)
+    starts = formats.start_ids_read(index_dir)
+    # the same construction through the C ABI
+    p = capi.build_params(R=16, k_b=24, batch=256, enhance_nap_batch=1000, n_start=8)
+    idx = capi.Index(base, None, None)
+    idx.build_graph(aux, p)
+    want_nbrs, want_dists, deg, want_starts = idx.get_graph(with_build_state=True)
+    idx.close()
+    assert np.array_equal(nbrs, want_nbrs) and dists.tobytes() == want_dists.tobytes()
+    assert starts.tolist() == want_starts.tolist() and len(starts) == 8
+    assert (deg > 0).all()
+    # and the search driver on that directory
+    cli = os.path.join(root, "coral_amd", "lib", "test_search_pipeline")
+    args = [cli, "--data_type", "float", "--dist", "l2", "--base_data_path", str(work / "base.fbin"), "--dataset",
+            "syn", "--query_path", str(work / "query.fbin"), "--gt_path", str(work / "gt.bin"), "--k", str(k),
+            "--max_degree", "16", "--L", "64", "--config_file", str(work / "config.json")]
+    r = subprocess.run(args, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    row = [l for l in r.stdout.splitlines() if l.startswith("64\t")][0].split()
+    oi, _, _, _ = orc.search_B(orc.Problem(base, nbrs, starts), q, k, 64, start_order=WAVE64, nbr_order=WAVE64)
+    assert abs(float(row[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
+    # refused: precomputed clusters, unknown metric
+    r = subprocess.run(args[:1] + ["--help"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0
+    bad = [os.path.join(root, "coral_amd", "lib", "test_build_pipeline"), "--data_type", "float", "--dist", "l2",
+           "--dataset", "syn", "--base_data_path", str(work / "base.fbin"), "--sampled_query_data_path",
+           str(work / "aux.fbin"), "--train_gt_file", "x.bin"]
+    r = subprocess.run(bad, cwd=work / "cwd", capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "train_gt_file" in r.stderr
