@@ -50,34 +50,50 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// one lane walks both rows: the accumulation order of include/utils.cuh:254-275 (L2) and :307-323 (IP)
+// one lane walks both rows: the accumulation order of include/utils.cuh:254-275 (L2) and :307-323 (IP).  The rows
+// are fetched eight float4 at a time ahead of the additions, so a lane waits for memory once per 32 dimensions
+// instead of once per 4; the chain of additions itself stays strictly in dimension order.
 __device__ __forceinline__ float seq_dist(const float* __restrict__ a, const float* __restrict__ b, int dim, int metric) {
+    constexpr int kAhead = 8;
     const float4* a4 = reinterpret_cast<const float4*>(a);
     const float4* b4 = reinterpret_cast<const float4*>(b);
+    const int n4 = dim / 4;
     float acc = 0.0f;
-    if (metric == CORAL_L2) {
-        for (int i = 0; i < dim / 4; ++i) {
-            const float4 x = a4[i], y = b4[i];
-            float t = x.x - y.x;
-            acc = fmaf(t, t, acc);
-            t = x.y - y.y;
-            acc = fmaf(t, t, acc);
-            t = x.z - y.z;
-            acc = fmaf(t, t, acc);
-            t = x.w - y.w;
-            acc = fmaf(t, t, acc);
+    for (int i0 = 0; i0 < n4; i0 += kAhead) {
+        float4 x[kAhead], y[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int i = i0 + u < n4 ? i0 + u : n4 - 1;
+            x[u] = a4[i];
+            y[u] = b4[i];
         }
-    } else {
-        for (int i = 0; i < dim / 4; ++i) {
-            const float4 x = a4[i], y = b4[i];
-            acc = fmaf(x.x, y.x, acc);
-            acc = fmaf(x.y, y.y, acc);
-            acc = fmaf(x.z, y.z, acc);
-            acc = fmaf(x.w, y.w, acc);
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            if (i0 + u < n4) {
+                if (metric == CORAL_L2) {
+                    float t = x[u].x - y[u].x;
+                    acc = fmaf(t, t, acc);
+                    t = x[u].y - y[u].y;
+                    acc = fmaf(t, t, acc);
+                    t = x[u].z - y[u].z;
+                    acc = fmaf(t, t, acc);
+                    t = x[u].w - y[u].w;
+                    acc = fmaf(t, t, acc);
+                } else {
+                    acc = fmaf(x[u].x, y[u].x, acc);
+                    acc = fmaf(x[u].y, y[u].y, acc);
+                    acc = fmaf(x[u].z, y[u].z, acc);
+                    acc = fmaf(x[u].w, y[u].w, acc);
+                }
+            }
         }
     }
     return acc;
 }
+
+// Member-pair distances are kept once per unordered pair: entry (r, q), r < q, of a kb x kb matrix.
+__device__ __forceinline__ int tri_index(int r, int q, int kb) { return r * (2 * kb - r - 1) / 2 + (q - r - 1); }
+__device__ __forceinline__ int pair_index(int a, int b, int kb) { return a < b ? tri_index(a, b, kb) : tri_index(b, a, kb); }
 
 // The candidate list of one pivot, private to one wavefront.
 struct WaveCands {
@@ -89,6 +105,12 @@ struct WaveCands {
     int16_t col[kMaxCand];
     uint8_t st[kMaxCand];
 };
+
+// bytes of the region that holds the staging rows first and the candidate lists afterwards
+__host__ __device__ inline size_t nap_union_bytes(int kb) {
+    const size_t a = (size_t)kb * (kChunk + 4) * sizeof(float), b = sizeof(WaveCands) * kWaves;
+    return ((a > b ? a : b) + 15) & ~(size_t)15;
+}
 
 __device__ __forceinline__ unsigned long long cand_key(float dist, int col, int metric) {
     const uint32_t o = ord32(dist);
@@ -119,10 +141,10 @@ __device__ int sort_cands(WaveCands& S, int C, int lane) {
 
 // candidate_ignore_kernel (src/upd_gpu.cu:203-247, src/enhance.cu:334-380): in order of distance a candidate not yet
 // ruled out is retained and rules out every later one that is closer to it than to the pivot; duplicates of an id
-// are marked.  Stops once R are retained.  G (optional) holds the member-pair distances, indexed by column.
+// are marked.  Stops once R are retained.  G (optional) holds the member-pair distances by pair of columns.
 template <bool HAVE_G>
 __device__ void prune_cands(WaveCands& S, int m, int lane, const float* __restrict__ vec, int dim, int metric, int R,
-                            const float* G, int ldg, int kb) {
+                            const float* G, int kb) {
     int nbr_num = 0;
     for (int i = 0; i < m && nbr_num < R; ++i) {
         const uint8_t st = S.st[i];
@@ -139,7 +161,7 @@ __device__ void prune_cands(WaveCands& S, int m, int lane, const float* __restri
                     const int colj = S.col[j];
                     float d;
                     if (HAVE_G && coli < kb && colj < kb)
-                        d = G[coli * ldg + colj];
+                        d = G[pair_index(coli, colj, kb)];
                     else
                         d = seq_dist(vi, vec + (size_t)idj * dim, dim, metric);
                     if (closer(S.dist[j], d, metric)) S.st[j] = ST_DISCARDED;
@@ -190,21 +212,22 @@ __global__ void claim_kernel(const int32_t* __restrict__ ids, int64_t count, int
         atomicMin(owner + ids[p], (int32_t)p);
 }
 
-// one workgroup per cluster; dynamic LDS: G[kb][kb+1] | stage[kb][kChunk+4] | ids[kb] | deg[kb] | WaveCands[kWaves]
+// one workgroup per cluster; dynamic LDS: G[kb(kb-1)/2] | stage[kb][kChunk+4] or WaveCands[kWaves] | ids[kb] | deg[kb]
+// (the staging rows of the distance phase and the candidate lists of the pivot phase are never live together)
 __global__ void __launch_bounds__(kThreads)
 nap_cluster_kernel(const float* __restrict__ vec, int dim, int metric, int R, const int32_t* __restrict__ nbrs,
                    const float* __restrict__ dists, const int32_t* __restrict__ deg, const int32_t* __restrict__ owner,
                    const int32_t* __restrict__ knn, int batch, int kb, int need_discard, int32_t* __restrict__ new_ids,
                    float* __restrict__ new_dists, int32_t* __restrict__ new_deg) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int ldg = kb + 1, lds = kChunk + 4;  // stage rows stay 16-byte aligned
+    const int lds = kChunk + 4;  // stage rows stay 16-byte aligned
+    const int npairs = kb * (kb - 1) / 2;
     float* G = reinterpret_cast<float*>(smem);
-    float* stage = G + ((kb * ldg + 3) & ~3);
-    int32_t* s_ids = reinterpret_cast<int32_t*>(stage + kb * lds);
+    float* stage = G + ((npairs + 3) & ~3);
+    WaveCands* cands = reinterpret_cast<WaveCands*>(stage);
+    const size_t shared_bytes = nap_union_bytes(kb);
+    int32_t* s_ids = reinterpret_cast<int32_t*>(reinterpret_cast<unsigned char*>(stage) + shared_bytes);
     int32_t* s_deg = s_ids + kb;
-    size_t off = (size_t)(reinterpret_cast<unsigned char*>(s_deg + kb) - smem);
-    off = (off + 15) & ~(size_t)15;
-    WaveCands* cands = reinterpret_cast<WaveCands*>(smem + off);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int C = kb + R;
 
@@ -215,8 +238,9 @@ nap_cluster_kernel(const float* __restrict__ vec, int dim, int metric, int R, co
             s_ids[r] = id;
             s_deg[r] = deg[id];
         }
-        // member-pair distances: entry t of the kb x kb matrix belongs to thread t % kThreads; between two chunks of
-        // dimensions the running sum of an entry waits in G, so the chain of additions is the sequential one
+        // member-pair distances, pair t of the folded enumeration to thread t % kThreads; between two chunks of
+        // dimensions the running sum of a pair waits in G, so the chain of additions is the sequential one
+        const int half = (kb + 1) / 2, rowlen = kb - 1;
         for (int d0 = 0; d0 < dim; d0 += kChunk) {
             const int cw = dim - d0 < kChunk ? dim - d0 : kChunk;
             __syncthreads();
@@ -225,11 +249,19 @@ nap_cluster_kernel(const float* __restrict__ vec, int dim, int metric, int R, co
                 stage[r * lds + c] = vec[(size_t)s_ids[r] * dim + d0 + c];
             }
             __syncthreads();
-            for (int t = tid; t < kb * kb; t += kThreads) {
-                const int r = t / kb, q = t - r * kb;
+            for (int t = tid; t < half * rowlen; t += kThreads) {
+                // folded enumeration of the pairs r < q: row fr and row kb-1-fr together hold kb-1 of them
+                const int fr = t / rowlen, c = t - fr * rowlen;
+                int r = fr, q = fr + 1 + c;
+                if (c >= rowlen - fr) {
+                    r = kb - 1 - fr;
+                    q = r + 1 + (c - (rowlen - fr));
+                    if (r == fr) continue;  // odd kb: the middle row is its own partner
+                }
+                const int g = tri_index(r, q, kb);
                 const float4* a = reinterpret_cast<const float4*>(stage + r * lds);
                 const float4* bq = reinterpret_cast<const float4*>(stage + q * lds);
-                float x = d0 ? G[r * ldg + q] : 0.0f;
+                float x = d0 ? G[g] : 0.0f;
                 if (metric == CORAL_L2) {
                     for (int c = 0; c < cw / 4; ++c) {
                         const float4 u = a[c], w = bq[c];
@@ -251,18 +283,27 @@ nap_cluster_kernel(const float* __restrict__ vec, int dim, int metric, int R, co
                         x = fmaf(u.w, w.w, x);
                     }
                 }
-                G[r * ldg + q] = x;
+                G[g] = x;
             }
         }
         __syncthreads();
 
         // pivots of the cluster, one wavefront each
+        int n_new = 0;  // members still without neighbours
+        for (int r0 = 0; r0 < kb; r0 += 64) n_new += __popcll(__ballot(r0 + lane < kb && s_deg[r0 + lane] == 0));
         WaveCands& S = cands[wave];
         for (int r = wave; r < kb; r += kWaves) {
             const int64_t p = (int64_t)b * kb + r;
             const int32_t pid = s_ids[r];
             if (owner[pid] != (int32_t)p) continue;  // uniform in the wavefront
             const int rdeg = s_deg[r];
+            if (rdeg > 0 && n_new == 0 && need_discard) {
+                // no member is new, so the candidates are the pivot's own row (at most R entries, sorted, no
+                // duplicates): whatever the occlusion rule retains, the fill puts the rest back in the same order.
+                // The row comes out as it went in: nothing to compute, nothing to write.
+                if (lane == 0) new_deg[p] = -1;
+                continue;
+            }
             for (int q = lane; q < C; q += 64) {
                 unsigned long long key = ~0ull;
                 int32_t id = -1;
@@ -271,7 +312,7 @@ nap_cluster_kernel(const float* __restrict__ vec, int dim, int metric, int R, co
                     // src/upd_gpu.cu:45-73: not itself, and one of the two must still be without neighbours
                     if (q != r && s_ids[q] != pid && !(rdeg > 0 && s_deg[q] > 0)) {
                         id = s_ids[q];
-                        d = G[r * ldg + q];
+                        d = G[pair_index(r, q, kb)];
                         key = cand_key(d, q, metric);
                     }
                 } else if (q - kb < rdeg) {  // src/upd_gpu.cu:48-52: the current row
@@ -284,7 +325,7 @@ nap_cluster_kernel(const float* __restrict__ vec, int dim, int metric, int R, co
                 S.udist[q] = d;
             }
             const int m = sort_cands(S, C, lane);
-            prune_cands<true>(S, m, lane, vec, dim, metric, R, G, ldg, kb);
+            prune_cands<true>(S, m, lane, vec, dim, metric, R, G, kb);
             const int nd = emit_row(S, m, lane, R, need_discard != 0, new_ids + (size_t)p * R, new_dists + (size_t)p * R);
             if (lane == 0) new_deg[p] = nd;
             wave_sync();
@@ -304,13 +345,13 @@ __global__ void nap_commit_kernel(const int32_t* __restrict__ knn, int64_t count
     const int32_t id = knn[p];
     if (owner[id] != (int32_t)p) return;
     const int nd = new_deg[p];
-    if (l < R) {
+    if (nd >= 0 && l < R) {
         nbrs[(size_t)id * R + l] = l < nd ? new_ids[(size_t)p * R + l] : -1;
         dists[(size_t)id * R + l] = l < nd ? new_dists[(size_t)p * R + l] : 0.0f;
     }
     __builtin_amdgcn_wave_barrier();
     if (l == 0) {
-        deg[id] = nd;
+        if (nd >= 0) deg[id] = nd;  // negative: the row stays as it is
         owner[id] = INT_MAX;
     }
 }
@@ -427,7 +468,7 @@ enh_rows_kernel(const float* __restrict__ vec, int dim, int metric, int R, int32
             S.udist[q] = d;
         }
         const int m = sort_cands(S, kn, lane);
-        prune_cands<false>(S, m, lane, vec, dim, metric, R, nullptr, 0, 0);
+        prune_cands<false>(S, m, lane, vec, dim, metric, R, nullptr, 0);
         int32_t* row = nbrs + (size_t)iso * R;
         float* rowd = dists + (size_t)iso * R;
         const int nd = emit_row(S, m, lane, R, true, row, rowd);
@@ -458,9 +499,8 @@ __global__ void gather_rows_kernel(const float* __restrict__ vec, int dim, const
 }  // namespace
 
 size_t nap_lds_bytes(int kb) {
-    size_t off = (((size_t)kb * (kb + 1) * 4 + 15) & ~(size_t)15) + (size_t)kb * (kChunk + 4) * 4 + (size_t)kb * 8;
-    off = (off + 15) & ~(size_t)15;
-    return off + sizeof(WaveCands) * kWaves;
+    const size_t g = ((size_t)(kb * (kb - 1) / 2 + 3) & ~(size_t)3) * sizeof(float);
+    return g + nap_union_bytes(kb) + (size_t)kb * 8;
 }
 
 hipError_t launch_nap_batch(const float* vec, int dim, int metric, int R, int32_t* nbrs, float* dists, int32_t* deg,

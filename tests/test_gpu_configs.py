@@ -2,8 +2,9 @@
 config 1 (100k x 128, exact 32-NN graph, k=10, L=64: the reference's CPU-runnable case),
 config 3 (inner product, 1M x 512, k=100, L=256), config 4 (10M x 200, batch sweep) and
 config 5 (100M x 200 with 10 % tombstones; skipped where memory is short).
-Graphs of configs 4 and 5 are cheap block graphs (coral_amd.synth.block_graph): these cases
-check parity and size handling, not recall."""
+Configs 2-4 search graphs made by the library's own builder from 100 000 auxiliary queries; config 5 uses a
+cheap block graph (coral_amd.synth.block_graph; building for 100M nodes would take several minutes): it checks
+parity and size handling, not recall."""
 import os
 import time
 
@@ -86,13 +87,19 @@ def test_config3_inner_product_1m_x_512(orc):
     idx.close()
 
 
-def big_case(orc, n, dim, Qs, L, k, tomb_seed=None):
+def big_case(orc, n, dim, Qs, L, k, tomb_seed=None, built=False):
     t0 = time.time()
     base = workloads.gaussian_base(4001 if n <= 10 ** 7 else 5001, n, dim)
     print("generated %d x %d in %.0f s" % (n, dim, time.time() - t0), flush=True)
-    nbrs = synth.block_graph(base, 32)
-    print("block graph at %.0f s" % (time.time() - t0), flush=True)
-    starts = (np.arange(16, dtype=np.int64) * (n // 16) + 5).astype(np.int32)
+    if built:
+        aux = synth.shifted_queries(100000, dim, 2002, 2003, 2005)
+        nbrs, starts, info = workloads.build_query_aware_graph(base, aux, "l2")
+        assert (nbrs[:, 0] >= 0).all()  # the enhancement left no node without neighbours
+        print("built graph at %.0f s: %s" % (time.time() - t0, info), flush=True)
+    else:
+        nbrs = synth.block_graph(base, 32)
+        print("block graph at %.0f s" % (time.time() - t0), flush=True)
+        starts = (np.arange(16, dtype=np.int64) * (n // 16) + 5).astype(np.int32)
     q = synth.shifted_queries(max(Qs), dim, 2002, 2003, 2004)
     idx = capi.Index(base, nbrs, starts)
     mask = None
@@ -125,7 +132,7 @@ def big_case(orc, n, dim, Qs, L, k, tomb_seed=None):
 
 
 def test_config4_10m_batch_sweep(orc):
-    big_case(orc, 10 ** 7, 200, (1000, 10000, 100000), 256, 100)
+    big_case(orc, 10 ** 7, 200, (1000, 10000, 100000), 256, 100, built=True)
 
 
 def _mem_available_gib():
