@@ -224,6 +224,12 @@ def enhance_batch(base, state, iso_ids, knn_ids, knn_dists, metric=L2):
     return stats
 
 
+def max_threads():
+    fn = lib().oracle_max_threads
+    fn.restype, fn.argtypes = C.c_int, []
+    return int(fn())
+
+
 def recall_hits(res, gt, k):
     res, gt = _i32(res), _i32(gt)
     return int(lib().oracle_recall_hits(res.shape[0], k, gt.shape[1], _p(res), _p(gt)))

@@ -107,3 +107,47 @@ def test_cli_flag_handling():
     assert r.returncode == 1 and "open file error" in r.stderr
     r = run_cli(*base, "--dist=l2", "--k", "ten")
     assert r.returncode == 255
+
+
+def test_build_cli_flag_handling():
+    cli = os.path.join(ROOT, "coral_amd", "lib", "test_build_pipeline")
+
+    def run(*args):
+        return subprocess.run([cli] + list(args), capture_output=True, text=True)
+
+    r = run("--help")
+    assert r.returncode == 0
+    for flag in ("--data_type", "--dist", "--N", "--dataset", "--base_data_path", "--train_gt_file",
+                 "--sampled_query_data_path", "--query_test_file", "--gt_test_file", "--M_sq", "--M_pjbp", "--L_pjpq",
+                 "--num_threads", "--CE", "--k", "--iso_thres", "--recall_thres", "--query_thres", "--log_file",
+                 "--config_file"):  # tests/test_build_pipeline.cpp:45-121
+        assert flag in r.stdout
+    r = run("--dist", "l2")
+    assert r.returncode == 255 and "required but missing" in r.stderr
+    base = ["--data_type", "float", "--dataset", "t", "--base_data_path", "/nonexistent.fbin",
+            "--sampled_query_data_path", "/nonexistent_sq.fbin", "--k", "100", "-T", "32", "--index_dir", "/tmp/x"]
+    r = run(*base, "--dist", "cosine")
+    assert r.returncode == 255 and "Unknown distance type" in r.stdout
+    r = run(*base, "--dist", "l2")
+    assert r.returncode == 1 and "open file error" in r.stderr
+    r = run(*base, "--dist", "l2", "--train_gt_file", "clusters.bin")
+    assert r.returncode == 255 and "train_gt_file" in r.stderr
+    r = run(*base, "--dist", "l2", "--CE", "x")
+    assert r.returncode == 255
+
+
+def test_build_entry_points_reject_bad_arguments_before_any_device_call():
+    lib = capi.lib()
+    assert lib.coral_build_begin(None, 32) == capi.ERR_ARG
+    assert lib.coral_build_nap_batch(None, None, 1, 10, 1) == capi.ERR_ARG
+    assert lib.coral_build_enhance_batch(None, None, None, None, 1, 10, None, None) == capi.ERR_ARG
+    assert lib.coral_build_connect_enhance(None, None, None) == capi.ERR_ARG
+    assert lib.coral_build_graph(None, None, 0, None, None) == capi.ERR_ARG
+    assert lib.coral_index_get_graph(None, None, None, None, None) == capi.ERR_ARG
+    assert lib.coral_start_ids_fps(None, 0, 1, None) == capi.ERR_ARG
+    assert lib.coral_index_mark_deleted(None, None, 0) == capi.ERR_ARG
+    p = capi.build_params()
+    assert (p.R, p.k_b, p.batch, p.need_discard, p.connect_enhance) == (32, 100, 1024, 1, 1)  # config.json:3-6,14
+    assert (p.enhance_search_batch, p.enhance_nap_batch, p.enhance_L, p.n_start) == (524288, 4096, 256, 16)
+    with pytest.raises(TypeError):
+        capi.build_params(no_such_field=1)

@@ -226,3 +226,62 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
            str(work / "aux.fbin"), "--train_gt_file", "x.bin"]
     r = subprocess.run(bad, cwd=work / "cwd", capture_output=True, text=True, timeout=60)
     assert r.returncode != 0 and "train_gt_file" in r.stderr
+
+
+def test_batch_update_and_enhancement_at_the_real_shape(orc):
+    """1M x 200, clusters of 100, rows of 32: single steps of a running construction against the oracle applied
+    to the state the device held before the step (the whole construction at this size is too slow for the CPU)."""
+    import time
+    import torch
+    from coral_amd import workloads
+    n, dim, kb, R, batch = 1000000, 200, 100, 32, 1024
+    base = workloads.gaussian_base(2001, n, dim)
+    aux = synth.shifted_queries(12 * batch, dim, 2002, 2003, 2005)
+    idx = capi.Index(base, None, None)
+    d_aux = torch.from_numpy(aux).cuda()
+    d_knn = torch.empty((aux.shape[0], kb), dtype=torch.int32, device="cuda")
+    idx.bruteforce_device(d_aux.data_ptr(), d_knn.data_ptr(), None, aux.shape[0], kb)
+    knn = d_knn.cpu().numpy()
+    idx.build_begin(R)
+
+    def state():
+        st = orc.GraphState(0, R)
+        st.nbrs, st.dists, st.deg, _ = idx.get_graph(with_build_state=True)
+        return st
+
+    for b in range(12):
+        check = b in (0, 6, 11)
+        if check:
+            st = state()
+        t0 = time.perf_counter()
+        idx.build_nap_batch(d_knn[b * batch:].data_ptr(), batch, kb, True)
+        t_gpu = time.perf_counter() - t0
+        if check:
+            t0 = time.perf_counter()
+            stats = orc.nap_batch(base, st, knn[b * batch:(b + 1) * batch])
+            print("batch %d: device %.1f ms (call), oracle on %d host threads %.0f ms; %d pivots written, %d distance "
+                  "evaluations of the occlusion rule" % (b, 1e3 * t_gpu, orc.max_threads(), 1e3 * (time.perf_counter() - t0),
+                                                         stats[0], stats[1]), flush=True)
+            assert stats[0] > 50000
+            assert_same_state(idx, st)
+    # one enhancement batch: entry points, the search for 4096 isolated nodes' own vectors, the batch itself
+    st = state()
+    assert ((st.nbrs >= 0).sum(1) == st.deg).all()
+    first = int(np.where(st.deg > 0)[0][0])
+    starts = idx.start_ids_fps(first, 16)
+    assert starts.tolist() == orc.fps(st.nbrs, first, 16).tolist()
+    idx.set_graph(st.nbrs, starts)
+    iso = np.where(st.deg == 0)[0][:4096].astype(np.int32)
+    ids, dd, _ = idx.search(base[iso], kb, 256)
+    assert (ids >= 0).all() and not np.isin(ids, iso).any()
+    t_iso, t_ids, t_dd = dev(iso), dev(ids), dev(dd)
+    t0 = time.perf_counter()
+    ins, rej = idx.build_enhance_batch(t_iso.data_ptr(), t_ids.data_ptr(), t_dd.data_ptr(), iso.size, kb)
+    t_gpu = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    stats = orc.enhance_batch(base, st, iso, ids, dd)
+    print("enhancement batch of %d: device %.1f ms (call), oracle on one host thread %.0f ms; %d reverse edges" %
+          (iso.size, 1e3 * t_gpu, 1e3 * (time.perf_counter() - t0), ins), flush=True)
+    assert (ins, rej) == (stats[0], stats[1]) and ins > 10000
+    assert_same_state(idx, st)
+    idx.close()
