@@ -101,6 +101,7 @@ SIGNATURES = {
                                             C.c_void_p, C.c_void_p]),
     "coral_build_connect_enhance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_build_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
+    "coral_build_graph_from_clusters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "coral_index_get_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_start_ids_fps": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
@@ -267,6 +268,16 @@ class Index:
         aux = np.ascontiguousarray(aux, dtype=np.float32)
         st = BuildStats()
         _check(lib().coral_build_graph(self._h, _ptr(aux), aux.shape[0], C.byref(params), C.byref(st)))
+        self.R, self.n_start = params.R, params.n_start
+        return st
+
+    def build_graph_from_clusters(self, clusters, params):
+        """The construction from precomputed clusters, int32 [A][k_b] (the reference's --train_gt_file)."""
+        c = np.ascontiguousarray(clusters, dtype=np.int32)
+        if c.ndim != 2 or c.shape[1] != params.k_b:
+            raise ValueError("clusters must be [A][k_b]")
+        st = BuildStats()
+        _check(lib().coral_build_graph_from_clusters(self._h, _ptr(c), c.shape[0], C.byref(params), C.byref(st)))
         self.R, self.n_start = params.R, params.n_start
         return st
 

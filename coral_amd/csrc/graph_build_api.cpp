@@ -235,9 +235,10 @@ int coral_build_connect_enhance(coral_index* idx, const coral_build_params* prm,
     return rc;
 }
 
-int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const coral_build_params* prm,
-                      coral_build_stats* stats) {
-    if (!idx || !h_aux || !prm) return fail(CORAL_ERR_ARG, "null argument");
+// the construction from auxiliary queries (h_aux) or from their precomputed clusters (h_clusters)
+static int build_impl(coral_index* idx, const float* h_aux, const int32_t* h_clusters, int64_t A,
+                      const coral_build_params* prm, coral_build_stats* stats) {
+    if (!idx || (!h_aux && !h_clusters) || !prm) return fail(CORAL_ERR_ARG, "null argument");
     if (A <= 0) return fail(CORAL_ERR_ARG, "no auxiliary queries");
     if (prm->batch <= 0) return fail(CORAL_ERR_ARG, "batch must be positive");
     if (prm->k_b > idx->n) return fail(CORAL_ERR_ARG, "k_b exceeds the number of base vectors");
@@ -253,18 +254,27 @@ int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const cor
     float* d_aux = nullptr;
     int32_t* d_knn = nullptr;
     int rc = CORAL_OK;
-    if (hipMalloc(&d_aux, (size_t)chunk * dim * sizeof(float)) != hipSuccess ||
+    if ((h_aux && hipMalloc(&d_aux, (size_t)chunk * dim * sizeof(float)) != hipSuccess) ||
         hipMalloc(&d_knn, (size_t)chunk * kb * sizeof(int32_t)) != hipSuccess)
         rc = fail(CORAL_ERR_MEMORY, "device allocation for the auxiliary queries failed");
     for (int64_t a0 = 0; rc == CORAL_OK && a0 < A; a0 += chunk) {
         const int64_t cq = std::min(chunk, A - a0);
-        if (hipMemcpy(d_aux, h_aux + (size_t)a0 * dim, (size_t)cq * dim * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
-            rc = fail(CORAL_ERR_DEVICE, "upload of auxiliary queries failed");
-            break;
+        if (h_clusters) {  // GraphTask's train_gt_file branch, src/index_gpu.cpp:505-524
+            if (hipMemcpy(d_knn, h_clusters + (size_t)a0 * kb, (size_t)cq * kb * sizeof(int32_t), hipMemcpyHostToDevice) !=
+                hipSuccess) {
+                rc = fail(CORAL_ERR_DEVICE, "upload of clusters failed");
+                break;
+            }
+        } else {
+            if (hipMemcpy(d_aux, h_aux + (size_t)a0 * dim, (size_t)cq * dim * sizeof(float), hipMemcpyHostToDevice) !=
+                hipSuccess) {
+                rc = fail(CORAL_ERR_DEVICE, "upload of auxiliary queries failed");
+                break;
+            }
+            double t = 0.0;
+            if ((rc = coral_bruteforce_knn_gpu(idx, d_aux, (int32_t)cq, kb, 0, d_knn, nullptr, nullptr, &t))) break;
+            S->knn_s += t;
         }
-        double t = 0.0;
-        if ((rc = coral_bruteforce_knn_gpu(idx, d_aux, (int32_t)cq, kb, 0, d_knn, nullptr, nullptr, &t))) break;
-        S->knn_s += t;
         const double t1 = now_s();
         for (int64_t b0 = 0; b0 < cq; b0 += prm->batch) {
             const int b = (int)std::min<int64_t>(prm->batch, cq - b0);
@@ -298,6 +308,18 @@ int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const cor
     for (int32_t d : deg) S->edges += d;
     S->total_s = now_s() - t0;
     return CORAL_OK;
+}
+
+int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const coral_build_params* prm,
+                      coral_build_stats* stats) {
+    if (!h_aux) return fail(CORAL_ERR_ARG, "null argument");
+    return build_impl(idx, h_aux, nullptr, A, prm, stats);
+}
+
+int coral_build_graph_from_clusters(coral_index* idx, const int32_t* h_clusters, int64_t A, const coral_build_params* prm,
+                                    coral_build_stats* stats) {
+    if (!h_clusters) return fail(CORAL_ERR_ARG, "null argument");
+    return build_impl(idx, nullptr, h_clusters, A, prm, stats);
 }
 
 int coral_index_get_graph(coral_index* idx, int32_t* h_nbrs, float* h_dists, int32_t* h_deg, int32_t* h_start_ids) {

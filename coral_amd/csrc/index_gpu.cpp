@@ -155,7 +155,7 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     k_ = parameters.Get<int>("k");
     metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
     graph_dir_ = parameters.Get<std::string>("graph_file");
-    if (!bp_data || !sq_data || n_bp == 0 || n_sq == 0) throw std::runtime_error("BuildGPU: empty input");
+    if (!bp_data || n_bp == 0) throw std::runtime_error("BuildGPU: empty input");
     if (bp_data != h_base_) {  // keep a copy, like RunPrepare does with caller-owned vectors
         std::free(h_base_);
         h_base_ = nullptr;
@@ -176,7 +176,19 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     p.R = max_degree_, p.k_b = k_, p.batch = PC.batch, p.need_discard = PC.need_discard, p.connect_enhance = CE;
     p.enhance_search_batch = PC.enhance_search_batch, p.enhance_nap_batch = PC.enhance_nap_batch;
     p.n_start = PC.search_start_nodes_num;
-    if (coral_build_graph(index_, sq_data, (int64_t)n_sq, &p, &last_build)) raise("BuildGPU");
+    const std::string train_gt = parameters.Get<std::string>("train_gt_file", std::string("None"));
+    if (train_gt != "None" && !train_gt.empty()) {
+        // clusters from a ground-truth file of the sampled queries (src/index_gpu.cpp:505-515: nq, k, ids)
+        int32_t nq = 0, gk = 0;
+        if (coral_gt_read_meta(train_gt.c_str(), &nq, &gk)) raise("train_gt_file");
+        if (gk != k_) throw std::runtime_error("BuildGPU: train_gt_file holds k=" + std::to_string(gk) + ", expected " +
+                                               std::to_string(k_));
+        std::vector<int32_t> clusters((size_t)nq * gk);
+        if (coral_gt_read(train_gt.c_str(), clusters.data(), nq, gk)) raise("train_gt_file");
+        if (coral_build_graph_from_clusters(index_, clusters.data(), nq, &p, &last_build)) raise("BuildGPU");
+    } else if (coral_build_graph(index_, sq_data, (int64_t)n_sq, &p, &last_build)) {
+        raise("BuildGPU");
+    }
     // Graph::save_build (include/graph.cuh:481-484): start ids, then every row with its distances
     nbrs_.assign(nd_ * (size_t)max_degree_, -1);
     std::vector<float> dists(nd_ * (size_t)max_degree_);

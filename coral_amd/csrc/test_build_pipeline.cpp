@@ -5,9 +5,9 @@
 //   --data_type --dist {l2,ip} --N --dataset --base_data_path --train_gt_file --sampled_query_data_path
 //   --query_test_file --gt_test_file --M_sq --M_pjbp --L_pjpq --num_threads/-T --CE --k --iso_thres
 //   --recall_thres --query_thres --log_file --config_file
-// --M_pjbp is the row width, --k the cluster size (nearest base points per sampled query).  --train_gt_file
-// (precomputed clusters), --query_test_file / --gt_test_file (searches during the build) and the knn cache are
-// not provided: naming a file for one of them is an error.
+// --M_pjbp is the row width, --k the cluster size (nearest base points per sampled query).  --train_gt_file names
+// precomputed clusters (a ground-truth file of the sampled queries with k ids per row).  --query_test_file /
+// --gt_test_file (searches during the build) and the knn cache are not provided: naming a test file is an error.
 // Extensions: --index_dir <dir> (overrides the derived <index_prefix><dataset>_<dist>_<R>_<thres>_<CE> path) and
 // --index_prefix (default ../indexes/).
 #include <chrono>
@@ -92,10 +92,6 @@ int main(int argc, char** argv) {
         std::cerr << "only --data_type float is provided\n";
         return -1;
     }
-    if (!str("train_gt_file").empty() && str("train_gt_file") != "None") {
-        std::cerr << "--train_gt_file is not provided: the clusters are computed from --sampled_query_data_path\n";
-        return -1;
-    }
     if (str("query_test_file") != "None" || str("gt_test_file") != "None") {
         std::cerr << "--query_test_file / --gt_test_file are not provided: run test_search_pipeline on the result\n";
         return -1;
@@ -145,6 +141,7 @@ int main(int argc, char** argv) {
         parameters.Set<std::string>("config_file", str("config_file"));
         parameters.Set<std::string>("dist", dist);
         parameters.Set<std::string>("dataset", dataset);
+        parameters.Set<std::string>("train_gt_file", str("train_gt_file").empty() ? "None" : str("train_gt_file"));
 
         IndexGPU index((size_t)base_stride, (size_t)(base_num + sq_num), dist_metric, nullptr);
         const auto s = std::chrono::high_resolution_clock::now();

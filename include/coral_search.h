@@ -244,6 +244,12 @@ CORAL_API int coral_build_connect_enhance(coral_index* idx, const coral_build_pa
 CORAL_API int coral_build_graph(coral_index* idx, const float* h_aux, int64_t A, const coral_build_params* params,
                                 coral_build_stats* stats);
 
+/* The same with the clusters given instead of computed: h_clusters int32 [A][k_b], row i = the k_b nearest base
+ * ids of auxiliary query i, distinct within a row (GraphTask's train_gt_file branch, src/index_gpu.cpp:505-537;
+ * the payload of a ground-truth file of the auxiliary queries with k = k_b). */
+CORAL_API int coral_build_graph_from_clusters(coral_index* idx, const int32_t* h_clusters, int64_t A,
+                                              const coral_build_params* params, coral_build_stats* stats);
+
 /* Download rows [n][R] (-1 padded) and start ids [n_start]; during a build also the per-neighbour distances
  * [n][R] and degrees [n] (the dists and deg fields of the reference's Slot).  Any pointer may be NULL. */
 CORAL_API int coral_index_get_graph(coral_index* idx, int32_t* h_nbrs, float* h_dists, int32_t* h_deg,

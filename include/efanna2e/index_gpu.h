@@ -104,7 +104,8 @@ class CORAL_API IndexGPU {
     // src/index_gpu.cpp:308-383: builds the graph over the n_bp base vectors from the n_sq auxiliary ("sampled")
     // queries and writes the index directory parameters["graph_file"] (graph.part*.idx/.data, graph.search_start_ids,
     // graph.batch_id).  Reads config_file, CE (0 or 1; 2, "only CE", is not provided), max_degree, k (the cluster
-    // size), dist, graph_file.  Both arrays hold rows of GetDimension() floats.  The built index stays loaded, so
+    // size), dist, graph_file, train_gt_file (optional: the clusters, as a ground-truth file of the sampled queries with k
+    // ids per row; sq_data is then unused).  Both arrays hold rows of GetDimension() floats.  The built index stays loaded, so
     // Search works right after.  The timings and counts of the run are in last_build.
     void BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data, Parameters& parameters);
     coral_build_stats last_build{};

@@ -130,8 +130,8 @@ def test_build_cli_flag_handling():
     assert r.returncode == 255 and "Unknown distance type" in r.stdout
     r = run(*base, "--dist", "l2")
     assert r.returncode == 1 and "open file error" in r.stderr
-    r = run(*base, "--dist", "l2", "--train_gt_file", "clusters.bin")
-    assert r.returncode == 255 and "train_gt_file" in r.stderr
+    r = run(*base, "--dist", "l2", "--gt_test_file", "gt.bin")
+    assert r.returncode == 255 and "gt_test_file" in r.stderr
     r = run(*base, "--dist", "l2", "--CE", "x")
     assert r.returncode == 255
 
@@ -143,6 +143,7 @@ def test_build_entry_points_reject_bad_arguments_before_any_device_call():
     assert lib.coral_build_enhance_batch(None, None, None, None, 1, 10, None, None) == capi.ERR_ARG
     assert lib.coral_build_connect_enhance(None, None, None) == capi.ERR_ARG
     assert lib.coral_build_graph(None, None, 0, None, None) == capi.ERR_ARG
+    assert lib.coral_build_graph_from_clusters(None, None, 0, None, None) == capi.ERR_ARG
     assert lib.coral_index_get_graph(None, None, None, None, None) == capi.ERR_ARG
     assert lib.coral_start_ids_fps(None, 0, 1, None) == capi.ERR_ARG
     assert lib.coral_index_mark_deleted(None, None, 0) == capi.ERR_ARG

@@ -93,6 +93,49 @@ def test_enhance_batches_equal_the_oracle(orc, metric, R, kn, seed):
     idx.close()
 
 
+def test_randomised_shapes_of_both_steps_equal_the_oracle(orc):
+    """Seeded random sizes, widths, cluster sizes, metrics and fill modes, small enough for the oracle; each case
+    runs a few batch updates and one enhancement batch."""
+    rng = np.random.RandomState(2024)
+    for case in range(30):
+        dim = int(rng.choice([4, 8, 12, 36, 64, 100, 128, 200, 256]))
+        R = int(rng.randint(1, 33))
+        kb = int(rng.choice([2, 3, 5, 17, 40, 64, 100, 128]))
+        n = int(rng.randint(kb + 20, 3000))
+        batch = int(rng.randint(1, 80))
+        metric = int(rng.randint(0, 2))
+        fill = int(rng.randint(0, 2))
+        print("case %d: n=%d dim=%d R=%d kb=%d batch=%d metric=%d fill=%d" % (case, n, dim, R, kb, batch, metric, fill),
+              flush=True)
+        base = base_of(n, dim, 1000 + case, metric)
+        if case % 7 == 0:
+            base = np.round(base * 2) / 2 if metric == capi.L2 else base  # ties
+        linked_n = max(kb + 1, (2 * n) // 3)
+        idx = capi.Index(base, None, None, metric=metric)
+        idx.build_begin(R)
+        st = orc.GraphState(n, R)
+        for it in range(3):
+            knn = np.stack([rng.choice(linked_n, kb, replace=False) for _ in range(batch)]).astype(np.int32)
+            t_knn = dev(knn)
+            idx.build_nap_batch(t_knn.data_ptr(), batch, kb, fill)
+            orc.nap_batch(base, st, knn, metric=metric, need_discard=fill)
+            assert_same_state(idx, st)
+        linked = np.where(st.deg > 0)[0].astype(np.int32)
+        iso = np.where(st.deg == 0)[0].astype(np.int32)[:50]
+        kn = int(min(linked.size, rng.choice([1, 7, 33, 100, 160])))
+        if iso.size and kn:
+            ids, dd = orc.bruteforce(base[linked], base[iso], kn, metric, order=SEQ)
+            ids = linked[ids]
+            if kn > 2:
+                ids[0, kn // 2:] = -1
+            t_iso, t_ids, t_dd = dev(iso), dev(ids), dev(dd)
+            ins, rej = idx.build_enhance_batch(t_iso.data_ptr(), t_ids.data_ptr(), t_dd.data_ptr(), iso.size, kn)
+            stats = orc.enhance_batch(base, st, iso, ids, dd, metric=metric)
+            assert (ins, rej) == (stats[0], stats[1])
+            assert_same_state(idx, st)
+        idx.close()
+
+
 def oracle_pipeline(orc, base, aux, metric, p):
     """IndexGPU::BuildGPU composed from the oracle's pieces, in the order coral_build_graph documents."""
     n = base.shape[0]
@@ -218,70 +261,19 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     row = [l for l in r.stdout.splitlines() if l.startswith("64\t")][0].split()
     oi, _, _, _ = orc.search_B(orc.Problem(base, nbrs, starts), q, k, 64, start_order=WAVE64, nbr_order=WAVE64)
     assert abs(float(row[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
-    # refused: precomputed clusters, unknown metric
-    r = subprocess.run(args[:1] + ["--help"], capture_output=True, text=True, timeout=60)
-    assert r.returncode == 0
-    bad = [os.path.join(root, "coral_amd", "lib", "test_build_pipeline"), "--data_type", "float", "--dist", "l2",
-           "--dataset", "syn", "--base_data_path", str(work / "base.fbin"), "--sampled_query_data_path",
-           str(work / "aux.fbin"), "--train_gt_file", "x.bin"]
-    r = subprocess.run(bad, cwd=work / "cwd", capture_output=True, text=True, timeout=60)
-    assert r.returncode != 0 and "train_gt_file" in r.stderr
-
-
-def test_batch_update_and_enhancement_at_the_real_shape(orc):
-    """1M x 200, clusters of 100, rows of 32: single steps of a running construction against the oracle applied
-    to the state the device held before the step (the whole construction at this size is too slow for the CPU)."""
-    import time
-    import torch
-    from coral_amd import workloads
-    n, dim, kb, R, batch = 1000000, 200, 100, 32, 1024
-    base = workloads.gaussian_base(2001, n, dim)
-    aux = synth.shifted_queries(12 * batch, dim, 2002, 2003, 2005)
-    idx = capi.Index(base, None, None)
-    d_aux = torch.from_numpy(aux).cuda()
-    d_knn = torch.empty((aux.shape[0], kb), dtype=torch.int32, device="cuda")
-    idx.bruteforce_device(d_aux.data_ptr(), d_knn.data_ptr(), None, aux.shape[0], kb)
-    knn = d_knn.cpu().numpy()
-    idx.build_begin(R)
-
-    def state():
-        st = orc.GraphState(0, R)
-        st.nbrs, st.dists, st.deg, _ = idx.get_graph(with_build_state=True)
-        return st
-
-    for b in range(12):
-        check = b in (0, 6, 11)
-        if check:
-            st = state()
-        t0 = time.perf_counter()
-        idx.build_nap_batch(d_knn[b * batch:].data_ptr(), batch, kb, True)
-        t_gpu = time.perf_counter() - t0
-        if check:
-            t0 = time.perf_counter()
-            stats = orc.nap_batch(base, st, knn[b * batch:(b + 1) * batch])
-            print("batch %d: device %.1f ms (call), oracle on %d host threads %.0f ms; %d pivots written, %d distance "
-                  "evaluations of the occlusion rule" % (b, 1e3 * t_gpu, orc.max_threads(), 1e3 * (time.perf_counter() - t0),
-                                                         stats[0], stats[1]), flush=True)
-            assert stats[0] > 50000
-            assert_same_state(idx, st)
-    # one enhancement batch: entry points, the search for 4096 isolated nodes' own vectors, the batch itself
-    st = state()
-    assert ((st.nbrs >= 0).sum(1) == st.deg).all()
-    first = int(np.where(st.deg > 0)[0][0])
-    starts = idx.start_ids_fps(first, 16)
-    assert starts.tolist() == orc.fps(st.nbrs, first, 16).tolist()
-    idx.set_graph(st.nbrs, starts)
-    iso = np.where(st.deg == 0)[0][:4096].astype(np.int32)
-    ids, dd, _ = idx.search(base[iso], kb, 256)
-    assert (ids >= 0).all() and not np.isin(ids, iso).any()
-    t_iso, t_ids, t_dd = dev(iso), dev(ids), dev(dd)
-    t0 = time.perf_counter()
-    ins, rej = idx.build_enhance_batch(t_iso.data_ptr(), t_ids.data_ptr(), t_dd.data_ptr(), iso.size, kb)
-    t_gpu = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    stats = orc.enhance_batch(base, st, iso, ids, dd)
-    print("enhancement batch of %d: device %.1f ms (call), oracle on one host thread %.0f ms; %d reverse edges" %
-          (iso.size, 1e3 * t_gpu, 1e3 * (time.perf_counter() - t0), ins), flush=True)
-    assert (ins, rej) == (stats[0], stats[1]) and ins > 10000
-    assert_same_state(idx, st)
-    idx.close()
+    # the same construction from precomputed clusters (--train_gt_file: a ground-truth file of the sampled queries)
+    clusters, _ = orc.bruteforce(base, aux, 24, order=SEQ)
+    formats.gt_write(work / "clusters.bin", clusters)
+    build_cli = os.path.join(root, "coral_amd", "lib", "test_build_pipeline")
+    args2 = [build_cli, "--data_type", "float", "--dist", "l2", "--dataset", "syn", "--base_data_path",
+             str(work / "base.fbin"), "--sampled_query_data_path", str(work / "aux.fbin"), "--M_pjbp", "16", "--k", "24",
+             "--config_file", str(work / "config.json"), "--train_gt_file", str(work / "clusters.bin"), "--index_dir",
+             str(work / "from_clusters")]
+    r = subprocess.run(args2, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr + r.stdout
+    nbrs2, dists2 = formats.graph_dir_read(work / "from_clusters", n, 16, want_dists=True)
+    assert np.array_equal(nbrs2, nbrs) and dists2.tobytes() == dists.tobytes()
+    assert formats.start_ids_read(work / "from_clusters").tolist() == starts.tolist()
+    r = subprocess.run(args2[:-4] + ["--k", "25", "--train_gt_file", str(work / "clusters.bin")], cwd=work / "cwd",
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1 and "expected 25" in r.stderr
