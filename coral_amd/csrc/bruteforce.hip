@@ -12,9 +12,10 @@
 //                         dimension -- the arithmetic of the reference's l2_distance / ip_distance
 //                         (include/utils.cuh:254-275, 307-323) -- so the distances, and hence the
 //                         ids, are reproducible bit for bit on a CPU.
-//   row_select_kernel     per query row: exact k-th smallest by an 8-bit radix select over the
-//                         order-preserving bit pattern, then ordered compaction (ties by id) and
-//                         a bitonic sort of the k winners.
+//   row_select_kernel     per query row: a threshold from the per-thread minima, one more pass that
+//                         collects the entries up to it into LDS, a sort by (value, id).  Rows with too
+//                         many ties at the threshold go to row_select_radix_kernel: exact k-th smallest by
+//                         an 8-bit radix select over the order-preserving bit pattern, ordered compaction.
 //   merge_segments_kernel per query: the k best of the per-segment winners (large bases are
 //                         processed in segments so the distance buffer stays bounded).
 #include <hip/hip_runtime.h>
@@ -128,14 +129,121 @@ __global__ __launch_bounds__(256) void distance_tile_kernel(const float* __restr
 // One workgroup per row of n floats: the k smallest under (value, index), sorted, as
 // keys ord32(value) << 32 | (id0 + index).  Fewer than k finite entries: padded with ~0.
 // Entries equal to +inf (tombstones) never win over finite ones and are dropped at the end.
-__global__ __launch_bounds__(256) void row_select_kernel(const float* __restrict__ D, int64_t ldD,
-                                                         int64_t n, int k, int64_t id0,
-                                                         unsigned long long* __restrict__ out,
-                                                         int64_t out_stride) {
+//
+// row_select_kernel is the fast path.  Every thread keeps the smallest value of the entries it reads; the k-th
+// smallest of those 1024 minima is a value that at least k entries of the row do not exceed (the minima are
+// distinct entries), and in a row of independent values hardly more than k do (about k + k^2/2048).  A second pass
+// collects the entries up to that value into LDS, a sort by (value, index) finishes.  Two coalesced reads of the
+// row, no atomics on the way.  A row with so many ties at the threshold that the candidates outgrow LDS is
+// flagged and left to row_select_radix_kernel, which makes no such assumption.
+constexpr int kSelThreads = 1024;
+constexpr int kSelCap = 4096;  // candidate keys in LDS
+
+__global__ __launch_bounds__(kSelThreads) void row_select_kernel(const float* __restrict__ D, int64_t ldD, int64_t n,
+                                                                 int k, int64_t id0,
+                                                                 unsigned long long* __restrict__ out,
+                                                                 int64_t out_stride, int* __restrict__ redo) {
+    __shared__ unsigned long long skeys[kSelCap];
+    __shared__ uint32_t smin[kSelThreads];
+    __shared__ unsigned int s_count;
+    const int tid = threadIdx.x;
+    const float* row = D + (size_t)blockIdx.x * ldD;
+    const int kk = (int)min((int64_t)k, n);
+    const int64_t n4 = n >> 2;
+    const float4* row4 = reinterpret_cast<const float4*>(row);  // rows start 16-byte aligned (ldD % 4 == 0)
+    // pass 1: per-thread minimum
+    uint32_t m = 0xffffffffu;
+    for (int64_t i = tid; i < n4; i += 2 * kSelThreads) {
+        const float4 v0 = row4[i];
+        const float4 v1 = i + kSelThreads < n4 ? row4[i + kSelThreads] : v0;
+        m = min(m, min(min(bf_ord32(v0.x), bf_ord32(v0.y)), min(bf_ord32(v0.z), bf_ord32(v0.w))));
+        m = min(m, min(min(bf_ord32(v1.x), bf_ord32(v1.y)), min(bf_ord32(v1.z), bf_ord32(v1.w))));
+    }
+    for (int64_t i = (n4 << 2) + tid; i < n; i += kSelThreads) m = min(m, bf_ord32(row[i]));
+    smin[tid] = m;
+    if (tid == 0) s_count = 0u;
+    __syncthreads();
+    // the kk-th smallest of the minima: bitonic sort of 1024 values
+    for (int k2 = 2; k2 <= kSelThreads; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1) {
+            if (tid < kSelThreads / 2) {
+                const int i = 2 * tid - (tid & (j - 1)), x = i + j;
+                const bool asc = (i & k2) == 0;
+                const uint32_t a = smin[i], b = smin[x];
+                if ((a > b) == asc) smin[i] = b, smin[x] = a;
+            }
+            __syncthreads();
+        }
+    const uint32_t thr = kk <= kSelThreads ? smin[kk - 1] : 0xffffffffu;
+    // pass 2: everything up to the threshold
+    for (int64_t i0 = 0; i0 < n4; i0 += kSelThreads) {
+        const int64_t i = i0 + tid;
+        float4 v = make_float4(0, 0, 0, 0);
+        bool hit = false;
+        uint32_t o[4] = {0, 0, 0, 0};
+        if (i < n4) {
+            v = row4[i];
+            o[0] = bf_ord32(v.x), o[1] = bf_ord32(v.y), o[2] = bf_ord32(v.z), o[3] = bf_ord32(v.w);
+            hit = o[0] <= thr || o[1] <= thr || o[2] <= thr || o[3] <= thr;
+        }
+        if (__ballot(hit) == 0ull) continue;  // uniform in the wavefront
+        if (hit) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (o[j] <= thr) {
+                    const unsigned pos = atomicAdd(&s_count, 1u);
+                    if (pos < (unsigned)kSelCap)
+                        skeys[pos] = ((unsigned long long)o[j] << 32) | (unsigned long long)(uint32_t)(id0 + 4 * i + j);
+                }
+        }
+    }
+    for (int64_t i = (n4 << 2) + tid; i < n; i += kSelThreads) {
+        const uint32_t o = bf_ord32(row[i]);
+        if (o <= thr) {
+            const unsigned pos = atomicAdd(&s_count, 1u);
+            if (pos < (unsigned)kSelCap) skeys[pos] = ((unsigned long long)o << 32) | (unsigned long long)(uint32_t)(id0 + i);
+        }
+    }
+    __syncthreads();
+    const unsigned count = s_count;
+    if (count > (unsigned)kSelCap) {  // too many ties at the threshold: the radix kernel takes this row
+        if (tid == 0) redo[blockIdx.x] = 1;
+        return;
+    }
+    if (tid == 0) redo[blockIdx.x] = 0;
+    int P = 2;
+    while (P < (int)count) P <<= 1;
+    for (int i = (int)count + tid; i < P; i += kSelThreads) skeys[i] = ~0ull;
+    __syncthreads();
+    for (int k2 = 2; k2 <= P; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1) {
+            for (int t = tid; t < (P >> 1); t += kSelThreads) {
+                const int i = 2 * t - (t & (j - 1)), x = i + j;
+                const bool asc = (i & k2) == 0;
+                const unsigned long long ka = skeys[i], kb = skeys[x];
+                if ((ka > kb) == asc) skeys[i] = kb, skeys[x] = ka;
+            }
+            __syncthreads();
+        }
+    unsigned long long* dst = out + (size_t)blockIdx.x * out_stride;
+    for (int i = tid; i < k; i += kSelThreads) {
+        unsigned long long key = i < kk ? skeys[i] : ~0ull;
+        if ((uint32_t)(key >> 32) == bf_ord32(__int_as_float(0x7f800000))) key = ~0ull;  // tombstoned
+        dst[i] = key;
+    }
+}
+
+// The general path: exact k-th smallest by an 8-bit radix select, then ordered compaction.  Only rows flagged in
+// redo (or all rows when redo is null) are processed.
+__global__ __launch_bounds__(256) void row_select_radix_kernel(const float* __restrict__ D, int64_t ldD,
+                                                               int64_t n, int k, int64_t id0,
+                                                               unsigned long long* __restrict__ out,
+                                                               int64_t out_stride, const int* __restrict__ redo) {
     extern __shared__ unsigned long long skeys[];  // pow2 >= k keys
     __shared__ unsigned int hist[256];
     __shared__ unsigned int s_prefix, s_need, s_count, s_base;
     const int tid = threadIdx.x;
+    if (redo && !redo[blockIdx.x]) return;
     const float* row = D + (size_t)blockIdx.x * ldD;
     const int kk = (int)min((int64_t)k, n);
 
@@ -301,11 +409,15 @@ hipError_t launch_distance_tile(const float* queries, const float* base, int nq,
 }
 
 hipError_t launch_row_select(const float* D, int64_t ldD, int nq, int64_t n, int k, int64_t id0,
-                             unsigned long long* out, int64_t out_stride, hipStream_t stream) {
+                             unsigned long long* out, int64_t out_stride, int* redo, hipStream_t stream) {
     int P = 2;
     while (P < k) P <<= 1;
-    hipLaunchKernelGGL(row_select_kernel, dim3(nq), dim3(256), (size_t)P * 8, stream, D, ldD, n, k, id0, out,
-                       out_stride);
+    const bool fast = redo != nullptr && k <= kSelThreads;
+    if (fast)
+        hipLaunchKernelGGL(row_select_kernel, dim3(nq), dim3(kSelThreads), 0, stream, D, ldD, n, k, id0, out, out_stride,
+                           redo);
+    hipLaunchKernelGGL(row_select_radix_kernel, dim3(nq), dim3(256), (size_t)P * 8, stream, D, ldD, n, k, id0, out,
+                       out_stride, fast ? redo : nullptr);
     return hipGetLastError();
 }
 

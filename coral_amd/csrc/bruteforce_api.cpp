@@ -37,9 +37,11 @@ int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q
     qc = std::min<int64_t>(qc, ((int64_t)Q + 127) & ~(int64_t)127);
     float* D = nullptr;
     unsigned long long* part = nullptr;
+    int* redo = nullptr;
     auto release = [&]() {
         (void)hipFree(D);
         (void)hipFree(part);
+        (void)hipFree(redo);
     };
 #define HIP_TRY_R(expr)                                                                  \
     do {                                                                                 \
@@ -52,6 +54,7 @@ int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q
     } while (0)
     HIP_TRY_R(hipMalloc(&D, (size_t)qc * ld * sizeof(float)));
     HIP_TRY_R(hipMalloc(&part, (size_t)Q * nseg * k * sizeof(unsigned long long)));
+    HIP_TRY_R(hipMalloc(&redo, (size_t)qc * sizeof(int)));
     hipEvent_t ev0, ev1;
     HIP_TRY_R(hipEventCreate(&ev0));
     HIP_TRY_R(hipEventCreate(&ev1));
@@ -65,7 +68,7 @@ int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q
                                                   idx->metric, have_delete ? idx->d_deleted : nullptr, b0, D, ld,
                                                   stream));
             HIP_TRY_R(coral::launch_row_select(D, ld, nq, nb, k, b0, part + ((size_t)q0 * nseg + s) * k,
-                                               nseg * k, stream));
+                                               nseg * k, redo, stream));
         }
     }
     HIP_TRY_R(coral::launch_merge_segments(part, Q, (int)nseg, k, idx->metric, d_ids, d_dists, stream));

@@ -99,6 +99,28 @@ def test_bruteforce_ties_are_ordered_by_id(orc):
     idx.close()
 
 
+def test_bruteforce_rows_with_thousands_of_ties_and_large_k(orc):
+    # 30 000 points on a 3 x 3 x 3 x 3 lattice: every distance value is shared by hundreds of points, so the
+    # candidates at the selection threshold outgrow the fast path's buffer and the radix path takes the rows;
+    # k above 1024 goes to the radix path directly
+    rng = np.random.RandomState(3)
+    pts = rng.randint(0, 3, (30000, 4)).astype(np.float32)
+    q = np.array([[1, 1, 1, 1], [0, 0, 0, 0], [0.5, 2, 1, 0], [7, 7, 7, 7]], np.float32)
+    idx = capi.Index(pts, None, None)
+    for k in (1, 100, 1000, 1025, 2000):
+        ids, dists, _ = idx.bruteforce(q, k)
+        oi, od = orc.bruteforce(pts, q, k, order=SEQ)
+        assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+    # a mix in one batch: rows with few ties next to rows with many
+    mixed = np.concatenate([pts[:15000], synth.gaussian_matrix(5, 15000, 4)])
+    idx2 = capi.Index(mixed, None, None)
+    q2 = np.concatenate([q, synth.gaussian_matrix(6, 4, 4)])
+    ids, dists, _ = idx2.bruteforce(q2, 64)
+    oi, od = orc.bruteforce(mixed, q2, 64, order=SEQ)
+    assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+    idx.close(), idx2.close()
+
+
 def test_bruteforce_segments(orc):
     # more base points than one pass holds (4M): per-segment winners are merged
     n, dim, Q, k = 5 * 1000 * 1000, 8, 40, 50
