@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
-Workload (BASELINE.json configs[1]): 1 000 000 x 200 fp32 base vectors N(0,I),
+Workload (the headline configuration): 1 000 000 x 200 fp32 base vectors N(0,I),
 10 000 queries from the shifted anisotropic law, degree-32 graph built from
 100 000 auxiliary queries, L2, k = 100, all queries in one batch, L in {256, 512}.
 One step = one search of the whole batch (one persistent kernel launch) with the
