@@ -73,15 +73,15 @@ def main():
     d_ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
     d_gt = torch.from_numpy(gt).cuda()
 
-    def run(L, steps, warmup):
-        idx.prepare(Q, L)
+    def run(L, steps, warmup, policy=capi.POLICY_ROUNDS):
+        idx.prepare(Q, L, policy=policy)
         for _ in range(warmup):
-            idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k)
+            idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k, policy=policy)
         torch.cuda.synchronize()
         t = time.perf_counter()
         kernel_s, st = 0.0, None
         for _ in range(steps):
-            st = idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k)
+            st = idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k, policy=policy)
             kernel_s += st.kernel_s
         torch.cuda.synchronize()
         wall = time.perf_counter() - t
@@ -102,6 +102,8 @@ def main():
         del src, dst
     other_L = 256 if args.L == 512 else 512
     also = None if args.only_L else run(other_L, max(3, args.steps // 2), 1)
+    # the CPU path's traversal (best-first) on the GPU, for the comparison with cpu_baseline at equal policy
+    best_first = None if args.only_L else run(args.L, 3, 1, policy=capi.POLICY_BEST_FIRST)
     head = run(args.L, args.steps, args.warmup)
 
     out = {
@@ -123,6 +125,9 @@ def main():
     if also:
         out["also"] = {k2: also[k2] for k2 in ("L", "qps", "recall", "kernel_ms", "gbps", "ms_per_step", "spills")}
         out["also"]["frac"] = also["gbps"] / HBM_PEAK_GBPS
+    if best_first:
+        out["best_first"] = {k2: best_first[k2] for k2 in ("L", "qps", "recall", "kernel_ms", "gbps",
+                                                           "dist_evals_per_query", "expansions_per_query")}
 
     # the IndexGPU::Search shape: host buffers in and out (device allocation, query upload,
     # search, id download); reported beside the headline, never as the headline
