@@ -260,15 +260,21 @@ class Index:
     def build_connect_enhance(self, params):
         st = BuildStats()
         _check(lib().coral_build_connect_enhance(self._h, C.byref(params), C.byref(st)))
-        self.n_start = params.n_start
+        self._refresh_n_start()
         return st
+
+    def _refresh_n_start(self):
+        m = C.c_int32()
+        _check(lib().coral_index_info(self._h, None, None, None, C.byref(m), None))
+        self.n_start = m.value
 
     def build_graph(self, aux, params):
         """IndexGPU::BuildGPU: the whole construction from host auxiliary queries [A][dim]."""
         aux = np.ascontiguousarray(aux, dtype=np.float32)
         st = BuildStats()
         _check(lib().coral_build_graph(self._h, _ptr(aux), aux.shape[0], C.byref(params), C.byref(st)))
-        self.R, self.n_start = params.R, params.n_start
+        self.R = params.R
+        self._refresh_n_start()
         return st
 
     def build_graph_from_clusters(self, clusters, params):
@@ -278,7 +284,8 @@ class Index:
             raise ValueError("clusters must be [A][k_b]")
         st = BuildStats()
         _check(lib().coral_build_graph_from_clusters(self._h, _ptr(c), c.shape[0], C.byref(params), C.byref(st)))
-        self.R, self.n_start = params.R, params.n_start
+        self.R = params.R
+        self._refresh_n_start()
         return st
 
     def get_graph(self, with_build_state=False):

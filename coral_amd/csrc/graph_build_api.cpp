@@ -33,7 +33,14 @@ double now_s() {
     return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
 
-int set_start_ids(coral_index* idx, const int32_t* ids, int M) {
+// The sampling repeats an id once every node it can reach is taken (a linked part smaller than the number of
+// entry points asked for); the search wants distinct start ids, so repeats are dropped here.
+int set_start_ids(coral_index* idx, const int32_t* all_ids, int count) {
+    std::vector<int32_t> uniq;
+    for (int i = 0; i < count; ++i)
+        if (std::find(uniq.begin(), uniq.end(), all_ids[i]) == uniq.end()) uniq.push_back(all_ids[i]);
+    const int32_t* ids = uniq.data();
+    const int M = (int)uniq.size();
     if (M != idx->M) {
         int32_t* p = nullptr;
         HIP_TRY(hipMalloc(&p, (size_t)M * sizeof(int32_t)));

@@ -192,7 +192,9 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     // Graph::save_build (include/graph.cuh:481-484): start ids, then every row with its distances
     nbrs_.assign(nd_ * (size_t)max_degree_, -1);
     std::vector<float> dists(nd_ * (size_t)max_degree_);
-    start_ids_.assign((size_t)p.n_start, 0);
+    int32_t n_start = 0;  // can be below p.n_start when fewer nodes are reachable
+    if (coral_index_info(index_, nullptr, nullptr, nullptr, &n_start, nullptr)) raise("BuildGPU");
+    start_ids_.assign((size_t)n_start, 0);
     if (coral_index_get_graph(index_, nbrs_.data(), dists.data(), nullptr, start_ids_.data())) raise("download graph");
     if (coral_build_end(index_)) raise("BuildGPU");
     if (coral_graph_dir_write(graph_dir_.c_str(), (int64_t)nd_, max_degree_, nbrs_.data(), dists.data()))

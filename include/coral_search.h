@@ -232,7 +232,8 @@ CORAL_API int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_i
 /* GPUFuncs::gpu_connect_enhance, isolated nodes (src/enhance.cu:728-803, enhance_mode 0): per search batch, entry
  * points by coral_start_ids_fps on the graph as it is, one CORAL_POLICY_ROUNDS search (k = k_b, L = enhance_L) for
  * the isolated nodes' own vectors, then coral_build_enhance_batch per enhance_nap_batch.  The entry points of the
- * last search batch stay the index's start ids, as in the reference.  Its second phase (top_hit_num most-hit nodes,
+ * last search batch stay the index's start ids, as in the reference (fewer than n_start when fewer nodes can be
+ * reached: an id is never listed twice).  Its second phase (top_hit_num most-hit nodes,
  * src/enhance.cu:819-856) is not built: it is off by the code's default (src/index_gpu.cpp:78) and reads past its
  * id array whenever top_hit_num exceeds n. */
 CORAL_API int coral_build_connect_enhance(coral_index* idx, const coral_build_params* params, coral_build_stats* stats);

@@ -277,3 +277,21 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     r = subprocess.run(args2[:-4] + ["--k", "25", "--train_gt_file", str(work / "clusters.bin")], cwd=work / "cwd",
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 1 and "expected 25" in r.stderr
+
+
+def test_fewer_reachable_nodes_than_entry_points(orc):
+    # one cluster of 5 nodes, no enhancement: the sampling runs out of reachable nodes after 5 ids and repeats
+    # itself (as the oracle's does); the index keeps each id once and still searches
+    n, dim = 64, 8
+    base = synth.gaussian_matrix(3, n, dim)
+    p = capi.build_params(R=4, k_b=5, batch=4, connect_enhance=0, n_start=16)
+    idx = capi.Index(base, None, None)
+    clusters = np.array([[10, 11, 12, 13, 14]], np.int32)
+    idx.build_graph_from_clusters(clusters, p)
+    nbrs, starts = idx.get_graph()
+    want = orc.fps(nbrs, 10, 16)
+    assert len(set(want.tolist())) < 16  # repeats in the raw sampling
+    assert starts.tolist() == list(dict.fromkeys(want.tolist())) and sorted(starts.tolist()) == [10, 11, 12, 13, 14]
+    ids, _, _ = idx.search(base[10:12], 3, 8)
+    assert set(ids.ravel().tolist()) <= {10, 11, 12, 13, 14}
+    idx.close()
