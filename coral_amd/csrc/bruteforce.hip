@@ -60,20 +60,33 @@ __global__ __launch_bounds__(256) void distance_tile_kernel(const float* __restr
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
 
-    // staging: 128 rows x 8 dims per operand = 256 float4; thread t loads row t/2, dims (t&1)*4..
+    // staging: 128 rows x KC dims per operand = 32*KC float4, KC/8 per thread: thread t loads row t/2, dims
+    // (t&1)*4 + 8*u.  The loads of the next stage are issued before the arithmetic of the current one.
+    constexpr int NL = KC / 8;
     const int lrow = tid >> 1, lk = (tid & 1) * 4;
+    float4 vq[NL], vb[NL];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < NL; ++u) {
+            vq[u] = make_float4(0, 0, 0, 0), vb[u] = make_float4(0, 0, 0, 0);
+            const int kd = k0 + lk + 8 * u;
+            if (kd < dim) {
+                if (q0 + lrow < nq) vq[u] = *reinterpret_cast<const float4*>(queries + (size_t)(q0 + lrow) * dim + kd);
+                if (b0 + lrow < nb) vb[u] = *reinterpret_cast<const float4*>(base + (size_t)(b0 + lrow) * dim + kd);
+            }
+        }
+    };
+    fetch(0);
     for (int k0 = 0; k0 < dim; k0 += KC) {
-        float4 vq = make_float4(0, 0, 0, 0), vb = make_float4(0, 0, 0, 0);
-        if (k0 + lk < dim) {
-            if (q0 + lrow < nq)
-                vq = *reinterpret_cast<const float4*>(queries + (size_t)(q0 + lrow) * dim + k0 + lk);
-            if (b0 + lrow < nb)
-                vb = *reinterpret_cast<const float4*>(base + (size_t)(b0 + lrow) * dim + k0 + lk);
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < NL; ++u) {
+            const int r = lk + 8 * u;
+            sq[r + 0][lrow] = vq[u].x, sq[r + 1][lrow] = vq[u].y, sq[r + 2][lrow] = vq[u].z, sq[r + 3][lrow] = vq[u].w;
+            sb[r + 0][lrow] = vb[u].x, sb[r + 1][lrow] = vb[u].y, sb[r + 2][lrow] = vb[u].z, sb[r + 3][lrow] = vb[u].w;
         }
         __syncthreads();
-        sq[lk + 0][lrow] = vq.x, sq[lk + 1][lrow] = vq.y, sq[lk + 2][lrow] = vq.z, sq[lk + 3][lrow] = vq.w;
-        sb[lk + 0][lrow] = vb.x, sb[lk + 1][lrow] = vb.y, sb[lk + 2][lrow] = vb.z, sb[lk + 3][lrow] = vb.w;
-        __syncthreads();
+        if (k0 + KC < dim) fetch(k0 + KC);
         const int kend = min(KC, dim - k0);
         for (int kk = 0; kk < kend; ++kk) {
             float a[8], b[8];
