@@ -1,6 +1,8 @@
 """Exact brute-force kNN on the GPU (the ground-truth / builder-kNN component that replaces
 faiss): bit-exact against the oracle's brute force in the same summation order, and within
 tolerance of the fp64 closed form."""
+import time
+
 import numpy as np
 import pytest
 
@@ -145,7 +147,11 @@ def test_bruteforce_ground_truth_at_full_size(orc):
           (t, pairs / t / 1e12, 3 * pairs / t / 1e12), flush=True)
     assert (np.diff(dists, axis=1) >= 0).all()
     sub = np.arange(0, Q, 313)
+    t0 = time.perf_counter()
     oi, od = orc.bruteforce(base, q[sub], k, order=SEQ)
+    t_cpu = time.perf_counter() - t0
+    print("oracle on %d host threads: %d queries in %.2f s = %.0f queries/s (device: %.0f queries/s)" %
+          (orc.max_threads(), len(sub), t_cpu, len(sub) / t_cpu, Q / t), flush=True)
     assert np.array_equal(ids[sub], oi) and dists[sub].tobytes() == od.tobytes()
     # agrees with a matmul-based top-k (|b|^2 - 2 q.b, another arithmetic altogether) up to near-ties
     tb, tq = torch.from_numpy(base).cuda(), torch.from_numpy(q[sub]).cuda()
