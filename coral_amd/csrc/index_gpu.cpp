@@ -111,7 +111,9 @@ void IndexGPU::LoadSearchNeededData(const char* base_file, const char* sampled_q
 }
 
 void IndexGPU::RunPrepare(Parameters& parameters, Mode mode, size_t n_bp, float* bp_data) {
-    if (mode != Mode::SEARCH) throw std::runtime_error("only Mode::SEARCH is provided by this library");
+    // Mode::UPD loads the same state as Mode::SEARCH here: deletions are tombstones, rows are never rewritten
+    if (mode != Mode::SEARCH && mode != Mode::UPD)
+        throw std::runtime_error("only Mode::SEARCH and Mode::UPD are provided by this library");
     SetParameters(parameters);
     load_config(parameters.Get<std::string>("config_file", std::string("default")));
     graph_dir_ = parameters.Get<std::string>("graph_file");

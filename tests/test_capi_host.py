@@ -152,3 +152,26 @@ def test_build_entry_points_reject_bad_arguments_before_any_device_call():
     assert (p.enhance_search_batch, p.enhance_nap_batch, p.enhance_L, p.n_start) == (524288, 4096, 256, 16)
     with pytest.raises(TypeError):
         capi.build_params(no_such_field=1)
+
+
+def test_update_drivers_flag_handling():
+    for tool, required in (("update_compute_gt", ("--dist", "--dataset", "--base_data_path", "--query_path",
+                                                  "--update_gt_file", "--k", "--upd_mode", "--data_type")),
+                           ("test_update", ("--dataset", "--base_data_path", "--update_gt_file",
+                                            "--sampled_query_data_path", "--dist", "--data_type", "--recall_thres",
+                                            "--query_thres", "--max_degree", "--k", "--L", "--query_path", "--upd_mode",
+                                            "--config_file"))):  # tests/update_compute_gt.cpp:40-55, tests/test_update.cpp:42-74
+        exe = os.path.join(ROOT, "coral_amd", "lib", tool)
+        r = subprocess.run([exe, "--help"], capture_output=True, text=True)
+        assert r.returncode == 0
+        for flag in required:
+            assert flag in r.stdout, (tool, flag)
+        r = subprocess.run([exe, "--dataset", "t"], capture_output=True, text=True)
+        assert r.returncode == 255 and "required but missing" in r.stderr
+    exe = os.path.join(ROOT, "coral_amd", "lib", "update_compute_gt")
+    args = ["--dist", "l2", "--dataset", "t", "--base_data_path", "/nonexistent.fbin", "--query_path", "/q.fbin",
+            "--update_gt_file", "/tmp/x", "--k", "10"]
+    r = subprocess.run([exe] + args + ["--upd_mode", "2"], capture_output=True, text=True)
+    assert r.returncode == 255 and "upd_mode 1" in r.stderr
+    r = subprocess.run([exe] + args + ["--upd_mode", "1"], capture_output=True, text=True)
+    assert r.returncode == 1 and "open file error" in r.stderr
