@@ -48,8 +48,8 @@ __global__ __launch_bounds__(256) void distance_tile_kernel(const float* __restr
                                                            const uint32_t* __restrict__ deleted,
                                                            int64_t base_id0, float* __restrict__ D,
                                                            int64_t ldD) {
-    __shared__ float sq[KC][TQ + 4];
-    __shared__ float sb[KC][TB + 4];
+    __shared__ float sq2[2][KC][TQ + 4];
+    __shared__ float sb2[2][KC][TB + 4];
     const int tid = threadIdx.x;
     const int tx = tid & 15, ty = tid >> 4;  // thread (ty, tx) owns queries ty*8.. and base tx*8..
     const int64_t b0 = (int64_t)blockIdx.x * TB;
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void distance_tile_kernel(const float* __restr
         for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
 
     // staging: 128 rows x KC dims per operand = 32*KC float4, KC/8 per thread: thread t loads row t/2, dims
-    // (t&1)*4 + 8*u.  The loads of the next stage are issued before the arithmetic of the current one.
+    // (t&1)*4 + 8*u
     constexpr int NL = KC / 8;
     const int lrow = tid >> 1, lk = (tid & 1) * 4;
     float4 vq[NL], vb[NL];
@@ -76,41 +76,55 @@ __global__ __launch_bounds__(256) void distance_tile_kernel(const float* __restr
             }
         }
     };
-    fetch(0);
-    for (int k0 = 0; k0 < dim; k0 += KC) {
-        __syncthreads();
+    // two staging buffers, one barrier per stage: while a stage is consumed the next one is fetched into registers
+    // and parked in the other buffer
+    auto park = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < NL; ++u) {
             const int r = lk + 8 * u;
-            sq[r + 0][lrow] = vq[u].x, sq[r + 1][lrow] = vq[u].y, sq[r + 2][lrow] = vq[u].z, sq[r + 3][lrow] = vq[u].w;
-            sb[r + 0][lrow] = vb[u].x, sb[r + 1][lrow] = vb[u].y, sb[r + 2][lrow] = vb[u].z, sb[r + 3][lrow] = vb[u].w;
+            sq2[buf][r + 0][lrow] = vq[u].x, sq2[buf][r + 1][lrow] = vq[u].y, sq2[buf][r + 2][lrow] = vq[u].z, sq2[buf][r + 3][lrow] = vq[u].w;
+            sb2[buf][r + 0][lrow] = vb[u].x, sb2[buf][r + 1][lrow] = vb[u].y, sb2[buf][r + 2][lrow] = vb[u].z, sb2[buf][r + 3][lrow] = vb[u].w;
         }
+    };
+    auto consume = [&](int buf, int kk) {
+        float a[8], b[8];
+        const float4 a0 = *reinterpret_cast<const float4*>(&sq2[buf][kk][ty * 8]);
+        const float4 a1 = *reinterpret_cast<const float4*>(&sq2[buf][kk][ty * 8 + 4]);
+        const float4 c0 = *reinterpret_cast<const float4*>(&sb2[buf][kk][tx * 8]);
+        const float4 c1 = *reinterpret_cast<const float4*>(&sb2[buf][kk][tx * 8 + 4]);
+        a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
+        b[0] = c0.x, b[1] = c0.y, b[2] = c0.z, b[3] = c0.w, b[4] = c1.x, b[5] = c1.y, b[6] = c1.z, b[7] = c1.w;
+        if (metric == 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float t = a[i] - b[j];
+                    acc[i][j] = __fmaf_rn(t, t, acc[i][j]);
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
+        }
+    };
+    fetch(0);
+    park(0);
+    __syncthreads();
+    int cur = 0;
+    for (int k0 = 0; k0 < dim; k0 += KC) {
+        const bool more = k0 + KC < dim;
+        if (more) fetch(k0 + KC);
+        if (dim - k0 >= KC) {
+#pragma unroll
+            for (int kk = 0; kk < KC; ++kk) consume(cur, kk);
+        } else {
+            for (int kk = 0; kk < dim - k0; ++kk) consume(cur, kk);
+        }
+        if (more) park(cur ^ 1);
         __syncthreads();
-        if (k0 + KC < dim) fetch(k0 + KC);
-        const int kend = min(KC, dim - k0);
-        for (int kk = 0; kk < kend; ++kk) {
-            float a[8], b[8];
-            const float4 a0 = *reinterpret_cast<const float4*>(&sq[kk][ty * 8]);
-            const float4 a1 = *reinterpret_cast<const float4*>(&sq[kk][ty * 8 + 4]);
-            const float4 c0 = *reinterpret_cast<const float4*>(&sb[kk][tx * 8]);
-            const float4 c1 = *reinterpret_cast<const float4*>(&sb[kk][tx * 8 + 4]);
-            a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
-            b[0] = c0.x, b[1] = c0.y, b[2] = c0.z, b[3] = c0.w, b[4] = c1.x, b[5] = c1.y, b[6] = c1.z, b[7] = c1.w;
-            if (metric == 0) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float t = a[i] - b[j];
-                        acc[i][j] = __fmaf_rn(t, t, acc[i][j]);
-                    }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
-            }
-        }
+        cur ^= 1;
     }
     const float inf = __int_as_float(0x7f800000);
 #pragma unroll
