@@ -15,6 +15,11 @@
  *     (DistanceL2::compare), comparisons include/utils.cuh:368-386 and the
  *     sentinels of include/uni.h:65-68
  *   - recall: tests/test_search_pipeline.cpp:25-39; normalisation src/uni.cpp:38-54
+ *   - exact kNN by brute force under (distance, id), in fp64 or in one of the fp32 orders above: what the
+ *     reference asks faiss for (tests/comp_gt.cpp:119-176, src/knn.cu:174-193)
+ *   - entry points by farthest-point sampling in hop distance: src/start.cu:10-145
+ *   - graph construction: one batch of neighbour-aware pruning (src/upd_gpu.cu:12-303) and one batch of the
+ *     connectivity enhancement (src/enhance.cu:131-208, 334-575, 660-689); see the section further down
  *
  * Pinning status (what fixes each function besides this text):
  *   - oracle_dist ORDER_CPU_AVX512, oracle_queue_*, oracle_search_A: bit-exact
@@ -32,6 +37,10 @@
  *     exit; equality with exact kNN on complete graphs and when L >= N;
  *     hand-computed traversals on path/ring graphs; an independent
  *     set-based pure-Python simulator on tiny inputs.
+ *   - oracle_bruteforce*: fp64 closed form, exact lattice cases with ties, top-k of a full sort.
+ *   - oracle_fps, oracle_nap_batch, oracle_enhance_batch: no executable reference (CUDA, faiss, outcomes that
+ *     depend on thread timing).  Pinned by code reading, hand-computed cases, the invariants of the occlusion
+ *     rule, an all-pairs brute force (FPS) and independent pure-Python statements on small random inputs.
  *
  * Graph rows are the compact form used on the device: int32 nbrs[N][R] where
  * a row's neighbours are its leading non-negative entries (deg = index of the
