@@ -114,6 +114,9 @@ class CORAL_API IndexGPU {
     void Delete(const std::vector<int> del_ids);
 
     // --- beyond the reference ---
+    // CORAL_POLICY_BEST_FIRST is the traversal of GPUFuncs::search_in_cpu; it starts from every start id of the index,
+    // where the CPU path takes the first search_start_nodes_num of them (src/search_in_cpu.cpp:26, 74-79): the same
+    // set whenever graph.search_start_ids holds that many ids, as the builder writes it
     void SetPolicy(int coral_policy) { policy_ = coral_policy; }
     // tombstones (src/update.cu:406-412): ceil(n/32) words, or nullptr to clear
     void SetDeleted(const uint32_t* mask_words);
