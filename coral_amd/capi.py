@@ -40,7 +40,7 @@ class Stats(C.Structure):
 
 class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
-                ("policy", C.c_int32), ("reserved", C.c_int32 * 4)]
+                ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("reserved", C.c_int32 * 3)]
 
 
 class BuildParams(C.Structure):
@@ -188,8 +188,8 @@ class Index:
         _check(lib().coral_index_get_deleted(self._h, _ptr(m)))
         return m
 
-    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS):
-        t = Tuning(visited_slots_log2, workgroups, threads, policy)
+    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False):
+        t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)))
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

@@ -36,6 +36,21 @@ struct SearchArgs {
     int32_t tcap, ccap;        // LDS todo / candidate capacities (multiples of 4, ccap >= tcap)
 };
 
+// What the wavefront-per-query best-first kernel (best_first.hip) needs beyond SearchArgs.
+struct BestFirstArgs {
+    uint8_t* visited;   // [slots][stride]: the epoch of the query that last visited the node, 0 = never
+    uint32_t* epochs;   // [slots]: last epoch used by the slot (kept across launches)
+    size_t stride;      // bytes per slot: n rounded up to a multiple of 16
+    int32_t slots;      // wavefronts = queries in flight
+};
+
+// LDS bytes of one wavefront: two beams of L keys, 64 candidate keys, 64 ids
+__host__ __device__ inline size_t best_first_wave_lds_bytes(int L) {
+    return (size_t)((L + 3) & ~3) * 16 + 64 * 8 + 64 * 4;
+}
+hipError_t best_first_prepare(int dim, int L, int* max_wg_per_cu);
+hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
+
 size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap, int ocap);
 hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu);
 hipError_t launch_search(const SearchArgs& a, int workgroups, int threads, size_t lds_bytes,

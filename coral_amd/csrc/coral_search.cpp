@@ -155,6 +155,8 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_scalars);
     (void)hipFree(idx->d_hit);
     (void)hipFree(idx->d_phase);
+    (void)hipFree(idx->d_bf_visited);
+    (void)hipFree(idx->d_bf_epochs);
     coral::free_build_state(idx);
     if (idx->h_counters) (void)hipHostFree(idx->h_counters);
     if (idx->stream) (void)hipStreamDestroy(idx->stream);
@@ -294,6 +296,34 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         HIP_TRY(hipHostMalloc(&idx->h_counters, need_counters * sizeof(int32_t)));
         idx->counters_alloc = need_counters;
     }
+    // Best-first: one wavefront per query with the visited state in HBM (best_first.hip), when the memory for it
+    // is there: n bytes per wavefront, up to a third of what is free and 64 GiB.
+    idx->bf_ready = false;
+    if (best_first && !t.best_first_in_lds) {
+        int bf_wg_per_cu = 0;
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, &bf_wg_per_cu));
+        const size_t stride = ((size_t)idx->n + 15) & ~(size_t)15;
+        size_t free_b = 0, total_b = 0;
+        HIP_TRY(hipMemGetInfo(&free_b, &total_b));
+        const size_t budget = std::min<size_t>((free_b + idx->bf_alloc_bytes) / 3, (size_t)64 << 30);
+        int64_t want = t.workgroups > 0 ? (int64_t)t.workgroups * 4 : (int64_t)bf_wg_per_cu * idx->num_cu * 4;
+        int slots = (int)std::min<int64_t>(want, (int64_t)Q);
+        slots = (int)std::min<size_t>((size_t)slots, budget / stride);
+        if (bf_wg_per_cu > 0 && (slots >= 256 || slots >= Q || t.workgroups > 0) && slots > 0) {
+            if (stride != idx->bf_stride || slots > idx->bf_alloc_slots) {
+                (void)hipFree(idx->d_bf_visited), (void)hipFree(idx->d_bf_epochs);
+                idx->d_bf_visited = nullptr, idx->d_bf_epochs = nullptr;
+                idx->bf_alloc_slots = 0, idx->bf_alloc_bytes = 0, idx->bf_stride = 0;
+                HIP_TRY(hipMalloc(&idx->d_bf_visited, stride * (size_t)slots));
+                HIP_TRY(hipMalloc(&idx->d_bf_epochs, (size_t)slots * sizeof(uint32_t)));
+                HIP_TRY(hipMemsetAsync(idx->d_bf_visited, 0, stride * (size_t)slots, idx->stream));
+                HIP_TRY(hipMemsetAsync(idx->d_bf_epochs, 0, (size_t)slots * sizeof(uint32_t), idx->stream));
+                idx->bf_stride = stride, idx->bf_alloc_slots = slots, idx->bf_alloc_bytes = stride * (size_t)slots;
+            }
+            idx->bf_slots = slots;
+            idx->bf_ready = true;
+        }
+    }
     HIP_TRY(hipStreamSynchronize(idx->stream));
     idx->Q = Q, idx->L = L, idx->slots_log2 = slots_log2, idx->vis_limit = vis_limit;
     idx->tcap = tcap, idx->ccap = tcap, idx->threads = threads, idx->workgroups = workgroups;
@@ -345,8 +375,15 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
 #endif
     // timed region, same scope as the reference: kernel + counter read-back
     HIP_TRY(hipEventRecord(ev0, stream));
-    const int wgs = std::min(idx->workgroups, (int)Q);
-    HIP_TRY(coral::launch_search(a, wgs, idx->threads, idx->lds_bytes, stream));
+    if (policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready) {
+        coral::BestFirstArgs b;
+        b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
+        b.slots = std::min(idx->bf_slots, (int)Q);
+        HIP_TRY(coral::launch_best_first(a, b, stream));
+    } else {
+        const int wgs = std::min(idx->workgroups, (int)Q);
+        HIP_TRY(coral::launch_search(a, wgs, idx->threads, idx->lds_bytes, stream));
+    }
     HIP_TRY(hipEventRecord(evk, stream));
     HIP_TRY(hipMemcpyAsync(idx->h_counters, idx->d_counters, (size_t)Q * 4 * sizeof(int32_t),
                            hipMemcpyDeviceToHost, stream));

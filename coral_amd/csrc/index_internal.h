@@ -45,6 +45,13 @@ struct coral_index {
     int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
     int last_Q = 0;
 
+    // best-first on one wavefront per query: per-slot visited epochs in global memory
+    bool bf_ready = false;
+    uint8_t* d_bf_visited = nullptr;
+    uint32_t* d_bf_epochs = nullptr;
+    size_t bf_stride = 0, bf_alloc_bytes = 0;
+    int bf_slots = 0, bf_alloc_slots = 0;
+
     // graph construction (coral_build_*): per-neighbour distances, degrees, the per-batch claim table
     // (INT_MAX when idle) and the staging rows of one batch
     bool building = false;

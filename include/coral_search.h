@@ -92,11 +92,16 @@ typedef struct {
 /* Optional launch tuning; zero-initialise for defaults. */
 typedef struct {
     int32_t visited_slots_log2; /* LDS visited table: log2 of its 16-bit cells, 10..16; 0 = chosen from L */
-    int32_t workgroups;         /* persistent workgroups; 0 = chosen from Q and the device */
+    int32_t workgroups;         /* persistent workgroups (of four query slots each on the wavefront-per-query
+                                   best-first kernel); 0 = chosen from Q and the device */
     int32_t threads;            /* threads per workgroup: 128, 256, 512 or 1024; 0 = chosen from the LDS need */
     int32_t policy;             /* the policy the scratch is sized for (CORAL_POLICY_*); best-first visits
                                    fewer nodes per beam entry and works on one graph row at a time */
-    int32_t reserved[4];
+    int32_t best_first_in_lds;  /* best-first normally runs one wavefront per query with a byte of visited state
+                                   per node and query slot in HBM (n bytes x up to 4096 slots); 1 keeps it on the
+                                   workgroup-per-query kernel with the visited set in LDS, as it also does by
+                                   itself when that memory is not to be had */
+    int32_t reserved[3];
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);

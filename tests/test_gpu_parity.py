@@ -70,22 +70,59 @@ def test_exact_against_same_order_oracle(orc, case):
                                  isolate=5 if rg else 0)
     q = make_queries(150, dim, 300 + dim, metric)
     print("case", case, flush=True)
-    idx = capi.Index(base, nbrs, starts, m)
-    idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy)
-    ids, dists, st = idx.search(q, k, L, policy=policy)
-    cnt = idx.query_counters(q.shape[0])
-    idx.close()
     prob = orc.Problem(base, nbrs, starts)
     if policy == 0:
         oi, od, os_, _ = orc.search_B(prob, q, k, L, metric=m, start_order=WAVE64, nbr_order=WAVE64)
     else:
         oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=m, order=WAVE64)
-    assert np.array_equal(ids, oi)
-    assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist()
-    assert np.array_equal(cnt, os_)
-    assert st.hops == int(os_[:, 0].sum()) and st.dist_evals == int(os_[:, 2].sum())
-    if slots == 11:
-        assert st.spills > 0
+    idx = capi.Index(base, nbrs, starts, m)
+    # best-first has two kernels: a wavefront per query (visited bytes in HBM) and a workgroup per query (LDS table)
+    for in_lds in ((False, True) if policy == 1 else (False,)):
+        idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy,
+                    best_first_in_lds=in_lds)
+        ids, dists, st = idx.search(q, k, L, policy=policy)
+        cnt = idx.query_counters(q.shape[0])
+        assert np.array_equal(ids, oi)
+        assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist()
+        assert np.array_equal(cnt, os_)
+        assert st.hops == int(os_[:, 0].sum()) and st.dist_evals == int(os_[:, 2].sum())
+        if slots == 11 and (policy == 0 or in_lds):
+            assert st.spills > 0
+    idx.close()
+
+
+def test_best_first_query_slots_are_reused(orc):
+    """The wavefront-per-query kernel keeps one byte of visited state per node and query slot and tells queries
+    apart by an epoch that wraps at 256: eight slots serve 2400 queries (300 each), twice, on a graph whose rows
+    repeat ids and with tombstones, and every answer and counter equals the oracle's."""
+    n, dim, R, L, k = 5000, 64, 16, 48, 20
+    base, nbrs, starts = problem(n, dim, R, seed=31, n_start=5, ragged_seed=9)
+    rng = np.random.RandomState(12)
+    rows = rng.choice(n, 1500, replace=False)
+    rows = rows[nbrs[rows, 7] >= 0]        # rows end at their first -1
+    nbrs[rows, 7] = nbrs[rows, 2]          # an id listed twice in a row
+    nbrs[rows[:500], 3] = nbrs[rows[:500], 2]
+    assert len(rows) > 600
+    mask = synth.tombstone_mask(n, 77, modulo=5)
+    q = make_queries(2400, dim, 41)
+    prob = orc.Problem(base, nbrs, starts, mask)
+    oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
+    idx = capi.Index(base, nbrs, starts)
+    idx.set_deleted(mask)
+    idx.prepare(q.shape[0], L, workgroups=2, policy=1)
+    for rep in range(2):
+        print("slot reuse pass", rep, flush=True)
+        ids, dists, st = idx.search(q, k, L, policy=1, have_delete=True)
+        cnt = idx.query_counters(q.shape[0])
+        assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(cnt, os_)
+        assert st.spills == 0
+    # fewer queries than slots, and the other kernel on the same index afterwards
+    ids, dists, _ = idx.search(q[:3], k, L, policy=1, have_delete=True)
+    assert np.array_equal(ids, oi[:3])
+    idx.prepare(q.shape[0], L, policy=1, best_first_in_lds=True)
+    ids, dists, _ = idx.search(q[:200], k, L, policy=1, have_delete=True)
+    assert np.array_equal(ids, oi[:200]) and dists.tobytes() == od[:200].tobytes()
+    idx.close()
 
 
 @pytest.mark.parametrize("metric,policy,dim,L,k", [("l2", 0, 200, 256, 100), ("l2", 0, 128, 64, 10),
