@@ -128,6 +128,8 @@ def main():
     if best_first:
         out["best_first"] = {k2: best_first[k2] for k2 in ("L", "qps", "recall", "kernel_ms", "gbps",
                                                            "dist_evals_per_query", "expansions_per_query")}
+        out["best_first"]["kernel"] = "best_first_wave_kernel"
+        out["best_first"]["frac"] = best_first["gbps"] / HBM_PEAK_GBPS
 
     # the IndexGPU::Search shape: host buffers in and out (device allocation, query upload,
     # search, id download); reported beside the headline, never as the headline

@@ -42,13 +42,14 @@ struct BestFirstArgs {
     uint32_t* epochs;   // [slots]: last epoch used by the slot (kept across launches)
     size_t stride;      // bytes per slot: n rounded up to a multiple of 16
     int32_t slots;      // wavefronts = queries in flight
+    int32_t rows_in_flight;  // 8 or 16: float4 registers of vector data a lane requests before it adds them up
 };
 
 // LDS bytes of one wavefront: two beams of L keys, 64 candidate keys, 64 ids
 __host__ __device__ inline size_t best_first_wave_lds_bytes(int L) {
     return (size_t)((L + 3) & ~3) * 16 + 64 * 8 + 64 * 4;
 }
-hipError_t best_first_prepare(int dim, int L, int* max_wg_per_cu);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, int* max_wg_per_cu);
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 
 size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap, int ocap);

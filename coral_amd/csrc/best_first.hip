@@ -5,11 +5,12 @@
 // measure the new ones, insert them, pick the closest entry not yet expanded.  Every step is a chain of dependent
 // memory accesses; what makes it fast on this GPU is how many such chains run side by side.  A workgroup per query
 // with the visited set in LDS (the form beam_search.hip gives this policy) holds two queries per CU.  Here a query
-// needs one wavefront and 9 KB of LDS (its sorted beam, twice, for the merge): sixteen queries per CU.  The visited
-// set moves to global memory in the form the CPU path itself uses (src/search_in_cpu.cpp:44-48, 68-71): one byte per
-// node and per query slot holding the epoch of the query that last visited the node, so nothing is cleared between
-// queries (every 255th query of a slot wipes its array).  With 288 GB of HBM four thousand such arrays are cheap
-// (4 GB at a million nodes).
+// needs one wavefront and 9 KB of LDS at L = 512 (its sorted beam, twice, for the merge): sixteen queries per CU,
+// enough to keep HBM busy (2.4 times the throughput of the other form at a million nodes).  The visited set moves to
+// global memory in the form the CPU path itself uses (src/search_in_cpu.cpp:44-48, 68-71): one byte per node and
+// query slot holding the epoch of the query that last visited the node, so nothing is cleared between queries
+// (every 255th query of a slot wipes its array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a
+// million nodes); each test costs a 128-byte line of HBM traffic, about a sixth of what the vectors cost.
 //
 // The arithmetic is that of beam_search.hip (same lane-strided accumulation, same butterfly, same 64-bit keys), so
 // results and counters are identical bit for bit; a wavefront needs no workgroup barrier anywhere.
@@ -32,8 +33,8 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int G, int CPL>
-__global__ __launch_bounds__(kWavesPerWg * 64) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
+template <int G, int CPL, int RIF>
+__global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = blockIdx.x * kWavesPerWg + wave;
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64) void best_first_wave_kernel(const
     uint32_t epoch = b.epochs[slot];
 
     constexpr int GPW = 64 / G;                    // row groups per wavefront
-    constexpr int U = (CPL >= 8) ? 1 : (8 / CPL);  // rows in flight per group
+    constexpr int U = (CPL >= RIF) ? 1 : (RIF / CPL);  // rows in flight per group
     constexpr int RPI = GPW * U;                   // rows per iteration
     const int gl = lane & (G - 1), grp = lane / G;
 
@@ -233,8 +234,10 @@ __global__ __launch_bounds__(kWavesPerWg * 64) void best_first_wave_kernel(const
             nd += T;
             wave_sync();
             measure_and_merge(T);
-            // the tags written in this step are read by later steps of this wavefront through other lanes: they must
-            // have reached L2 (where the tag loads go) before the next row is tested
+            // The tags written in this step are read by later steps of this wavefront through other lanes.  Tag loads
+            // and stores are agent-scope atomics, so both go to L2 past the CU's cache; the fence makes the wavefront
+            // wait for its stores to be acknowledged before it issues the next step's loads.  (A fence of agent scope
+            // would also write the whole L2 back each step, which no other wavefront needs: slots are private.)
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         }
 
@@ -286,21 +289,27 @@ __global__ __launch_bounds__(kWavesPerWg * 64) void best_first_wave_kernel(const
 
 using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 
-bf_kernel_fn pick_bf_kernel(int dim) {
-    const int chunks = dim / 4;
-    if (chunks <= 16) return best_first_wave_kernel<16, 1>;
-    if (chunks <= 32) return best_first_wave_kernel<32, 1>;
-    if (chunks <= 64) return best_first_wave_kernel<64, 1>;
-    if (chunks <= 128) return best_first_wave_kernel<64, 2>;
-    if (chunks <= 256) return best_first_wave_kernel<64, 4>;
-    if (chunks <= 512) return best_first_wave_kernel<64, 8>;
+// RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
+// dependent memory waits of a step against 8 and needs 128 registers
+template <int RIF>
+bf_kernel_fn pick_bf_kernel_rif(int chunks) {
+    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF>;
+    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF>;
+    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF>;
+    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF>;
+    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF>;
+    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF>;
     return nullptr;
+}
+
+bf_kernel_fn pick_bf_kernel(int dim, int rif) {
+    return rif >= 16 ? pick_bf_kernel_rif<16>(dim / 4) : pick_bf_kernel_rif<8>(dim / 4);
 }
 
 }  // namespace
 
-hipError_t best_first_prepare(int dim, int L, int* max_wg_per_cu) {
-    bf_kernel_fn fn = pick_bf_kernel(dim);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, int* max_wg_per_cu) {
+    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight);
     if (!fn) return hipErrorInvalidValue;
     const size_t lds = best_first_wave_lds_bytes(L) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -314,7 +323,7 @@ hipError_t best_first_prepare(int dim, int L, int* max_wg_per_cu) {
 }
 
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream) {
-    bf_kernel_fn fn = pick_bf_kernel(a.dim);
+    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_wave_lds_bytes(a.L) * kWavesPerWg, stream, a, b);

@@ -301,7 +301,11 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     idx->bf_ready = false;
     if (best_first && !t.best_first_in_lds) {
         int bf_wg_per_cu = 0;
-        HIP_TRY(coral::best_first_prepare(idx->dim, L, &bf_wg_per_cu));
+        // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling
+        const int chunks = idx->dim / 4;
+        const int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
+        idx->bf_rows_in_flight = rif;
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, &bf_wg_per_cu));
         const size_t stride = ((size_t)idx->n + 15) & ~(size_t)15;
         size_t free_b = 0, total_b = 0;
         HIP_TRY(hipMemGetInfo(&free_b, &total_b));
@@ -309,7 +313,8 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         int64_t want = t.workgroups > 0 ? (int64_t)t.workgroups * 4 : (int64_t)bf_wg_per_cu * idx->num_cu * 4;
         int slots = (int)std::min<int64_t>(want, (int64_t)Q);
         slots = (int)std::min<size_t>((size_t)slots, budget / stride);
-        if (bf_wg_per_cu > 0 && (slots >= 256 || slots >= Q || t.workgroups > 0) && slots > 0) {
+        // below about four wavefronts per CU the workgroup-per-query kernel is the faster one
+        if (bf_wg_per_cu > 0 && (slots >= 4 * idx->num_cu || slots >= Q || t.workgroups > 0) && slots > 0) {
             if (stride != idx->bf_stride || slots > idx->bf_alloc_slots) {
                 (void)hipFree(idx->d_bf_visited), (void)hipFree(idx->d_bf_epochs);
                 idx->d_bf_visited = nullptr, idx->d_bf_epochs = nullptr;
@@ -379,6 +384,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         coral::BestFirstArgs b;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
+        b.rows_in_flight = idx->bf_rows_in_flight;
         HIP_TRY(coral::launch_best_first(a, b, stream));
     } else {
         const int wgs = std::min(idx->workgroups, (int)Q);

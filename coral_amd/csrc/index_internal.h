@@ -50,7 +50,7 @@ struct coral_index {
     uint8_t* d_bf_visited = nullptr;
     uint32_t* d_bf_epochs = nullptr;
     size_t bf_stride = 0, bf_alloc_bytes = 0;
-    int bf_slots = 0, bf_alloc_slots = 0;
+    int bf_slots = 0, bf_alloc_slots = 0, bf_rows_in_flight = 8;
 
     // graph construction (coral_build_*): per-neighbour distances, degrees, the per-batch claim table
     // (INT_MAX when idle) and the staging rows of one batch
