@@ -315,18 +315,27 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         slots = (int)std::min<size_t>((size_t)slots, budget / stride);
         // below about four wavefronts per CU the workgroup-per-query kernel is the faster one
         if (bf_wg_per_cu > 0 && (slots >= 4 * idx->num_cu || slots >= Q || t.workgroups > 0) && slots > 0) {
-            if (stride != idx->bf_stride || slots > idx->bf_alloc_slots) {
+            bool have = stride == idx->bf_stride && slots <= idx->bf_alloc_slots;
+            if (!have) {
                 (void)hipFree(idx->d_bf_visited), (void)hipFree(idx->d_bf_epochs);
                 idx->d_bf_visited = nullptr, idx->d_bf_epochs = nullptr;
                 idx->bf_alloc_slots = 0, idx->bf_alloc_bytes = 0, idx->bf_stride = 0;
-                HIP_TRY(hipMalloc(&idx->d_bf_visited, stride * (size_t)slots));
-                HIP_TRY(hipMalloc(&idx->d_bf_epochs, (size_t)slots * sizeof(uint32_t)));
-                HIP_TRY(hipMemsetAsync(idx->d_bf_visited, 0, stride * (size_t)slots, idx->stream));
-                HIP_TRY(hipMemsetAsync(idx->d_bf_epochs, 0, (size_t)slots * sizeof(uint32_t), idx->stream));
-                idx->bf_stride = stride, idx->bf_alloc_slots = slots, idx->bf_alloc_bytes = stride * (size_t)slots;
+                // a refused allocation is no error: the workgroup-per-query kernel serves the policy then
+                hipError_t e = hipMalloc(&idx->d_bf_visited, stride * (size_t)slots);
+                if (e == hipSuccess) e = hipMalloc(&idx->d_bf_epochs, (size_t)slots * sizeof(uint32_t));
+                if (e == hipSuccess) {
+                    HIP_TRY(hipMemsetAsync(idx->d_bf_visited, 0, stride * (size_t)slots, idx->stream));
+                    HIP_TRY(hipMemsetAsync(idx->d_bf_epochs, 0, (size_t)slots * sizeof(uint32_t), idx->stream));
+                    idx->bf_stride = stride, idx->bf_alloc_slots = slots;
+                    idx->bf_alloc_bytes = stride * (size_t)slots;
+                    have = true;
+                } else {
+                    (void)hipGetLastError();
+                    (void)hipFree(idx->d_bf_visited);
+                    idx->d_bf_visited = nullptr;
+                }
             }
-            idx->bf_slots = slots;
-            idx->bf_ready = true;
+            if (have) idx->bf_slots = slots, idx->bf_ready = true;
         }
     }
     HIP_TRY(hipStreamSynchronize(idx->stream));

@@ -59,6 +59,12 @@ CASES = [
     (20000, 128, 32, "l2", 1, 128, 100, 1, 7, 0, 0),
     (12000, 512, 32, "ip", 1, 64, 10, 16, None, 0, 0),
     (20000, 200, 32, "l2", 1, 128, 16, 16, None, 11, 0),
+    (12000, 64, 32, "l2", 1, 128, 20, 16, None, 0, 0),      # best-first at every vector-width variant
+    (12000, 256, 24, "ip", 1, 96, 32, 8, 5, 0, 0),
+    (6000, 1024, 16, "l2", 1, 64, 10, 4, None, 0, 0),
+    (6000, 2048, 8, "ip", 1, 32, 8, 2, None, 0, 0),
+    (20000, 128, 32, "l2", 1, 160, 50, 100, None, 0, 0),    # more start ids than a wavefront measures at a time
+    (20000, 200, 32, "l2", 1, 1024, 100, 16, None, 0, 0),   # a long beam
 ]
 
 
