@@ -6,10 +6,13 @@
 //   --query_test_file --gt_test_file --M_sq --M_pjbp --L_pjpq --num_threads/-T --CE --k --iso_thres
 //   --recall_thres --query_thres --log_file --config_file
 // --M_pjbp is the row width, --k the cluster size (nearest base points per sampled query).  --train_gt_file names
-// precomputed clusters (a ground-truth file of the sampled queries with k ids per row).  --query_test_file /
-// --gt_test_file (searches during the build) and the knn cache are not provided: naming a test file is an error.
+// precomputed clusters (a ground-truth file of the sampled queries with k ids per row).  --query_test_file with
+// --gt_test_file: the reference searches these queries with beam test_beam_capacity when the graph is complete and
+// logs recall and hops (src/index_gpu.cpp:376-378, include/gpufuncs.cuh:688-702); so does this driver, on stdout.
+// The knn cache is not provided.
 // Extensions: --index_dir <dir> (overrides the derived <index_prefix><dataset>_<dist>_<R>_<thres>_<CE> path) and
 // --index_prefix (default ../indexes/).
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -92,8 +95,9 @@ int main(int argc, char** argv) {
         std::cerr << "only --data_type float is provided\n";
         return -1;
     }
-    if (str("query_test_file") != "None" || str("gt_test_file") != "None") {
-        std::cerr << "--query_test_file / --gt_test_file are not provided: run test_search_pipeline on the result\n";
+    const bool test_search = str("query_test_file") != "None";
+    if (test_search != (str("gt_test_file") != "None")) {
+        std::cerr << "--query_test_file and --gt_test_file go together\n";
         return -1;
     }
     std::cout << "sampled query: " << str("sampled_query_data_path") << std::endl;
@@ -155,6 +159,26 @@ int main(int argc, char** argv) {
                   << std::endl;
         std::cout << "indexing time: " << diff.count() << std::endl;
         std::cout << "Save index to " << graph_file << std::endl;
+        if (test_search) {
+            int64_t q_num = 0;
+            int32_t q_stride = 0, gt_num = 0, gt_dim = 0;
+            std::vector<float> queries = load_padded(str("query_test_file"), &q_num, &q_stride);
+            if (q_stride != base_stride) throw std::runtime_error("base and test-query dimensions differ");
+            if (dist_metric == efanna2e::INNER_PRODUCT) coral_normalize_l2(queries.data(), q_num, q_stride);
+            if (coral_gt_read_meta(str("gt_test_file").c_str(), &gt_num, &gt_dim))
+                throw std::runtime_error(coral_last_error());
+            if (gt_num < q_num || gt_dim < k) throw std::runtime_error("test ground truth smaller than queries x k");
+            std::vector<int> gt((size_t)gt_num * gt_dim), gt_k((size_t)q_num * k);
+            if (coral_gt_read(str("gt_test_file").c_str(), gt.data(), gt_num, gt_dim))
+                throw std::runtime_error(coral_last_error());
+            for (int64_t q = 0; q < q_num; ++q)  // the device count takes rows k apart (src/index_gpu.cpp:96-98)
+                std::copy_n(gt.data() + (size_t)q * gt_dim, k, gt_k.data() + (size_t)q * k);
+            const int L = std::max(PC.test_beam_capacity, k);
+            Test_Result tr = index.Search_and_Verify(queries.data(), gt_k.data(), (int)q_num, L);
+            std::cout << "test search: L " << L << ", recall@" << k << " " << tr.calc_recall((int)q_num * k)
+                      << " %, avg hops " << tr.avg_hops((int)q_num) << ", QPS " << (double)q_num / tr.get_time()
+                      << std::endl;
+        }
     } catch (const std::exception& ex) {
         std::cerr << ex.what() << std::endl;
         return 1;

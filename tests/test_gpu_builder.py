@@ -235,7 +235,10 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     cli = os.path.join(root, "coral_amd", "lib", "test_build_pipeline")
     args = [cli, "--data_type", "float", "--dist", "l2", "--dataset", "syn", "--base_data_path", str(work / "base.fbin"),
             "--sampled_query_data_path", str(work / "aux.fbin"), "--M_pjbp", "16", "--k", "24", "--CE", "1",
-            "--query_thres", "1.0", "--config_file", str(work / "config.json"), "-T", "8"]
+            "--query_thres", "1.0", "--config_file", str(work / "config.json"), "-T", "8",
+            "--query_test_file", str(work / "query.fbin"), "--gt_test_file", str(work / "gt24.bin")]
+    gt24, _ = orc.bruteforce(base, q, 24)
+    formats.gt_write(work / "gt24.bin", gt24)
     r = subprocess.run(args, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr + r.stdout
     index_dir = work / "indexes" / "syn_l2_16_1.0_1"  # ../indexes/<dataset>_<dist>_<R>_<thres>_<CE>
@@ -251,6 +254,12 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     assert np.array_equal(nbrs, want_nbrs) and dists.tobytes() == want_dists.tobytes()
     assert starts.tolist() == want_starts.tolist() and len(starts) == 8
     assert (deg > 0).all()
+    # the search the build driver ran on the finished graph (test_beam_capacity = 512, k = the cluster size)
+    line = [l for l in r.stdout.splitlines() if l.startswith("test search:")][0]
+    o24, _, os24, _ = orc.search_B(orc.Problem(base, nbrs, starts), q, 24, 512, start_order=WAVE64, nbr_order=WAVE64)
+    assert "L 512, recall@24 " in line
+    assert abs(float(line.split("recall@24 ")[1].split(" %")[0]) - 100.0 * orc.recall_hits(o24, gt24, 24) / (Q * 24)) < 1e-3
+    assert abs(float(line.split("avg hops ")[1].split(",")[0]) - os24[:, 0].sum() / Q) < 1e-2
     # and the search driver on that directory
     cli = os.path.join(root, "coral_amd", "lib", "test_search_pipeline")
     args = [cli, "--data_type", "float", "--dist", "l2", "--base_data_path", str(work / "base.fbin"), "--dataset",
