@@ -55,6 +55,32 @@ def config2(n=1000000, dim=200, Q=10000, A=100000, device="cuda", verbose=False)
                 Ls=(256, 512), build=info)
 
 
+def structured(n=1000000, dim=200, latent=16, Q=10000, A=100000, noise=0.1, seed=6001):
+    """Data with neighbourhood structure, unlike the isotropic configurations: points near a `latent`-dimensional
+    subspace of R^dim (x = z P + noise * e, z ~ N(0, I_latent), P a fixed latent x dim Gaussian matrix scaled to unit
+    column variance, e ~ N(0, I_dim)); base, queries and auxiliary queries follow the same law.  Same graph
+    construction and k as configuration 2.  Not a configuration of the benchmark: it shows what beam the graph
+    search needs for recall@100 >= 0.90 when the data lets a degree-32 graph work."""
+    proj = (synth.gaussian_matrix(seed, latent, dim) / np.sqrt(latent)).astype(np.float32)
+
+    def draw(count, seed_z, seed_e):
+        out = gaussian_base(seed_e, count, dim)
+        out *= np.float32(noise)
+        step = 1 << 16
+        for r in range(0, count, step):
+            z = synth.gaussian_matrix(seed_z, min(step, count - r), latent, row0=r)
+            out[r:r + step] += z @ proj
+        return out
+
+    base = draw(n, seed + 1, seed + 2)
+    queries = draw(Q, seed + 3, seed + 4)
+    aux = draw(A, seed + 5, seed + 6)
+    nbrs, starts, info = build_query_aware_graph(base, aux, "l2")
+    return dict(name="%dx%d fp32 L2 near a %d-dimensional subspace, R=32 query-aware graph (k_b=100, %d aux queries), "
+                     "%d queries, k=100" % (n, dim, latent, A, Q), base=base, queries=queries, nbrs=nbrs,
+                starts=starts, metric="l2", k=100, Ls=(128, 256, 512), build=info)
+
+
 def config3(n=1000000, dim=512, Q=10000, A=100000, device="cuda", verbose=False):
     """Inner product: unit-normalised 1M x 512 base, cone-gap queries, k=100, L=256."""
     base = synth.normalize_rows(gaussian_base(3001, n, dim))
