@@ -241,6 +241,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         // (best-first: about 31 first visits per entry, 48 cells)
         slots_log2 = 12;
         while ((1 << slots_log2) < (best_first ? 48 : 112) * L && slots_log2 < 16) ++slots_log2;
+        if (idx->bump_L == L) slots_log2 = std::min(16, slots_log2 + idx->bump_log2);  // see coral_search_gpu
         while (slots_log2 > 12 &&
                coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap) + 64 > (size_t)kMaxLdsBytes)
             --slots_log2;
@@ -343,6 +344,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     idx->tcap = tcap, idx->ccap = tcap, idx->threads = threads, idx->workgroups = workgroups;
     idx->id_bits = id_bits, idx->rem_bits = rem_bits, idx->dmax = dmax, idx->ocap = ocap;
     idx->prepared_policy = t.policy;
+    idx->tuning = t;
     idx->lds_bytes = lds, idx->spill_words = spill_words;
     idx->prepared = true;
     return CORAL_OK;
@@ -425,6 +427,20 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     }
 #endif
     idx->last_Q = Q;
+    // The table size the library picks assumes about 75 first visits per beam entry.  Data on which a query visits
+    // more sends queries to the global bitmap (same results, slower): when more than a twentieth of a batch went
+    // there, the next launches get a table twice the size.
+    const bool lds_table = !(policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready);
+    if (lds_table && idx->tuning.visited_slots_log2 == 0 && (int64_t)scal[1] * 20 > Q && idx->slots_log2 < 16) {
+        const int had = idx->slots_log2;
+        idx->bump_log2 = idx->bump_L == idx->L ? idx->bump_log2 + 1 : 1;
+        idx->bump_L = idx->L;
+        coral_tuning t = idx->tuning;
+        if (coral_search_prepare(idx, idx->Q, idx->L, &t) != CORAL_OK || idx->slots_log2 == had) {
+            idx->bump_log2 -= 1;  // no room in LDS for more: stay
+            if (!idx->prepared) return fail(CORAL_ERR_DEVICE, "could not restore the search scratch");
+        }
+    }
     if (stats) {
         std::memset(stats, 0, sizeof *stats);
         stats->time_s = ms / 1000.0;

@@ -51,6 +51,10 @@ struct coral_index {
     uint32_t* d_bf_epochs = nullptr;
     size_t bf_stride = 0, bf_alloc_bytes = 0;
     int bf_slots = 0, bf_alloc_slots = 0, bf_rows_in_flight = 8;
+    // the tuning of the last prepare, and what the searches since have taught about the visited table:
+    // at beam capacity bump_L the library's own choice of table size is raised by bump_log2
+    coral_tuning tuning{};
+    int bump_L = 0, bump_log2 = 0;
 
     // graph construction (coral_build_*): per-neighbour distances, degrees, the per-batch claim table
     // (INT_MAX when idle) and the staging rows of one batch

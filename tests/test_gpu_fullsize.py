@@ -63,3 +63,26 @@ def test_full_size_properties(orc):
     assert fps.tolist() == orc.fps(nbrs, int(starts[0]), 16).tolist()
     assert len(set(fps.tolist())) == 16
     idx.close()
+
+
+def test_visited_table_grows_when_batches_outgrow_it():
+    """The LDS visited table is sized for about 75 first visits per beam entry.  On the structured 1M x 200 workload
+    a query at L = 128 visits 88 per entry and four in ten queries continue on the global bitmap; the library then
+    doubles the table for the following launches (results are the same either way).  A size the caller names stays."""
+    from coral_amd import workloads
+    w = workloads.structured()
+    q, k, L = w["queries"], 100, 128
+    Q = q.shape[0]
+    idx = capi.Index(w["base"], w["nbrs"], w["starts"])
+    ids1, d1, st1 = idx.search(q, k, L)
+    ids2, d2, st2 = idx.search(q, k, L)
+    print("spills %d -> %d, kernel %.2f -> %.2f ms" % (st1.spills, st2.spills, 1e3 * st1.kernel_s, 1e3 * st2.kernel_s),
+          flush=True)
+    assert st1.spills > Q // 20 and st2.spills < Q // 20
+    assert np.array_equal(ids1, ids2) and d1.tobytes() == d2.tobytes()
+    assert st2.kernel_s < st1.kernel_s
+    idx.prepare(Q, L, visited_slots_log2=14)
+    _, _, st3 = idx.search(q, k, L)
+    _, _, st4 = idx.search(q, k, L)
+    assert st3.spills > Q // 20 and st4.spills > Q // 20  # (the count varies a little with the order of inserts)
+    idx.close()
