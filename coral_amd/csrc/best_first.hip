@@ -5,12 +5,13 @@
 // measure the new ones, insert them, pick the closest entry not yet expanded.  Every step is a chain of dependent
 // memory accesses; what makes it fast on this GPU is how many such chains run side by side.  A workgroup per query
 // with the visited set in LDS (the form beam_search.hip gives this policy) holds two queries per CU.  Here a query
-// needs one wavefront and 9 KB of LDS at L = 512 (its sorted beam, twice, for the merge): sixteen queries per CU,
-// enough to keep HBM busy (2.4 times the throughput of the other form at a million nodes).  The visited set moves to
-// global memory in the form the CPU path itself uses (src/search_in_cpu.cpp:44-48, 68-71): one byte per node and
-// query slot holding the epoch of the query that last visited the node, so nothing is cleared between queries
-// (every 255th query of a slot wipes its array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a
-// million nodes); each test costs a 128-byte line of HBM traffic, about a sixth of what the vectors cost.
+// needs one wavefront and 5.4 KB of LDS at L = 512 (its sorted beam, merged in place): sixteen queries per CU, as
+// many as 128 registers per lane allow, enough to keep HBM busy (2.6 times the throughput of the other form at a
+// million nodes; more wavefronts add nothing).  The visited set moves to global memory in the form the CPU path
+// itself uses (src/search_in_cpu.cpp:44-48, 68-71): one byte per node and query slot holding the epoch of the
+// query that last visited the node, so nothing is cleared between queries (every 255th query of a slot wipes its
+// array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a million nodes); each test costs a
+// 128-byte line of HBM traffic and each mark a 32-byte write, together about a quarter of what the vectors cost.
 //
 // The arithmetic is that of beam_search.hip (same lane-strided accumulation, same butterfly, same 64-bit keys), so
 // results and counters are identical bit for bit; a wavefront needs no workgroup barrier anywhere.
@@ -33,8 +34,20 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// inclusive prefix sum over the 64 lanes: four steps inside the rows of 16 lanes, then the totals of the rows
+// before (row_bcast15 into rows 1 and 3, row_bcast31 into rows 2 and 3); lanes without a source add 0
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast15
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast31
+    return v;
+}
+
 template <int G, int CPL, int RIF>
-__global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
+__global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = blockIdx.x * kWavesPerWg + wave;
@@ -42,10 +55,11 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
     const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2, M = a.M;
     const int Lp = (L + 3) & ~3;
     unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L);
-    uint64_t* beam0 = reinterpret_cast<uint64_t*>(mine_lds);
-    uint64_t* beam1 = beam0 + Lp;
-    uint64_t* cand = beam1 + Lp;                                 // kBatch keys
+    uint64_t* beam = reinterpret_cast<uint64_t*>(mine_lds);      // L keys, sorted
+    uint64_t* cand = beam + Lp;                                   // kBatch keys
     uint32_t* todo = reinterpret_cast<uint32_t*>(cand + kBatch);  // kBatch ids
+    uint32_t* marks = todo + kBatch;                              // Lp byte counters, zero between merges
+    for (int i = lane; i < (Lp >> 2); i += 64) marks[i] = 0u;
 
     uint8_t* vis = b.visited + (size_t)slot * b.stride;
     uint32_t epoch = b.epochs[slot];
@@ -80,7 +94,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
             }
         }
 
-        int nb = 0, cur = 0, cursor = 0;
+        int nb = 0, cursor = 0;
         uint64_t live = kKeyMax;
         int hops = M, nd = M, ne = 0, rounds = 0;
 
@@ -151,34 +165,43 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
             }
             wave_sync();
             if (nc == 0) return;
-            // few keys: a key's place is its own index plus the number of smaller keys in the other list
-            const uint64_t* src = cur ? beam1 : beam0;
-            uint64_t* dst = cur ? beam0 : beam1;
-            for (int i = lane; i < nb; i += 64) {
-                const uint64_t key = src[i];
-                int below = 0;
-                for (int c = 0; c < nc; ++c) below += cand[c] < key;
-                if (i + below < L) dst[i + below] = key;
-            }
-            int first_pos = L;
+            // In place: a candidate's place is its rank among the candidates plus the number of beam keys below it
+            // (p); a beam key moves up by the number of candidates with p at or below its index.  Those counts come
+            // from one byte counter per beam position and a prefix sum, chunk by chunk from the top, so that what a
+            // chunk overwrites has been read already; nothing below the first insertion moves.
+            uint64_t ck = 0;
+            int p = 0x7fffffff, rank = 0;
             if (lane < nc) {
-                const uint64_t key = cand[lane];
-                int below = 0;
-                for (int c = 0; c < nc; ++c) below += cand[c] < key;
-                const int pos = below + lower_bound_u64(src, nb, key);
-                if (pos < L) dst[pos] = key;
-                if (below == 0) first_pos = pos;
+                ck = cand[lane];
+                for (int c = 0; c < nc; ++c) rank += cand[c] < ck;
+                p = lower_bound_u64(beam, nb, ck);
+                if (p < nb) atomicAdd(&marks[p >> 2], 1u << ((p & 3) * 8));
             }
+            const uint64_t mz = __ballot(lane < nc && rank == 0);  // the closest candidate: exactly one lane
+            const int fp = __builtin_amdgcn_readlane(p, __ffsll((long long)mz) - 1);
             // entries before the cursor are all expanded: the closest new key may land before it
-            const uint64_t mf = __ballot(first_pos < L);
-            if (mf) {
-                const int fp = __shfl(first_pos, __ffsll((long long)mf) - 1, 64);
-                cursor = fp < cursor ? fp : cursor;
+            if (fp < L && fp < cursor) cursor = fp;
+            wave_sync();
+            if (fp < nb) {
+                for (int base = (nb - 1) & ~63; base >= (fp & ~63); base -= 64) {
+                    const int i = base + lane;
+                    const bool act = i < nb;
+                    const uint64_t key = act ? beam[i] : 0ull;
+                    const int m = act ? (int)((marks[i >> 2] >> ((i & 3) * 8)) & 0xffu) : 0;
+                    const int carry = __popcll(__ballot(lane < nc && p < base));
+                    const int shift = carry + wave_inclusive_sum(m);
+                    wave_sync();  // every read of this chunk before its writes
+                    if (act && shift > 0 && i + shift < L) beam[i + shift] = key;
+                }
+            }
+            wave_sync();
+            if (lane < nc) {
+                if (p + rank < L) beam[p + rank] = ck;
+                if (p < nb) marks[p >> 2] = 0u;
             }
             wave_sync();
             nb = nb + nc < L ? nb + nc : L;
-            cur ^= 1;
-            live = nb == L ? dst[L - 1] : kKeyMax;
+            live = nb == L ? beam[L - 1] : kKeyMax;
         };
 
         // ---- seeds: every start id is visited and measured (src/search_in_cpu.cpp:74-79)
@@ -196,7 +219,6 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
 
         // ---- one expansion per step
         for (;;) {
-            uint64_t* beam = cur ? beam1 : beam0;
             int c = cursor, found = nb;
             while (c < nb) {
                 const int i = c + lane;
@@ -220,14 +242,14 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
             if (lane < R) v = a.nbrs[(size_t)eid * R + lane];
             bool isnew = false;
             if (v >= 0) isnew = __hip_atomic_load(vis + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != tag;
-            if (__ballot(isnew)) {
+            if (!b.rows_unique && __ballot(isnew)) {
                 // an id listed twice in the row counts once (the first listing)
                 for (int k = 0; k < R; ++k) {
                     const int vk = __builtin_amdgcn_readlane(v, k);
                     if (k < lane && vk == v) isnew = false;
                 }
-                if (isnew) __hip_atomic_store(vis + v, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
+            if (isnew) __hip_atomic_store(vis + v, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const uint64_t m = __ballot(isnew);
             const int T = __popcll(m);
             if (isnew) todo[prefix_popc(m)] = (uint32_t)v;
@@ -243,7 +265,6 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
 
         // ---- output: the k closest live entries, closest first
         {
-            const uint64_t* beam = cur ? beam1 : beam0;
             int32_t* ids_out = a.ids_out + (size_t)qid * a.k;
             float* dists_out = a.dists_out ? a.dists_out + (size_t)qid * a.k : nullptr;
             int outpos = 0;
@@ -287,6 +308,21 @@ __global__ __launch_bounds__(kWavesPerWg * 64, 4) void best_first_wave_kernel(co
     if (lane == 0) b.epochs[slot] = epoch;
 }
 
+// one thread per graph row: does it list an id twice?
+__global__ __launch_bounds__(256) void find_repeated_ids_kernel(const int32_t* __restrict__ nbrs, int64_t n, int R,
+                                                                uint32_t* flag) {
+    const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= n) return;
+    const int32_t* r = nbrs + row * R;
+    bool rep = false;
+    for (int i = 1; i < R; ++i) {
+        const int32_t v = r[i];
+        if (v < 0) break;  // rows end at their first -1
+        for (int j = 0; j < i; ++j) rep |= r[j] == v;
+    }
+    if (rep) atomicOr(flag, 1u);
+}
+
 using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 
 // RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
@@ -327,6 +363,13 @@ hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStr
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_wave_lds_bytes(a.L) * kWavesPerWg, stream, a, b);
+    return hipGetLastError();
+}
+
+hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream) {
+    const int64_t blocks = (n + 255) / 256;
+    if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(find_repeated_ids_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, nbrs, n, R, flag);
     return hipGetLastError();
 }
 

@@ -178,6 +178,7 @@ int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const int32_t* 
         idx->M = n_start;
         idx->prepared = false;
     }
+    idx->rows_unique = -1;
     HIP_TRY(hipMemcpy(idx->d_nbrs, nbrs, (size_t)idx->n * idx->R * sizeof(int32_t),
                       hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(idx->d_start, start_ids, (size_t)n_start * sizeof(int32_t),
@@ -379,6 +380,17 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     a.tcap = idx->tcap, a.ccap = idx->ccap;
     a.id_bits = idx->id_bits, a.rem_bits = idx->rem_bits, a.dmax = idx->dmax, a.ocap = idx->ocap;
 
+    const bool wave_kernel = policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready;
+    if (wave_kernel && idx->rows_unique < 0) {
+        // once per graph: rows without repeated ids let the kernel skip its comparison of a row with itself
+        uint32_t flag = 0;
+        HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_scalars, 4, 0u, stream));
+        HIP_TRY(coral::launch_find_repeated_ids(idx->d_nbrs, idx->n, idx->R, (uint32_t*)idx->d_scalars + 2, stream));
+        HIP_TRY(hipMemcpyAsync(&flag, idx->d_scalars + 2, sizeof flag, hipMemcpyDeviceToHost, stream));
+        HIP_TRY(hipStreamSynchronize(stream));
+        idx->rows_unique = flag ? 0 : 1;
+    }
+
     hipEvent_t ev0, evk, ev1;
     HIP_TRY(hipEventCreate(&ev0));
     HIP_TRY(hipEventCreate(&evk));
@@ -391,8 +403,9 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
 #endif
     // timed region, same scope as the reference: kernel + counter read-back
     HIP_TRY(hipEventRecord(ev0, stream));
-    if (policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready) {
+    if (wave_kernel) {
         coral::BestFirstArgs b;
+        b.rows_unique = idx->rows_unique == 1;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;

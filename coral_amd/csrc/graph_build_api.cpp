@@ -103,6 +103,7 @@ int coral_build_begin(coral_index* idx, int32_t R) {
         idx->R = R;
     }
     idx->prepared = false;
+    idx->rows_unique = -1;
     HIP_TRY(hipMalloc(&idx->d_nbr_dists, n * R * sizeof(float)));
     HIP_TRY(hipMalloc(&idx->d_deg, n * sizeof(int32_t)));
     HIP_TRY(hipMalloc(&idx->d_owner, n * sizeof(int32_t)));
@@ -135,6 +136,7 @@ int coral_build_nap_batch(coral_index* idx, const int32_t* d_knn_ids, int32_t ba
     HIP_TRY(hipSetDevice(idx->device));
     if (int rc = ensure_stage(idx, (size_t)batch * k_b)) return rc;
     if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * k_b, false, "cluster ids")) return rc;
+    idx->rows_unique = -1;
     HIP_TRY(coral::launch_nap_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists, idx->d_deg,
                                     idx->d_owner, d_knn_ids, batch, k_b, need_discard, idx->d_new_ids, idx->d_new_dists,
                                     idx->d_new_deg, idx->stream));
@@ -160,6 +162,7 @@ int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_ids, const 
     }
     if (int rc = check_ids(idx, d_iso_ids, batch, false, "isolated ids")) return rc;
     if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * kn, true, "found ids")) return rc;
+    idx->rows_unique = -1;
     HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_build_stats, 4, 0u, idx->stream));
     HIP_TRY(coral::launch_enhance_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists,
                                         idx->d_deg, idx->d_owner, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn, idx->d_len,
