@@ -170,7 +170,7 @@ def main():
         out["best_first"]["kernel"] = "best_first_wave_kernel"
         out["best_first"]["frac"] = best_first["gbps"] / HBM_PEAK_GBPS
 
-    # the IndexGPU::Search shape: host buffers in and out (device allocation, query upload,
+    # the IndexGPU::Search shape: host buffers in and out (query upload to the index's staging buffers,
     # search, id download); reported beside the headline, never as the headline
     idx.search(queries, k, head["L"], want_dists=False)
     t = time.perf_counter()

@@ -157,6 +157,11 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_phase);
     (void)hipFree(idx->d_bf_visited);
     (void)hipFree(idx->d_bf_epochs);
+    (void)hipFree(idx->d_io_q);
+    (void)hipFree(idx->d_io_ids);
+    (void)hipFree(idx->d_io_dists);
+    for (hipEvent_t e : idx->ev)
+        if (e) (void)hipEventDestroy(e);
     coral::free_build_state(idx);
     if (idx->h_counters) (void)hipHostFree(idx->h_counters);
     if (idx->stream) (void)hipStreamDestroy(idx->stream);
@@ -391,10 +396,9 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         idx->rows_unique = flag ? 0 : 1;
     }
 
-    hipEvent_t ev0, evk, ev1;
-    HIP_TRY(hipEventCreate(&ev0));
-    HIP_TRY(hipEventCreate(&evk));
-    HIP_TRY(hipEventCreate(&ev1));
+    for (hipEvent_t& e : idx->ev)
+        if (!e) HIP_TRY(hipEventCreate(&e));
+    hipEvent_t ev0 = idx->ev[0], evk = idx->ev[1], ev1 = idx->ev[2];
     HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_scalars, 4, 0u, stream));
 #ifdef CORAL_PHASE_TIMERS
     if (!idx->d_phase) HIP_TRY(hipMalloc(&idx->d_phase, 8 * sizeof(unsigned long long)));
@@ -422,9 +426,6 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     float ms = 0.f, ms_kernel = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
     HIP_TRY(hipEventElapsedTime(&ms_kernel, ev0, evk));
-    (void)hipEventDestroy(ev0);
-    (void)hipEventDestroy(evk);
-    (void)hipEventDestroy(ev1);
     int scal[2] = {0, 0};
     HIP_TRY(hipMemcpyAsync(scal, idx->d_scalars, sizeof scal, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
@@ -488,38 +489,27 @@ int coral_search(coral_index* idx, const float* h_queries, int32_t Q, int32_t k,
         t.policy = policy;
         if (int rc = coral_search_prepare(idx, Q, L, &t)) return rc;
     }
-    float* d_q = nullptr;
-    int32_t* d_ids = nullptr;
-    float* d_dists = nullptr;
-    int rc = CORAL_OK;
-    const size_t qbytes = (size_t)Q * idx->dim * sizeof(float);
-    auto release = [&]() {
-        (void)hipFree(d_q);
-        (void)hipFree(d_ids);
-        (void)hipFree(d_dists);
+    // device copies of the caller's buffers: kept with the index and grown when a call needs more
+    auto grow = [](void** p, size_t* have, size_t need) -> hipError_t {
+        if (need <= *have) return hipSuccess;
+        (void)hipFree(*p);
+        *p = nullptr, *have = 0;
+        const hipError_t e = hipMalloc(p, need);
+        if (e == hipSuccess) *have = need;
+        return e;
     };
-#define HIP_TRY_R(expr)                                                                         \
-    do {                                                                                        \
-        hipError_t e_ = (expr);                                                                 \
-        if (e_ != hipSuccess) {                                                                 \
-            release();                                                                          \
-            return fail(e_ == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE,        \
-                        "%s failed: %s", #expr, hipGetErrorString(e_));                         \
-        }                                                                                       \
-    } while (0)
-    HIP_TRY_R(hipMalloc(&d_q, qbytes));
-    HIP_TRY_R(hipMalloc(&d_ids, (size_t)Q * k * sizeof(int32_t)));
-    if (h_dists) HIP_TRY_R(hipMalloc(&d_dists, (size_t)Q * k * sizeof(float)));
-    HIP_TRY_R(hipMemcpy(d_q, h_queries, qbytes, hipMemcpyHostToDevice));
-    rc = coral_search_gpu(idx, d_q, d_ids, d_dists, Q, k, policy, have_delete, nullptr, stats);
-    if (rc == CORAL_OK) {
-        HIP_TRY_R(hipMemcpy(h_ids, d_ids, (size_t)Q * k * sizeof(int32_t), hipMemcpyDeviceToHost));
-        if (h_dists)
-            HIP_TRY_R(hipMemcpy(h_dists, d_dists, (size_t)Q * k * sizeof(float), hipMemcpyDeviceToHost));
-    }
-#undef HIP_TRY_R
-    release();
-    return rc;
+    const size_t qbytes = (size_t)Q * idx->dim * sizeof(float);
+    const size_t ibytes = (size_t)Q * k * sizeof(int32_t), dbytes = (size_t)Q * k * sizeof(float);
+    HIP_TRY(grow((void**)&idx->d_io_q, &idx->io_q_bytes, qbytes));
+    HIP_TRY(grow((void**)&idx->d_io_ids, &idx->io_ids_bytes, ibytes));
+    if (h_dists) HIP_TRY(grow((void**)&idx->d_io_dists, &idx->io_dists_bytes, dbytes));
+    HIP_TRY(hipMemcpy(idx->d_io_q, h_queries, qbytes, hipMemcpyHostToDevice));
+    const int rc = coral_search_gpu(idx, idx->d_io_q, idx->d_io_ids, h_dists ? idx->d_io_dists : nullptr, Q, k, policy,
+                                    have_delete, nullptr, stats);
+    if (rc != CORAL_OK) return rc;
+    HIP_TRY(hipMemcpy(h_ids, idx->d_io_ids, ibytes, hipMemcpyDeviceToHost));
+    if (h_dists) HIP_TRY(hipMemcpy(h_dists, idx->d_io_dists, dbytes, hipMemcpyDeviceToHost));
+    return CORAL_OK;
 }
 
 int coral_search_verify(coral_index* idx, const int32_t* d_ids_res, const int32_t* d_ids_gt, int32_t Q,

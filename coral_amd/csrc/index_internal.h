@@ -44,6 +44,12 @@ struct coral_index {
     unsigned long long* d_phase = nullptr;  // debug builds only
     int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
     int last_Q = 0;
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};  // start, kernel end, read-back end of a search
+    // device staging of the host-buffer entry point (grow-only)
+    float* d_io_q = nullptr;
+    int32_t* d_io_ids = nullptr;
+    float* d_io_dists = nullptr;
+    size_t io_q_bytes = 0, io_ids_bytes = 0, io_dists_bytes = 0;
 
     // best-first on one wavefront per query: per-slot visited epochs in global memory
     bool bf_ready = false;
