@@ -47,13 +47,14 @@ class BuildParams(C.Structure):
     _fields_ = [("R", C.c_int32), ("k_b", C.c_int32), ("batch", C.c_int32), ("need_discard", C.c_int32),
                 ("connect_enhance", C.c_int32), ("enhance_search_batch", C.c_int32), ("enhance_nap_batch", C.c_int32),
                 ("enhance_L", C.c_int32), ("n_start", C.c_int32), ("first_start_id", C.c_int32),
-                ("reserved", C.c_int32 * 6)]
+                ("top_hit_num", C.c_int32), ("reserved", C.c_int32 * 5)]
 
 
 class BuildStats(C.Structure):
     _fields_ = [("knn_s", C.c_double), ("nap_s", C.c_double), ("enhance_s", C.c_double), ("total_s", C.c_double),
                 ("batches", C.c_int64), ("isolated", C.c_int64), ("reverse_edges", C.c_int64),
-                ("reverse_rejected", C.c_int64), ("edges", C.c_int64)]
+                ("reverse_rejected", C.c_int64), ("edges", C.c_int64), ("top_hit_nodes", C.c_int64),
+                ("top_reverse_edges", C.c_int64)]
 
     def as_dict(self):
         return {f: getattr(self, f) for f, _ in self._fields_}
@@ -99,6 +100,9 @@ SIGNATURES = {
     "coral_build_nap_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32]),
     "coral_build_enhance_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                             C.c_void_p, C.c_void_p]),
+    "coral_build_enhance_top_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                                C.c_void_p, C.c_void_p]),
+    "coral_build_top_hit_ids": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "coral_build_connect_enhance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_build_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "coral_build_graph_from_clusters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
@@ -256,6 +260,19 @@ class Index:
         _check(lib().coral_build_enhance_batch(self._h, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn, C.byref(ins),
                                                C.byref(rej)))
         return ins.value, rej.value
+
+    def build_enhance_top_batch(self, d_top_ids, d_knn_ids, d_knn_dists, batch, k):
+        ins, rej = C.c_int64(), C.c_int64()
+        _check(lib().coral_build_enhance_top_batch(self._h, d_top_ids, d_knn_ids, d_knn_dists, batch, k, C.byref(ins),
+                                                   C.byref(rej)))
+        return ins.value, rej.value
+
+    def build_top_hit_ids(self, top_n):
+        """(ids [top_n] by hits descending then id, hits [n])"""
+        ids = np.empty(top_n, np.int32)
+        hits = np.empty(self.n, np.uint32)
+        _check(lib().coral_build_top_hit_ids(self._h, top_n, _ptr(ids), _ptr(hits)))
+        return ids, hits
 
     def build_connect_enhance(self, params):
         st = BuildStats()

@@ -360,7 +360,7 @@ __global__ void nap_commit_kernel(const int32_t* __restrict__ knn, int64_t count
 
 // one wavefront per isolated node: length of its found list (an id of -1 ends it) and the claims on the found nodes
 __global__ void enh_claim_kernel(const int32_t* __restrict__ knn_ids, int batch, int kn, int32_t* __restrict__ len,
-                                 int32_t* __restrict__ owner) {
+                                 const int32_t* __restrict__ rev_len, int32_t* __restrict__ owner) {
     const int lane = threadIdx.x & 63;
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
     for (int b = wave; b < batch; b += nwaves) {
@@ -374,6 +374,7 @@ __global__ void enh_claim_kernel(const int32_t* __restrict__ knn_ids, int batch,
             }
         }
         if (lane == 0) len[b] = n;
+        if (rev_len) n = min(n, rev_len[b]);  // only these entries insert reverse edges
         for (int i = lane; i < n; i += 64) atomicMin(owner + knn_ids[(size_t)b * kn + i], b * kn + i);
     }
 }
@@ -383,7 +384,8 @@ __global__ void enh_claim_kernel(const int32_t* __restrict__ knn_ids, int batch,
 __global__ void enh_reverse_kernel(const float* __restrict__ vec, int dim, int metric, int R, int32_t* __restrict__ nbrs,
                                    float* __restrict__ dists, int32_t* __restrict__ deg, int32_t* __restrict__ owner,
                                    const int32_t* __restrict__ iso_ids, const int32_t* __restrict__ knn_ids,
-                                   const float* __restrict__ knn_dists, const int32_t* __restrict__ len, int batch, int kn,
+                                   const float* __restrict__ knn_dists, const int32_t* __restrict__ len,
+                                   const int32_t* __restrict__ rev_len, int batch, int kn,
                                    unsigned long long* __restrict__ stats) {
     const int gtid = blockIdx.x * blockDim.x + threadIdx.x;
     const int l = gtid & 31, shift = threadIdx.x & 32;
@@ -396,7 +398,7 @@ __global__ void enh_reverse_kernel(const float* __restrict__ vec, int dim, int m
         int b = 0, v = -1;
         if (active) {
             b = pair / kn;
-            active = pair - b * kn < len[b];
+            active = pair - b * kn < (rev_len ? min(len[b], rev_len[b]) : len[b]);
         }
         if (active) {
             v = knn_ids[pair];
@@ -478,6 +480,50 @@ enh_rows_kernel(const float* __restrict__ vec, int dim, int metric, int R, int32
     }
 }
 
+// build_candidate_kernel of the second phase (src/enhance.cu:58-129), the part that lists the candidates: what the
+// search found for the node (up to the first -1), then the node's current row with its stored distances; -1 pads.
+// One wavefront per node; out lists are [batch][k + R], rev_len[b] = number of found entries.
+__global__ void enh_top_lists_kernel(int R, const int32_t* __restrict__ nbrs, const float* __restrict__ dists,
+                                     const int32_t* __restrict__ deg, const int32_t* __restrict__ top_ids,
+                                     const int32_t* __restrict__ knn_ids, const float* __restrict__ knn_dists, int batch,
+                                     int k, int32_t* __restrict__ out_ids, float* __restrict__ out_dists,
+                                     int32_t* __restrict__ rev_len) {
+    const int lane = threadIdx.x & 63;
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
+    const int kn = k + R;
+    for (int b = wave; b < batch; b += nwaves) {
+        int nf = k;
+        for (int i0 = 0; i0 < k; i0 += 64) {
+            const int i = i0 + lane;
+            const unsigned long long neg = __ballot(i < k && knn_ids[(size_t)b * k + i] < 0);
+            if (neg) {
+                nf = i0 + __ffsll((long long)neg) - 1;
+                break;
+            }
+        }
+        const int32_t t = top_ids[b];
+        const int d = deg[t];
+        for (int q = lane; q < kn; q += 64) {
+            int32_t id = -1;
+            float dist = 0.0f;
+            if (q < nf) {
+                id = knn_ids[(size_t)b * k + q], dist = knn_dists[(size_t)b * k + q];
+            } else if (q - nf < d) {
+                id = nbrs[(size_t)t * R + (q - nf)], dist = dists[(size_t)t * R + (q - nf)];
+            }
+            out_ids[(size_t)b * kn + q] = id;
+            out_dists[(size_t)b * kn + q] = dist;
+        }
+        if (lane == 0) rev_len[b] = nf;
+    }
+}
+
+// hits_update_kernel (src/knn.cu:60-73): one more cluster contains these nodes
+__global__ void count_hits_kernel(const int32_t* __restrict__ ids, int64_t count, uint32_t* __restrict__ hits) {
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (int64_t)gridDim.x * blockDim.x)
+        atomicAdd(hits + ids[t], 1u);
+}
+
 __global__ void count_bad_ids_kernel(const int32_t* __restrict__ ids, int64_t count, int64_t n, int minus_one_ok,
                                      unsigned long long* __restrict__ bad) {
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (int64_t)gridDim.x * blockDim.x) {
@@ -526,17 +572,33 @@ hipError_t launch_nap_batch(const float* vec, int dim, int metric, int R, int32_
 
 hipError_t launch_enhance_batch(const float* vec, int dim, int metric, int R, int32_t* nbrs, float* dists, int32_t* deg,
                                 int32_t* owner, const int32_t* iso_ids, const int32_t* knn_ids, const float* knn_dists,
-                                int batch, int kn, int32_t* len, unsigned long long* stats, hipStream_t st) {
+                                int batch, int kn, int32_t* len, const int32_t* rev_len, unsigned long long* stats,
+                                hipStream_t st) {
     const int waves_per_block = 4;
     int blocks = (batch + waves_per_block - 1) / waves_per_block;
-    hipLaunchKernelGGL(enh_claim_kernel, dim3(blocks), dim3(256), 0, st, knn_ids, batch, kn, len, owner);
+    hipLaunchKernelGGL(enh_claim_kernel, dim3(blocks), dim3(256), 0, st, knn_ids, batch, kn, len, rev_len, owner);
     const int64_t pairs = (int64_t)batch * kn;
     int64_t rb = (pairs * 32 + 255) / 256;
     rb = rb > 8192 ? 8192 : rb;
     hipLaunchKernelGGL(enh_reverse_kernel, dim3((unsigned)rb), dim3(256), 0, st, vec, dim, metric, R, nbrs, dists, deg,
-                       owner, iso_ids, knn_ids, knn_dists, len, batch, kn, stats);
+                       owner, iso_ids, knn_ids, knn_dists, len, rev_len, batch, kn, stats);
     hipLaunchKernelGGL(enh_rows_kernel, dim3(blocks), dim3(kThreads), 0, st, vec, dim, metric, R, nbrs, dists, deg,
                        iso_ids, knn_ids, knn_dists, len, batch, kn);
+    return hipGetLastError();
+}
+
+hipError_t launch_enhance_top_lists(int R, const int32_t* nbrs, const float* dists, const int32_t* deg,
+                                    const int32_t* top_ids, const int32_t* knn_ids, const float* knn_dists, int batch, int k,
+                                    int32_t* out_ids, float* out_dists, int32_t* rev_len, hipStream_t st) {
+    hipLaunchKernelGGL(enh_top_lists_kernel, dim3((batch + 3) / 4), dim3(256), 0, st, R, nbrs, dists, deg, top_ids, knn_ids,
+                       knn_dists, batch, k, out_ids, out_dists, rev_len);
+    return hipGetLastError();
+}
+
+hipError_t launch_count_hits(const int32_t* ids, int64_t count, uint32_t* hits, hipStream_t st) {
+    int64_t blocks = (count + 255) / 256;
+    blocks = blocks > 2048 ? 2048 : (blocks < 1 ? 1 : blocks);
+    hipLaunchKernelGGL(count_hits_kernel, dim3((unsigned)blocks), dim3(256), 0, st, ids, count, hits);
     return hipGetLastError();
 }
 

@@ -18,11 +18,13 @@ namespace coral {
 void free_build_state(coral_index* idx) {
     (void)hipFree(idx->d_nbr_dists), (void)hipFree(idx->d_deg), (void)hipFree(idx->d_owner);
     (void)hipFree(idx->d_new_ids), (void)hipFree(idx->d_new_dists), (void)hipFree(idx->d_new_deg);
-    (void)hipFree(idx->d_len), (void)hipFree(idx->d_build_stats);
+    (void)hipFree(idx->d_len), (void)hipFree(idx->d_build_stats), (void)hipFree(idx->d_hits);
+    (void)hipFree(idx->d_top_ids_list), (void)hipFree(idx->d_top_dists_list), (void)hipFree(idx->d_rev_len);
     idx->d_nbr_dists = nullptr, idx->d_deg = nullptr, idx->d_owner = nullptr;
     idx->d_new_ids = nullptr, idx->d_new_dists = nullptr, idx->d_new_deg = nullptr;
-    idx->d_len = nullptr, idx->d_build_stats = nullptr;
-    idx->stage_rows = 0, idx->len_alloc = 0;
+    idx->d_len = nullptr, idx->d_build_stats = nullptr, idx->d_hits = nullptr;
+    idx->d_top_ids_list = nullptr, idx->d_top_dists_list = nullptr, idx->d_rev_len = nullptr;
+    idx->stage_rows = 0, idx->len_alloc = 0, idx->top_list_cells = 0, idx->rev_len_alloc = 0;
     idx->building = false;
 }
 }  // namespace coral
@@ -108,6 +110,8 @@ int coral_build_begin(coral_index* idx, int32_t R) {
     HIP_TRY(hipMalloc(&idx->d_deg, n * sizeof(int32_t)));
     HIP_TRY(hipMalloc(&idx->d_owner, n * sizeof(int32_t)));
     HIP_TRY(hipMalloc(&idx->d_build_stats, 4 * sizeof(unsigned long long)));
+    HIP_TRY(hipMalloc(&idx->d_hits, n * sizeof(uint32_t)));
+    HIP_TRY(coral::launch_fill_u32(idx->d_hits, n, 0u, idx->stream));
     HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_nbrs, n * R, 0xffffffffu, idx->stream));
     HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_nbr_dists, n * R, 0u, idx->stream));
     HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_deg, n, 0u, idx->stream));
@@ -137,10 +141,35 @@ int coral_build_nap_batch(coral_index* idx, const int32_t* d_knn_ids, int32_t ba
     if (int rc = ensure_stage(idx, (size_t)batch * k_b)) return rc;
     if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * k_b, false, "cluster ids")) return rc;
     idx->rows_unique = -1;
+    HIP_TRY(coral::launch_count_hits(d_knn_ids, (int64_t)batch * k_b, idx->d_hits, idx->stream));
     HIP_TRY(coral::launch_nap_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists, idx->d_deg,
                                     idx->d_owner, d_knn_ids, batch, k_b, need_discard, idx->d_new_ids, idx->d_new_dists,
                                     idx->d_new_deg, idx->stream));
     HIP_TRY(hipStreamSynchronize(idx->stream));
+    return CORAL_OK;
+}
+
+// the common part of the two enhancement batches: lists [batch][kn], of which the first rev_len[b] (all, if null)
+// insert reverse edges
+static int enhance_lists(coral_index* idx, const int32_t* d_node_ids, const int32_t* d_ids, const float* d_dists,
+                         int32_t batch, int32_t kn, const int32_t* d_rev_len, int64_t* reverse_edges,
+                         int64_t* reverse_rejected) {
+    if ((size_t)batch > idx->len_alloc) {
+        (void)hipFree(idx->d_len);
+        idx->d_len = nullptr, idx->len_alloc = 0;
+        HIP_TRY(hipMalloc(&idx->d_len, (size_t)batch * sizeof(int32_t)));
+        idx->len_alloc = (size_t)batch;
+    }
+    idx->rows_unique = -1;
+    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_build_stats, 4, 0u, idx->stream));
+    HIP_TRY(coral::launch_enhance_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists,
+                                        idx->d_deg, idx->d_owner, d_node_ids, d_ids, d_dists, batch, kn, idx->d_len,
+                                        d_rev_len, idx->d_build_stats, idx->stream));
+    unsigned long long st[2] = {0, 0};
+    HIP_TRY(hipMemcpyAsync(st, idx->d_build_stats, sizeof(st), hipMemcpyDeviceToHost, idx->stream));
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    if (reverse_edges) *reverse_edges = (int64_t)st[0];
+    if (reverse_rejected) *reverse_rejected = (int64_t)st[1];
     return CORAL_OK;
 }
 
@@ -154,24 +183,73 @@ int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_ids, const 
         return fail(CORAL_ERR_ARG, "found-list length must be in 1..%d (got %d)", coral::kBuildMaxKb + coral::kBuildMaxR, kn);
     if ((int64_t)batch * kn > INT_MAX / 2) return fail(CORAL_ERR_ARG, "batch * list length too large");
     HIP_TRY(hipSetDevice(idx->device));
-    if ((size_t)batch > idx->len_alloc) {
-        (void)hipFree(idx->d_len);
-        idx->d_len = nullptr, idx->len_alloc = 0;
-        HIP_TRY(hipMalloc(&idx->d_len, (size_t)batch * sizeof(int32_t)));
-        idx->len_alloc = (size_t)batch;
-    }
     if (int rc = check_ids(idx, d_iso_ids, batch, false, "isolated ids")) return rc;
     if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * kn, true, "found ids")) return rc;
-    idx->rows_unique = -1;
-    HIP_TRY(coral::launch_fill_u32((uint32_t*)idx->d_build_stats, 4, 0u, idx->stream));
-    HIP_TRY(coral::launch_enhance_batch(idx->d_vec, idx->dim, idx->metric, idx->R, idx->d_nbrs, idx->d_nbr_dists,
-                                        idx->d_deg, idx->d_owner, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn, idx->d_len,
-                                        idx->d_build_stats, idx->stream));
-    unsigned long long st[2] = {0, 0};
-    HIP_TRY(hipMemcpyAsync(st, idx->d_build_stats, sizeof(st), hipMemcpyDeviceToHost, idx->stream));
+    return enhance_lists(idx, d_iso_ids, d_knn_ids, d_knn_dists, batch, kn, nullptr, reverse_edges, reverse_rejected);
+}
+
+int coral_build_enhance_top_batch(coral_index* idx, const int32_t* d_top_ids, const int32_t* d_knn_ids,
+                                  const float* d_knn_dists, int32_t batch, int32_t k, int64_t* reverse_edges,
+                                  int64_t* reverse_rejected) {
+    if (!idx || !d_top_ids || !d_knn_ids || !d_knn_dists) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->building) return fail(CORAL_ERR_STATE, "coral_build_begin has not been called");
+    if (batch <= 0) return fail(CORAL_ERR_ARG, "batch must be positive");
+    if (k < 1 || k > coral::kBuildMaxKb) return fail(CORAL_ERR_ARG, "found-list length must be in 1..%d (got %d)", coral::kBuildMaxKb, k);
+    const int kn = k + idx->R;
+    if ((int64_t)batch * kn > INT_MAX / 2) return fail(CORAL_ERR_ARG, "batch * list length too large");
+    HIP_TRY(hipSetDevice(idx->device));
+    if (int rc = check_ids(idx, d_top_ids, batch, false, "node ids")) return rc;
+    if (int rc = check_ids(idx, d_knn_ids, (int64_t)batch * k, true, "found ids")) return rc;
+    const size_t cells = (size_t)batch * kn;
+    if (cells > idx->top_list_cells) {
+        (void)hipFree(idx->d_top_ids_list), (void)hipFree(idx->d_top_dists_list);
+        idx->d_top_ids_list = nullptr, idx->d_top_dists_list = nullptr, idx->top_list_cells = 0;
+        HIP_TRY(hipMalloc(&idx->d_top_ids_list, cells * sizeof(int32_t)));
+        HIP_TRY(hipMalloc(&idx->d_top_dists_list, cells * sizeof(float)));
+        idx->top_list_cells = cells;
+    }
+    if ((size_t)batch > idx->rev_len_alloc) {
+        (void)hipFree(idx->d_rev_len);
+        idx->d_rev_len = nullptr, idx->rev_len_alloc = 0;
+        HIP_TRY(hipMalloc(&idx->d_rev_len, (size_t)batch * sizeof(int32_t)));
+        idx->rev_len_alloc = (size_t)batch;
+    }
+    HIP_TRY(coral::launch_enhance_top_lists(idx->R, idx->d_nbrs, idx->d_nbr_dists, idx->d_deg, d_top_ids, d_knn_ids,
+                                            d_knn_dists, batch, k, idx->d_top_ids_list, idx->d_top_dists_list,
+                                            idx->d_rev_len, idx->stream));
+    return enhance_lists(idx, d_top_ids, idx->d_top_ids_list, idx->d_top_dists_list, batch, kn, idx->d_rev_len,
+                         reverse_edges, reverse_rejected);
+}
+
+int coral_build_top_hit_ids(coral_index* idx, int64_t top_n, int32_t* h_ids, uint32_t* h_hits) {
+    if (!idx || (!h_ids && !h_hits)) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->building) return fail(CORAL_ERR_STATE, "coral_build_begin has not been called");
+    if (top_n < 0 || top_n > idx->n) return fail(CORAL_ERR_ARG, "top_n must be in 0..n");
+    HIP_TRY(hipSetDevice(idx->device));
+    std::vector<uint32_t> local;
+    uint32_t* hits = h_hits;
+    if (!hits) {
+        local.resize((size_t)idx->n);
+        hits = local.data();
+    }
+    HIP_TRY(hipMemcpyAsync(hits, idx->d_hits, (size_t)idx->n * sizeof(uint32_t), hipMemcpyDeviceToHost, idx->stream));
     HIP_TRY(hipStreamSynchronize(idx->stream));
-    if (reverse_edges) *reverse_edges = (int64_t)st[0];
-    if (reverse_rejected) *reverse_rejected = (int64_t)st[1];
+    if (!h_ids || top_n == 0) return CORAL_OK;
+    // counting sort, most hits first, ids ascending within a count
+    uint32_t mx = 0;
+    for (int64_t i = 0; i < idx->n; ++i) mx = std::max(mx, hits[i]);
+    std::vector<int64_t> at((size_t)mx + 2, 0);  // at[h] = ids with more than h hits = where count h starts
+    for (int64_t i = 0; i < idx->n; ++i) ++at[hits[i]];
+    int64_t run = 0;
+    for (int64_t h = mx; h >= 0; --h) {
+        const int64_t c = at[(size_t)h];
+        at[(size_t)h] = run;
+        run += c;
+    }
+    for (int64_t i = 0; i < idx->n; ++i) {
+        const int64_t pos = at[hits[i]]++;
+        if (pos < top_n) h_ids[pos] = (int32_t)i;
+    }
     return CORAL_OK;
 }
 
@@ -201,47 +279,64 @@ int coral_build_connect_enhance(coral_index* idx, const coral_build_params* prm,
     if (first < 0 || first >= n) return fail(CORAL_ERR_STATE, "no node has neighbours yet: nothing to search from");
     if (deg[first] == 0) return fail(CORAL_ERR_ARG, "first_start_id %d has no neighbours", first);
     std::vector<int32_t> starts((size_t)prm->n_start);
-    if (iso.empty()) {
-        if (int rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data())) return rc;
-        return set_start_ids(idx, starts.data(), prm->n_start);
-    }
     const int64_t iso_num = (int64_t)iso.size();
-    const int64_t sb = std::min<int64_t>(prm->enhance_search_batch, iso_num);
-    int32_t *d_iso = nullptr, *d_res = nullptr;
-    float *d_iso_vec = nullptr, *d_res_d = nullptr;
-    auto release = [&]() { (void)hipFree(d_iso), (void)hipFree(d_res), (void)hipFree(d_iso_vec), (void)hipFree(d_res_d); };
     int rc = CORAL_OK;
-    auto ok = [&](hipError_t e, const char* what) {
-        if (e == hipSuccess) return true;
-        rc = fail(e == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE, "%s failed: %s", what, hipGetErrorString(e));
-        return false;
-    };
-    if (ok(hipMalloc(&d_iso, (size_t)iso_num * sizeof(int32_t)), "hipMalloc") &&
-        ok(hipMalloc(&d_iso_vec, (size_t)sb * dim * sizeof(float)), "hipMalloc") &&
-        ok(hipMalloc(&d_res, (size_t)sb * kb * sizeof(int32_t)), "hipMalloc") &&
-        ok(hipMalloc(&d_res_d, (size_t)sb * kb * sizeof(float)), "hipMalloc"))
-        ok(hipMemcpy(d_iso, iso.data(), (size_t)iso_num * sizeof(int32_t), hipMemcpyHostToDevice), "hipMemcpy");
-    for (int64_t i = 0; rc == CORAL_OK && i < iso_num; i += sb) {
-        const int batch = (int)std::min<int64_t>(sb, iso_num - i);
-        // src/enhance.cu:793-795: fresh entry points on the graph as it is now, then one search over the batch
-        if ((rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data()))) break;
-        if ((rc = set_start_ids(idx, starts.data(), prm->n_start))) break;
-        if (!ok(coral::launch_gather_rows(idx->d_vec, dim, d_iso + i, batch, d_iso_vec, st), "gather")) break;
-        coral_tuning tun{};
-        tun.policy = CORAL_POLICY_ROUNDS;
-        if ((rc = coral_search_prepare(idx, batch, prm->enhance_L, &tun))) break;
-        if ((rc = coral_search_gpu(idx, d_iso_vec, d_res, d_res_d, batch, kb, CORAL_POLICY_ROUNDS, 0, nullptr, nullptr)))
-            break;
-        for (int64_t j = 0; j < batch; j += prm->enhance_nap_batch) {
-            const int b1 = (int)std::min<int64_t>(prm->enhance_nap_batch, batch - j);
-            int64_t ins = 0, rej = 0;
-            if ((rc = coral_build_enhance_batch(idx, d_iso + i + j, d_res + (size_t)j * kb, d_res_d + (size_t)j * kb, b1, kb,
-                                                &ins, &rej)))
+    // One phase: per search batch fresh entry points on the graph as it is now (src/enhance.cu:793-795, 843), one
+    // search for the nodes' own vectors, then the rewiring per enhance_nap_batch nodes.
+    auto phase = [&](const std::vector<int32_t>& ids, bool top) {
+        const int64_t count = (int64_t)ids.size();
+        const int64_t sb = std::min<int64_t>(prm->enhance_search_batch, count);
+        int32_t *d_ids = nullptr, *d_res = nullptr;
+        float *d_vecs = nullptr, *d_res_d = nullptr;
+        auto ok = [&](hipError_t e, const char* what) {
+            if (e == hipSuccess) return true;
+            rc = fail(e == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE, "%s failed: %s", what,
+                      hipGetErrorString(e));
+            return false;
+        };
+        if (ok(hipMalloc(&d_ids, (size_t)count * sizeof(int32_t)), "hipMalloc") &&
+            ok(hipMalloc(&d_vecs, (size_t)sb * dim * sizeof(float)), "hipMalloc") &&
+            ok(hipMalloc(&d_res, (size_t)sb * kb * sizeof(int32_t)), "hipMalloc") &&
+            ok(hipMalloc(&d_res_d, (size_t)sb * kb * sizeof(float)), "hipMalloc"))
+            ok(hipMemcpy(d_ids, ids.data(), (size_t)count * sizeof(int32_t), hipMemcpyHostToDevice), "hipMemcpy");
+        for (int64_t i = 0; rc == CORAL_OK && i < count; i += sb) {
+            const int batch = (int)std::min<int64_t>(sb, count - i);
+            if ((rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data()))) break;
+            if ((rc = set_start_ids(idx, starts.data(), prm->n_start))) break;
+            if (!ok(coral::launch_gather_rows(idx->d_vec, dim, d_ids + i, batch, d_vecs, st), "gather")) break;
+            coral_tuning tun{};
+            tun.policy = CORAL_POLICY_ROUNDS;
+            if ((rc = coral_search_prepare(idx, batch, prm->enhance_L, &tun))) break;
+            if ((rc = coral_search_gpu(idx, d_vecs, d_res, d_res_d, batch, kb, CORAL_POLICY_ROUNDS, 0, nullptr, nullptr)))
                 break;
-            if (stats) stats->reverse_edges += ins, stats->reverse_rejected += rej;
+            for (int64_t j = 0; j < batch; j += prm->enhance_nap_batch) {
+                const int b1 = (int)std::min<int64_t>(prm->enhance_nap_batch, batch - j);
+                int64_t ins = 0, rej = 0;
+                rc = top ? coral_build_enhance_top_batch(idx, d_ids + i + j, d_res + (size_t)j * kb, d_res_d + (size_t)j * kb,
+                                                         b1, kb, &ins, &rej)
+                         : coral_build_enhance_batch(idx, d_ids + i + j, d_res + (size_t)j * kb, d_res_d + (size_t)j * kb, b1,
+                                                     kb, &ins, &rej);
+                if (rc) break;
+                if (stats && top) stats->top_reverse_edges += ins;
+                if (stats && !top) stats->reverse_edges += ins, stats->reverse_rejected += rej;
+            }
         }
+        (void)hipFree(d_ids), (void)hipFree(d_res), (void)hipFree(d_vecs), (void)hipFree(d_res_d);
+    };
+    if (iso_num > 0) phase(iso, false);
+    // src/enhance.cu:819-856: the nodes most clusters contain, as many as top_hit_num exceeds the isolated ones
+    int64_t top_n = rc == CORAL_OK && prm->top_hit_num > iso_num ? std::min<int64_t>(prm->top_hit_num - iso_num, n) : 0;
+    if (top_n > 0) {
+        if (prm->k_b > coral::kBuildMaxKb) return fail(CORAL_ERR_ARG, "k_b must be at most %d", coral::kBuildMaxKb);
+        std::vector<int32_t> top((size_t)top_n);
+        if ((rc = coral_build_top_hit_ids(idx, top_n, top.data(), nullptr))) return rc;
+        if (stats) stats->top_hit_nodes = top_n;
+        phase(top, true);
     }
-    release();
+    if (rc == CORAL_OK && iso_num == 0 && top_n == 0) {
+        if ((rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data()))) return rc;
+        rc = set_start_ids(idx, starts.data(), prm->n_start);
+    }
     return rc;
 }
 

@@ -81,6 +81,7 @@ void IndexGPU::load_config(const std::string& config_file) {
     if (json_number(text, "search_in_cpu", &v)) pc.search_in_cpu = (int)v;
     if (json_number(text, "need_discard", &v)) pc.need_discard = (int)v;
     if (json_number(text, "enhance_nap_batch", &v)) pc.enhance_nap_batch = (int)v;
+    if (json_number(text, "top_hit_num", &v)) pc.top_hit_num = (int)v;
     if (json_number(text, "enhance_search_batch", &v)) pc.enhance_search_batch = (int)v;
 }
 
@@ -177,6 +178,7 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     coral_build_params_default(&p);
     p.R = max_degree_, p.k_b = k_, p.batch = PC.batch, p.need_discard = PC.need_discard, p.connect_enhance = CE;
     p.enhance_search_batch = PC.enhance_search_batch, p.enhance_nap_batch = PC.enhance_nap_batch;
+    p.top_hit_num = PC.top_hit_num;
     p.n_start = PC.search_start_nodes_num;
     const std::string train_gt = parameters.Get<std::string>("train_gt_file", std::string("None"));
     if (train_gt != "None" && !train_gt.empty()) {

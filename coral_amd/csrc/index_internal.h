@@ -75,6 +75,12 @@ struct coral_index {
     size_t stage_rows = 0;
     int32_t* d_len = nullptr;  // found-list lengths of one enhancement batch
     size_t len_alloc = 0;
+    uint32_t* d_hits = nullptr;  // [n] clusters of this build that contain the node
+    // second enhancement phase: candidate lists (found + current row) of one batch and their found-part lengths
+    int32_t* d_top_ids_list = nullptr;
+    float* d_top_dists_list = nullptr;
+    int32_t* d_rev_len = nullptr;
+    size_t top_list_cells = 0, rev_len_alloc = 0;
     unsigned long long* d_build_stats = nullptr;  // [0] reverse edges inserted, [1] turned away, [2] ids out of range
 };
 

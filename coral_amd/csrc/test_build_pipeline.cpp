@@ -153,8 +153,8 @@ int main(int argc, char** argv) {
         const std::chrono::duration<double> diff = std::chrono::high_resolution_clock::now() - s;
         const coral_build_stats& b = index.last_build;
         std::cout << "batches: " << b.batches << ", isolated after the batches: " << b.isolated
-                  << ", reverse edges: " << b.reverse_edges << ", average degree: " << (double)b.edges / (double)base_num
-                  << std::endl;
+                  << ", reverse edges: " << b.reverse_edges << ", most-hit nodes rewired: " << b.top_hit_nodes
+                  << ", average degree: " << (double)b.edges / (double)base_num << std::endl;
         std::cout << "knn " << b.knn_s << " s, batch updates " << b.nap_s << " s, enhancement " << b.enhance_s << " s"
                   << std::endl;
         std::cout << "indexing time: " << diff.count() << std::endl;

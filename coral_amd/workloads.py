@@ -51,7 +51,7 @@ def config2(n=1000000, dim=200, Q=10000, A=100000, device="cuda", verbose=False)
     aux = synth.shifted_queries(A, dim, 2002, 2003, 2005)
     nbrs, starts, info = build_query_aware_graph(base, aux, "l2")
     return dict(name="%dx%d fp32 L2, R=32 query-aware graph (k_b=100, %d aux queries), %d queries, k=100" %
-                (n, dim, A, Q), base=base, queries=queries, nbrs=nbrs, starts=starts, metric="l2", k=100,
+                (n, dim, A, Q), base=base, queries=queries, aux=aux, nbrs=nbrs, starts=starts, metric="l2", k=100,
                 Ls=(256, 512), build=info)
 
 

@@ -196,7 +196,10 @@ typedef struct {
     int32_t n_start;              /* entry points: config.json "search_start_nodes_num" (16) */
     int32_t first_start_id;       /* first id of the farthest-point sampling (the reference draws it from
                                      std::random_device, src/start.cu:77-86); -1 = lowest id that has neighbours */
-    int32_t reserved[6];
+    int32_t top_hit_num;          /* config.json "top_hit_num": after the isolated nodes, the (top_hit_num - isolated)
+                                     nodes that most clusters contain are searched for and rewired too; 0 (the code's
+                                     default, src/index_gpu.cpp:78) = no such phase */
+    int32_t reserved[5];
 } coral_build_params;
 
 typedef struct {
@@ -209,6 +212,8 @@ typedef struct {
     int64_t reverse_edges;     /* isolated nodes inserted into rows of the nodes found for them */
     int64_t reverse_rejected;  /* ... turned away by a full row */
     int64_t edges;             /* sum of degrees at the end */
+    int64_t top_hit_nodes;     /* nodes the second enhancement phase went over */
+    int64_t top_reverse_edges; /* reverse edges of that phase */
 } coral_build_stats;
 
 /* the values of the reference's config.json and CLI defaults */
@@ -238,10 +243,24 @@ CORAL_API int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_i
  * points by coral_start_ids_fps on the graph as it is, one CORAL_POLICY_ROUNDS search (k = k_b, L = enhance_L) for
  * the isolated nodes' own vectors, then coral_build_enhance_batch per enhance_nap_batch.  The entry points of the
  * last search batch stay the index's start ids, as in the reference (fewer than n_start when fewer nodes can be
- * reached: an id is never listed twice).  Its second phase (top_hit_num most-hit nodes,
- * src/enhance.cu:819-856) is not built: it is off by the code's default (src/index_gpu.cpp:78) and reads past its
- * id array whenever top_hit_num exceeds n. */
+ * reached: an id is never listed twice).  Second phase (src/enhance.cu:819-856) when params->top_hit_num exceeds the
+ * number of isolated nodes: the (top_hit_num - isolated) nodes of coral_build_top_hit_ids, capped at n (the reference
+ * reads past its id array beyond that), go through the same search and coral_build_enhance_top_batch. */
 CORAL_API int coral_build_connect_enhance(coral_index* idx, const coral_build_params* params, coral_build_stats* stats);
+
+/* The five-argument GPUFuncs::enhance_neibor_aware_gpu (src/enhance.cu:632-658, 58-129): d_top_ids [batch] nodes that
+ * have rows, d_knn_ids / d_knn_dists [batch][k] what the search found for their vectors (the node itself included, as
+ * in the reference).  A node's candidates are its found list followed by its current row; the found part inserts
+ * reverse edges like coral_build_enhance_batch, and the node's row is rebuilt from all candidates.  Rows are read as
+ * they were before the batch (the reference reads them while the same kernel changes them). */
+CORAL_API int coral_build_enhance_top_batch(coral_index* idx, const int32_t* d_top_ids, const int32_t* d_knn_ids,
+                                            const float* d_knn_dists, int32_t batch, int32_t k, int64_t* reverse_edges,
+                                            int64_t* reverse_rejected);
+
+/* get_top_hit_nodes (src/knn.cu:140-150): the top_n ids by the number of clusters of this build that contain them
+ * (counted by coral_build_nap_batch as src/knn.cu:60-73 does), most first, equal counts by ascending id.  h_hits
+ * (optional) receives the n counts. */
+CORAL_API int coral_build_top_hit_ids(coral_index* idx, int64_t top_n, int32_t* h_ids, uint32_t* h_hits);
 
 /* IndexGPU::BuildGPU: begin; exact k_b-NN of the A auxiliary queries (host, [A][dim]; what the reference asks faiss
  * for, src/knn.cu:174-193) in order, `batch` at a time through coral_build_nap_batch; then the enhancement (or, with

@@ -48,6 +48,7 @@ struct ProConfig {
     int need_discard = 1;
     int enhance_nap_batch = 4096;
     int enhance_search_batch = 524288;
+    int top_hit_num = 0;  // include/uni.h:124; the shipped config.json sets 5000000
 };
 CORAL_API ProConfig& GetProConfig();
 #define PC (::efanna2e::GetProConfig())

@@ -224,6 +224,30 @@ def enhance_batch(base, state, iso_ids, knn_ids, knn_dists, metric=L2):
     return stats
 
 
+def enhance_top_batch(base, state, top_ids, knn_ids, knn_dists, metric=L2):
+    """One batch of the second enhancement phase (most-hit nodes): candidates = found list + current row."""
+    base, top_ids, knn_ids, knn_dists = _f32(base), _i32(top_ids), _i32(knn_ids), _f32(knn_dists)
+    stats = np.zeros(3, np.int64)
+    fn = lib().oracle_enhance_top_batch
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+    rc = fn(_p(base), base.shape[0], base.shape[1], metric, state.nbrs.shape[1], _p(state.nbrs), _p(state.dists),
+            _p(state.deg), _p(top_ids), _p(knn_ids), _p(knn_dists), top_ids.size, knn_ids.shape[1], _p(stats))
+    if rc:
+        raise MemoryError("oracle_enhance_top_batch")
+    return stats
+
+
+def top_hit_ids(hits, top_n):
+    hits = np.ascontiguousarray(hits, dtype=np.uint32)
+    out = np.empty(top_n, np.int32)
+    fn = lib().oracle_top_hit_ids
+    fn.restype, fn.argtypes = None, [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+    fn(_p(hits), hits.size, top_n, _p(out))
+    return out
+
+
 def max_threads():
     fn = lib().oracle_max_threads
     fn.restype, fn.argtypes = C.c_int, []

@@ -18,8 +18,9 @@
  *   - exact kNN by brute force under (distance, id), in fp64 or in one of the fp32 orders above: what the
  *     reference asks faiss for (tests/comp_gt.cpp:119-176, src/knn.cu:174-193)
  *   - entry points by farthest-point sampling in hop distance: src/start.cu:10-145
- *   - graph construction: one batch of neighbour-aware pruning (src/upd_gpu.cu:12-303) and one batch of the
- *     connectivity enhancement (src/enhance.cu:131-208, 334-575, 660-689); see the section further down
+ *   - graph construction: one batch of neighbour-aware pruning (src/upd_gpu.cu:12-303), one batch of the
+ *     connectivity enhancement for isolated nodes (src/enhance.cu:131-208, 334-575, 660-689) and for the most-hit
+ *     nodes (src/enhance.cu:58-129, 632-658; their choice: src/knn.cu:140-150); see the section further down
  *
  * Pinning status (what fixes each function besides this text):
  *   - oracle_dist ORDER_CPU_AVX512, oracle_queue_*, oracle_search_A: bit-exact
@@ -38,7 +39,7 @@
  *     hand-computed traversals on path/ring graphs; an independent
  *     set-based pure-Python simulator on tiny inputs.
  *   - oracle_bruteforce*: fp64 closed form, exact lattice cases with ties, top-k of a full sort.
- *   - oracle_fps, oracle_nap_batch, oracle_enhance_batch: no executable reference (CUDA, faiss, outcomes that
+ *   - oracle_fps, oracle_nap_batch, oracle_enhance_batch, oracle_enhance_top_batch: no executable reference (CUDA, faiss, outcomes that
  *     depend on thread timing).  Pinned by code reading, hand-computed cases, the invariants of the occlusion
  *     rule, an all-pairs brute force (FPS) and independent pure-Python statements on small random inputs.
  *
@@ -905,9 +906,10 @@ ORACLE_API int oracle_nap_batch(const float* base, int64_t n, int dim, int metri
  *   2. the isolated node's own row: its found list through the occlusion rule, filled with discarded ones
  *      (src/enhance.cu:334-380, 519-575).
  * stats (optional): [0] reverse edges inserted, [1] claims rejected by a full row, [2] distance evaluations. */
-ORACLE_API int oracle_enhance_batch(const float* base, int64_t n, int dim, int metric, int R, int32_t* nbrs,
-                                    float* dists, int32_t* deg, const int32_t* iso_ids, const int32_t* knn_ids,
-                                    const float* knn_dists, int batch, int kn, int64_t* stats) {
+/* rev_len (optional) [batch]: only the first rev_len[b] entries of list b claim nodes and insert reverse edges */
+static int enhance_core(const float* base, int64_t n, int dim, int metric, int R, int32_t* nbrs, float* dists,
+                        int32_t* deg, const int32_t* iso_ids, const int32_t* knn_ids, const float* knn_dists, int batch,
+                        int kn, const int32_t* rev_len, int64_t* stats) {
     uint8_t* claimed = (uint8_t*)calloc((size_t)n, 1);
     cand_t* c = (cand_t*)malloc((size_t)kn * sizeof(cand_t));
     if (!claimed || !c) return -1;
@@ -915,7 +917,8 @@ ORACLE_API int oracle_enhance_batch(const float* base, int64_t n, int dim, int m
     for (int b = 0; b < batch; ++b) {
         const int32_t iso = iso_ids[b];
         const float* iv = base + (size_t)iso * dim;
-        for (int i = 0; i < kn; ++i) {
+        const int nrev = rev_len ? rev_len[b] : kn;
+        for (int i = 0; i < nrev; ++i) {
             const int32_t v = knn_ids[(size_t)b * kn + i];
             if (v < 0) break;
             const float vd = knn_dists[(size_t)b * kn + i];
@@ -975,6 +978,61 @@ ORACLE_API int oracle_enhance_batch(const float* base, int64_t n, int dim, int m
     if (stats) stats[0] = inserted, stats[1] = rejected, stats[2] = evals;
     free(claimed), free(c);
     return 0;
+}
+
+ORACLE_API int oracle_enhance_batch(const float* base, int64_t n, int dim, int metric, int R, int32_t* nbrs,
+                                    float* dists, int32_t* deg, const int32_t* iso_ids, const int32_t* knn_ids,
+                                    const float* knn_dists, int batch, int kn, int64_t* stats) {
+    return enhance_core(base, n, dim, metric, R, nbrs, dists, deg, iso_ids, knn_ids, knn_dists, batch, kn, NULL, stats);
+}
+
+/* One batch of the second enhancement phase, over the nodes that most clusters contain ("top hit" nodes): the
+ * five-argument GPUFuncs::enhance_neibor_aware_gpu (src/enhance.cu:632-658) with its build_candidate_kernel
+ * (src/enhance.cu:58-129).  top_ids [batch] already have rows; knn_ids / knn_dists [batch][k] is what the beam search
+ * found for their vectors (the node itself is normally the first entry, at distance 0, and stays a candidate as in
+ * the reference).  A node's candidates are its found list followed by its current row with the stored distances;
+ * only the found part claims nodes and inserts reverse edges; the node's row is rebuilt from all candidates by the
+ * rule of the first phase.  The reference reads the current rows while other thread blocks of the same kernel
+ * insert reverse edges into them; here every row is read as it was before the batch.  It also reads all R cells
+ * of a row whatever its degree; here the deg valid ones. */
+ORACLE_API int oracle_enhance_top_batch(const float* base, int64_t n, int dim, int metric, int R, int32_t* nbrs,
+                                        float* dists, int32_t* deg, const int32_t* top_ids, const int32_t* knn_ids,
+                                        const float* knn_dists, int batch, int k, int64_t* stats) {
+    const int kn = k + R;
+    int32_t* ids = (int32_t*)malloc((size_t)batch * kn * sizeof(int32_t));
+    float* ds = (float*)malloc((size_t)batch * kn * sizeof(float));
+    int32_t* rev = (int32_t*)malloc((size_t)batch * sizeof(int32_t));
+    if (!ids || !ds || !rev) return -1;
+    for (int b = 0; b < batch; ++b) {
+        const int32_t t = top_ids[b];
+        int m = 0;
+        for (int i = 0; i < k; ++i) {
+            if (knn_ids[(size_t)b * k + i] < 0) break;
+            ids[(size_t)b * kn + m] = knn_ids[(size_t)b * k + i];
+            ds[(size_t)b * kn + m] = knn_dists[(size_t)b * k + i];
+            ++m;
+        }
+        rev[b] = m;
+        for (int j = 0; j < deg[t]; ++j, ++m) {
+            ids[(size_t)b * kn + m] = nbrs[(size_t)t * R + j];
+            ds[(size_t)b * kn + m] = dists[(size_t)t * R + j];
+        }
+        for (; m < kn; ++m) ids[(size_t)b * kn + m] = -1, ds[(size_t)b * kn + m] = 0.0f;
+    }
+    const int rc = enhance_core(base, n, dim, metric, R, nbrs, dists, deg, top_ids, ids, ds, batch, kn, rev, stats);
+    free(ids), free(ds), free(rev);
+    return rc;
+}
+
+/* get_top_hit_nodes (src/knn.cu:140-150): the top_n ids by number of clusters that contain them (hits), most first;
+ * equal counts keep ascending id (the reference sorts (hits, iota) pairs with a stable descending radix sort). */
+ORACLE_API void oracle_top_hit_ids(const uint32_t* hits, int64_t n, int64_t top_n, int32_t* out) {
+    uint32_t mx = 0;
+    for (int64_t i = 0; i < n; ++i) mx = hits[i] > mx ? hits[i] : mx;
+    int64_t w = 0;
+    for (int64_t h = mx; h >= 0 && w < top_n; --h)
+        for (int64_t i = 0; i < n && w < top_n; ++i)
+            if (hits[i] == (uint32_t)h) out[w++] = (int32_t)i;
 }
 
 ORACLE_API int oracle_max_threads(void) {

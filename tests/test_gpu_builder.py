@@ -114,8 +114,10 @@ def test_randomised_shapes_of_both_steps_equal_the_oracle(orc):
         idx = capi.Index(base, None, None, metric=metric)
         idx.build_begin(R)
         st = orc.GraphState(n, R)
+        all_knn = []
         for it in range(3):
             knn = np.stack([rng.choice(linked_n, kb, replace=False) for _ in range(batch)]).astype(np.int32)
+            all_knn.append(knn)
             t_knn = dev(knn)
             idx.build_nap_batch(t_knn.data_ptr(), batch, kb, fill)
             orc.nap_batch(base, st, knn, metric=metric, need_discard=fill)
@@ -133,6 +135,24 @@ def test_randomised_shapes_of_both_steps_equal_the_oracle(orc):
             stats = orc.enhance_batch(base, st, iso, ids, dd, metric=metric)
             assert (ins, rej) == (stats[0], stats[1])
             assert_same_state(idx, st)
+        # the second-phase step over some linked nodes: what is nearest among the linked (themselves first) + own row
+        linked = np.where(st.deg > 0)[0].astype(np.int32)
+        top = rng.choice(linked, min(40, linked.size), replace=False).astype(np.int32)
+        k2 = int(min(linked.size, rng.choice([1, 6, 30, 100, 128])))
+        ids, dd = orc.bruteforce(base[linked], base[top], k2, metric, order=SEQ)
+        ids = linked[ids]
+        if k2 > 2:
+            ids[0, k2 // 2:] = -1
+        t_top, t_ids, t_dd = dev(top), dev(ids), dev(dd)
+        ins, rej = idx.build_enhance_top_batch(t_top.data_ptr(), t_ids.data_ptr(), t_dd.data_ptr(), top.size, k2)
+        stats = orc.enhance_top_batch(base, st, top, ids, dd, metric=metric)
+        assert (ins, rej) == (stats[0], stats[1])
+        assert_same_state(idx, st)
+        got_ids, got_hits = idx.build_top_hit_ids(min(n, 50))
+        want_hits = np.zeros(n, np.uint32)
+        for knn in all_knn:
+            np.add.at(want_hits, knn.ravel(), 1)
+        assert np.array_equal(got_hits, want_hits) and got_ids.tolist() == orc.top_hit_ids(want_hits, min(n, 50)).tolist()
         idx.close()
 
 
@@ -140,39 +160,53 @@ def oracle_pipeline(orc, base, aux, metric, p):
     """IndexGPU::BuildGPU composed from the oracle's pieces, in the order coral_build_graph documents."""
     n = base.shape[0]
     st = orc.GraphState(n, p.R)
+    hits = np.zeros(n, np.uint32)
     for a0 in range(0, aux.shape[0], p.batch):
         knn, _ = orc.bruteforce(base, aux[a0:a0 + p.batch], p.k_b, metric, order=SEQ)
+        np.add.at(hits, knn.ravel(), 1)
         orc.nap_batch(base, st, knn, metric=metric, need_discard=p.need_discard)
     iso = np.where(st.deg == 0)[0].astype(np.int32)
     first = int(np.where(st.deg > 0)[0][0]) if p.first_start_id < 0 else p.first_start_id
     starts = None
-    if p.connect_enhance:
-        for i in range(0, iso.size, p.enhance_search_batch):
-            part = iso[i:i + p.enhance_search_batch]
+
+    def phase(nodes, step):
+        nonlocal starts
+        for i in range(0, nodes.size, p.enhance_search_batch):
+            part = nodes[i:i + p.enhance_search_batch]
             starts = orc.fps(st.nbrs, first, p.n_start)
             prob = orc.Problem(base, st.nbrs.copy(), starts)
             ids, dd, _, _ = orc.search_B(prob, base[part], p.k_b, p.enhance_L, metric=metric, start_order=WAVE64,
                                          nbr_order=WAVE64)
             for j in range(0, part.size, p.enhance_nap_batch):
                 sl = slice(j, j + p.enhance_nap_batch)
-                orc.enhance_batch(base, st, part[sl], ids[sl], dd[sl], metric=metric)
+                step(base, st, part[sl], ids[sl], dd[sl], metric=metric)
+
+    if p.connect_enhance:
+        phase(iso, orc.enhance_batch)
+        if p.top_hit_num > iso.size:  # the second phase: the nodes most clusters contain
+            phase(orc.top_hit_ids(hits, min(p.top_hit_num - iso.size, n)), orc.enhance_top_batch)
     if starts is None:
         starts = orc.fps(st.nbrs, first, p.n_start)
     return st, starts, iso.size
 
 
-@pytest.mark.parametrize("metric,ce,seed", [(capi.L2, 1, 0), (capi.IP, 1, 1), (capi.L2, 0, 2)])
-def test_whole_construction_equals_the_oracle_pipeline(orc, metric, ce, seed):
+@pytest.mark.parametrize("metric,ce,seed,top_hit_num", [(capi.L2, 1, 0, 0), (capi.IP, 1, 1, 0), (capi.L2, 0, 2, 0),
+                                                        (capi.L2, 1, 3, 9000), (capi.IP, 1, 4, 1000000)])
+def test_whole_construction_equals_the_oracle_pipeline(orc, metric, ce, seed, top_hit_num):
     n, dim, A = 12000, 48, 900
     base = base_of(n, dim, 300 + seed, metric)
     aux = make_queries(A, dim, 400 + seed, "ip" if metric == capi.IP else "l2")
     p = capi.build_params(R=16, k_b=24, batch=128, connect_enhance=ce, enhance_search_batch=5000,
-                          enhance_nap_batch=700, enhance_L=64, n_start=8)
+                          enhance_nap_batch=700, enhance_L=64, n_start=8, top_hit_num=top_hit_num)
     idx = capi.Index(base, None, None, metric=metric)
     stats = idx.build_graph(aux, p)
     nbrs, dists, deg, starts = idx.get_graph(with_build_state=True)
     st, want_starts, iso_n = oracle_pipeline(orc, base, aux, metric, p)
     assert stats.isolated == iso_n and iso_n > 1000
+    assert stats.top_hit_nodes == (min(top_hit_num - iso_n, n) if top_hit_num > iso_n else 0)
+    if top_hit_num:
+        assert stats.top_hit_nodes > 0 and stats.top_reverse_edges > 0
+        print("second phase over %d nodes, %d reverse edges" % (stats.top_hit_nodes, stats.top_reverse_edges), flush=True)
     assert stats.batches == (A + p.batch - 1) // p.batch
     assert np.array_equal(deg, st.deg) and np.array_equal(nbrs, st.nbrs) and dists.tobytes() == st.dists.tobytes()
     assert starts.tolist() == want_starts.tolist()

@@ -311,3 +311,115 @@ def test_enhance_batches_match_the_python_statement(orc, metric, seed):
         assert np.array_equal(st.deg, dg) and np.array_equal(st.nbrs, nb) and st.dists.tobytes() == ds.tobytes()
         linked = np.where(st.deg > 0)[0]
     assert (st.deg[300:] > 0).all()
+
+
+# ------------------------------------------------------------------ second enhancement phase: the most-hit nodes
+
+def test_top_hit_ids_are_ordered_by_hits_then_id(orc):
+    rng = np.random.RandomState(5)
+    hits = rng.randint(0, 6, 500).astype(np.uint32)
+    want = np.lexsort((np.arange(500), -hits.astype(np.int64)))
+    for top_n in (1, 37, 500):
+        assert orc.top_hit_ids(hits, top_n).tolist() == want[:top_n].tolist()
+    assert orc.top_hit_ids(np.array([0, 3, 3, 1], np.uint32), 3).tolist() == [1, 2, 3]
+
+
+def test_enhance_top_candidates_are_the_found_list_and_the_current_row(orc):
+    #            0    1    2    3     4     5
+    base = line([0.0, 1.0, 2.0, 4.0, -1.0, 8.0])
+    rows = {0: [(1, 1.0), (3, 16.0)], 1: [(0, 1.0)], 2: [(1, 1.0)], 3: [(2, 4.0)], 4: [(0, 1.0)], 5: [(3, 16.0)]}
+    st = state_from_rows(orc, 6, 3, rows)
+    # node 0 searched for itself: found 0 (itself, 0), 4 (1), 1 (1), 2 (4)
+    knn = np.array([[0, 4, 1, 2]], np.int32)
+    kd = np.array([[0.0, 1.0, 1.0, 4.0]], np.float32)
+    stats = orc.enhance_top_batch(base, st, [0], knn, kd)
+    # reverse edges, found part only (0, 4, 1, 2; never 3, which is only in the current row):
+    #   into the row of 0 itself (then overwritten by its rebuilt row), of 4: [0 (1)] -> 0 in front of the equal entry,
+    #   of 1: [0 (1)] -> in front, of 2: [1 (1)] -> behind
+    assert st.nbrs[4].tolist() == [0, 0, -1] and st.nbrs[1].tolist() == [0, 0, -1] and st.nbrs[2].tolist() == [1, 0, -1]
+    assert st.nbrs[3].tolist() == [2, -1, -1]
+    assert stats[0] == 4
+    # own row from [0 (0), 4 (1), 1 (1), 2 (4)] + current row [1 (1), 3 (16)], sorted, ties in that order:
+    #   0 (itself) kept, occludes nobody (its distance to j equals the pivot's); 4 kept; 1: d(4,1)=4 > 1 kept; full.
+    assert st.nbrs[0].tolist() == [0, 4, 1] and st.dists[0].tolist() == [0.0, 1.0, 1.0] and st.deg[0] == 3
+    # with a wider row the second listing of 1 is dropped, 2 (d(1,2)=1 < 4) and 3 (d(1,3)=9 < 16) are ruled out and
+    # fill the row in distance order
+    st = state_from_rows(orc, 6, 6, rows)
+    orc.enhance_top_batch(base, st, [0], knn, kd)
+    assert st.nbrs[0].tolist() == [0, 4, 1, 2, 3, -1] and st.deg[0] == 5
+
+
+def test_enhance_top_rows_are_read_as_of_before_the_batch(orc):
+    #            0    1    2     3
+    base = line([0.0, 1.0, 3.0, -2.0])
+    rows = {0: [(1, 1.0)], 1: [(0, 1.0)], 2: [(1, 4.0)], 3: [(0, 4.0)]}
+    st = state_from_rows(orc, 4, 4, rows)
+    # both 0 and 1 are processed in one batch; 0 found 1 and 1 found 0: each gets a reverse edge from the other before
+    # its row is rebuilt from (found list + the row of before the batch), which holds the other anyway
+    knn = np.array([[0, 1, 3], [1, 0, 2]], np.int32)
+    kd = np.array([[0.0, 1.0, 4.0], [0.0, 1.0, 4.0]], np.float32)
+    orc.enhance_top_batch(base, st, [0, 1], knn, kd)
+    # node 0: [0 (0), 1 (1), 3 (4)] + [1 (1)]: 0 kept, 1 kept, 3: d(1,3)=9 > 4 kept, second 1 dropped
+    assert st.nbrs[0].tolist() == [0, 1, 3, -1]
+    # node 1: [1 (0), 0 (1), 2 (4)] + [0 (1)]: 1, 0 kept, 2: d(0,2)=9 > 4 kept
+    assert st.nbrs[1].tolist() == [1, 0, 2, -1]
+    # 3 was claimed by node 0 (first in the batch), 2 by node 1
+    assert st.nbrs[3].tolist() == [0, 0, -1, -1] and st.nbrs[2].tolist() == [1, 1, -1, -1]
+
+
+def py_enhance_top_batch(orc, base, nbrs, dists, deg, top_ids, knn_ids, knn_dists, R, metric):
+    k = knn_ids.shape[1]
+    lists = []
+    for b, t in enumerate(top_ids):  # every list from the rows of before the batch
+        found = [(int(v), float(d)) for v, d in zip(knn_ids[b], knn_dists[b])]
+        if any(v < 0 for v, _ in found):
+            found = found[:[v < 0 for v, _ in found].index(True)]
+        lists.append((found, [(int(nbrs[t, j]), float(dists[t, j])) for j in range(deg[t])]))
+    rev_ids = np.full((len(top_ids), k), -1, np.int32)
+    rev_d = np.zeros((len(top_ids), k), np.float32)
+    for b, (found, _) in enumerate(lists):
+        for i, (v, d) in enumerate(found):
+            rev_ids[b, i], rev_d[b, i] = v, d
+    own = {}
+    scratch = (nbrs.copy(), dists.copy(), deg.copy())
+    py_enhance_batch(orc, base, nbrs, dists, deg, top_ids, rev_ids, rev_d, R, metric)  # reverse edges (+ rows, redone below)
+    for b, t in enumerate(top_ids):
+        found, row = lists[b]
+        own[int(t)] = py_prune(orc, base, [(d, v) for v, d in found + row], R, metric, True)
+    for t, row in own.items():
+        nbrs[t], dists[t] = -1, 0
+        for j, (u, d) in enumerate(row):
+            nbrs[t, j], dists[t, j] = u, d
+        deg[t] = len(row)
+    del scratch
+
+
+@pytest.mark.parametrize("metric,seed", [(0, 0), (1, 1)])
+def test_enhance_top_batches_match_the_python_statement(orc, metric, seed):
+    rng = np.random.RandomState(10 + seed)
+    n, dim, R, k = 300, 8, 5, 8
+    base = synth.gaussian_matrix(60 + seed, n, dim)
+    if metric == 1:
+        base = synth.normalize_rows(base)
+    sign = 1.0 if metric == 0 else -1.0
+    st = orc.GraphState(n, R)
+    for t in range(10):
+        knn = np.stack([rng.choice(n, 7, replace=False) for _ in range(25)]).astype(np.int32)
+        orc.nap_batch(base, st, knn, metric=metric, need_discard=bool(t % 2))
+    linked = np.where(st.deg > 0)[0]
+    nb, ds, dg = st.nbrs.copy(), st.dists.copy(), st.deg.copy()
+    for rep in range(2):
+        top = rng.choice(linked, 40, replace=False).astype(np.int32)
+        ids = np.empty((40, k), np.int32)
+        dd = np.empty((40, k), np.float32)
+        for i, p in enumerate(top):  # the exact nearest linked nodes (the node itself first) stand in for the search
+            d = np.array([orc.dist(base[p], base[v], metric, SEQ) for v in linked], np.float32)
+            o = np.argsort(sign * d, kind="stable")[:k]
+            ids[i], dd[i] = linked[o], d[o]
+        assert (ids[:, 0] == top).all()
+        ids[5, 6:] = -1
+        orc.enhance_top_batch(base, st, top, ids, dd, metric=metric)
+        py_enhance_top_batch(orc, base, nb, ds, dg, top, ids, dd, R, metric)
+        assert np.array_equal(st.deg, dg) and np.array_equal(st.nbrs, nb) and st.dists.tobytes() == ds.tobytes()
+    # every rebuilt row starts with the node itself (distance 0 sorts first; for IP the self product is the largest)
+    assert all(st.nbrs[t, 0] == t for t in top)
