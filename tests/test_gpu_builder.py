@@ -265,7 +265,8 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     formats.fbin_write(work / "query.fbin", q)
     gt, _ = orc.bruteforce(base, q, k)
     formats.gt_write(work / "gt.bin", gt)
-    (work / "config.json").write_text('{"batch": 256, "enhance_nap_batch": 1000, "search_start_nodes_num": 8}')
+    (work / "config.json").write_text('{"batch": 256, "enhance_nap_batch": 1000, "search_start_nodes_num": 8, '
+                                      '"top_hit_num": 20000}')
     cli = os.path.join(root, "coral_amd", "lib", "test_build_pipeline")
     args = [cli, "--data_type", "float", "--dist", "l2", "--dataset", "syn", "--base_data_path", str(work / "base.fbin"),
             "--sampled_query_data_path", str(work / "aux.fbin"), "--M_pjbp", "16", "--k", "24", "--CE", "1",
@@ -280,7 +281,8 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     nbrs, dists = formats.graph_dir_read(index_dir, n, 16, want_dists=True)
     starts = formats.start_ids_read(index_dir)
     # the same construction through the C ABI
-    p = capi.build_params(R=16, k_b=24, batch=256, enhance_nap_batch=1000, n_start=8)
+    assert "most-hit nodes rewired: " in r.stdout and "most-hit nodes rewired: 0," not in r.stdout
+    p = capi.build_params(R=16, k_b=24, batch=256, enhance_nap_batch=1000, n_start=8, top_hit_num=20000)
     idx = capi.Index(base, None, None)
     idx.build_graph(aux, p)
     want_nbrs, want_dists, deg, want_starts = idx.get_graph(with_build_state=True)
