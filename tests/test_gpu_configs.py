@@ -151,6 +151,17 @@ def big_case(orc, n, dim, Qs, L, k, tomb_seed=None, built=False):
     if mask is not None:
         dead = (mask[ids >> 5] >> (ids & 31).astype(np.uint32)) & 1
         assert not dead.any()
+    # the CPU path's traversal at this size (a wavefront per query while n bytes per query slot fit the memory
+    # budget, else a workgroup per query)
+    Qb = min(max(Qs), 10000)
+    ids, dists, st = idx.search(q[:Qb], k, L, policy=capi.POLICY_BEST_FIRST, have_delete=mask is not None)
+    cnt = idx.query_counters(Qb)
+    B = st.expansions * 128 + st.dist_evals * dim * 4 + Qb * (dim * 4 + k * 8)
+    print("n=%d Q=%d best-first: %.0f QPS, %.0f GB/s algorithmic" % (n, Qb, Qb / st.kernel_s, B / st.kernel_s / 1e9),
+          flush=True)
+    sub = np.arange(0, Qb, max(1, Qb // 48))
+    oi, od, os_, _ = orc.search_A(prob, q[sub], k, L, order=WAVE64)
+    assert np.array_equal(ids[sub], oi) and dists[sub].tobytes() == od.tobytes() and np.array_equal(cnt[sub], os_)
     idx.close()
 
 
