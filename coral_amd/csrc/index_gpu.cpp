@@ -229,7 +229,7 @@ void IndexGPU::SetDeleted(const uint32_t* mask_words) {
 Test_Result IndexGPU::run(const float* queries, int num, int L, int* ids_res, float* dists_res) {
     if (!index_) throw std::runtime_error("Search before RunPrepare");
     coral_stats st;
-    if (coral_search(index_, queries, num, k_, L, policy_, have_delete_ ? 1 : 0, ids_res, dists_res, &st))
+    if (coral_search(index_, queries, num, k_, L, GetPolicy(), have_delete_ ? 1 : 0, ids_res, dists_res, &st))
         raise("Search");
     Test_Result tr(-1, (size_t)st.hops, (float)st.time_s);
     tr.expansions = (size_t)st.expansions, tr.dist_evals = (size_t)st.dist_evals;
@@ -275,7 +275,7 @@ Test_Result IndexGPU::Search_and_Verify(const float* queries, const int* gts, in
     }
     coral_stats st;
     int64_t hits = 0;
-    if (coral_search_gpu(index_, d_q, d_ids, nullptr, num, k_, policy_, have_delete_ ? 1 : 0, nullptr, &st) ||
+    if (coral_search_gpu(index_, d_q, d_ids, nullptr, num, k_, GetPolicy(), have_delete_ ? 1 : 0, nullptr, &st) ||
         coral_search_verify(index_, d_ids, d_gt, num, k_, &hits)) {
         release();
         raise("Search_and_Verify");

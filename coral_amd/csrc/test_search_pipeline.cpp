@@ -8,7 +8,8 @@
 //   --log_file --res_file --recall_thres --max_recall --max_hop
 // plus -T / --num_threads, which the reference documents (README.md:117) but
 // does not register; it is accepted and ignored.
-// Extensions: --policy {rounds,best_first}, --index_dir <dir> (overrides the
+// Extensions: --policy {auto,rounds,best_first} (auto: rounds up to 10 010 000 nodes, best-first above, the
+// reference's choice of GPU or CPU search by size, src/index_gpu.cpp:257), --index_dir <dir> (overrides the
 // derived ../indexes/<dataset>_<dist>_<R>_<thres>_<CE> path), --index_prefix
 // and --evaluation_prefix (default ../indexes/ and ../evaluation/),
 // --device_recall 1 (recall through IndexGPU::Search_and_Verify, the loop of
@@ -52,7 +53,7 @@ const cli::Option kOptions[] = {
     {"CE", false, false, "1", "Use connectivity enhancement or not"},
     {"index_type", false, false, "", ""},
     {"num_threads", false, false, "0", "accepted for compatibility, unused"},
-    {"policy", false, false, "rounds", "traversal <rounds/best_first>"},
+    {"policy", false, false, "auto", "traversal <auto/rounds/best_first>; auto = by index size, as the reference"},
     {"index_dir", false, false, "", "index directory (overrides the derived name)"},
     {"index_prefix", false, false, "../indexes/", "directory holding index directories"},
     {"evaluation_prefix", false, false, "../evaluation/", "directory receiving the CSV"},
@@ -164,10 +165,13 @@ int main(int argc, char** argv) {
         const std::string policy = str("policy");
         if (policy == "best_first")
             index.SetPolicy(CORAL_POLICY_BEST_FIRST);
-        else if (policy != "rounds") {
+        else if (policy == "rounds")
+            index.SetPolicy(CORAL_POLICY_ROUNDS);
+        else if (policy != "auto") {
             std::cerr << "unknown policy: " << policy << '\n';
             return -1;
         }
+        std::cout << "traversal: " << (index.GetPolicy() == CORAL_POLICY_BEST_FIRST ? "best_first" : "rounds") << std::endl;
 
         std::cout << "k: " << k << std::endl;
         std::vector<int> res((size_t)q_pts * k, 0);

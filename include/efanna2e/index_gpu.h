@@ -118,7 +118,12 @@ class CORAL_API IndexGPU {
     // CORAL_POLICY_BEST_FIRST is the traversal of GPUFuncs::search_in_cpu; it starts from every start id of the index,
     // where the CPU path takes the first search_start_nodes_num of them (src/search_in_cpu.cpp:26, 74-79): the same
     // set whenever graph.search_start_ids holds that many ids, as the builder writes it
+    // Unless named here, the traversal is the one the reference would run for an index of this size: the CUDA kernel's
+    // rounds up to GPU_N = 10 010 000 nodes, the CPU path's best-first above (src/index_gpu.cpp:257, include/uni.h:70).
     void SetPolicy(int coral_policy) { policy_ = coral_policy; }
+    int GetPolicy() const {
+        return policy_ >= 0 ? policy_ : (nd_ > 10010000 ? CORAL_POLICY_BEST_FIRST : CORAL_POLICY_ROUNDS);
+    }
     // tombstones (src/update.cu:406-412): ceil(n/32) words, or nullptr to clear
     void SetDeleted(const uint32_t* mask_words);
     // as Search, also returning distances (num*k floats)
@@ -139,7 +144,7 @@ class CORAL_API IndexGPU {
     DIST_METRIC metric_ = DIST_METRIC::L2_;
     Parameters parameters_;
     int k_ = 0, max_degree_ = 32;
-    int policy_ = CORAL_POLICY_ROUNDS;
+    int policy_ = -1;  // -1: by size, see GetPolicy
     bool have_delete_ = false;
     float* h_base_ = nullptr;
     std::vector<int> start_ids_;

@@ -313,6 +313,7 @@ def test_cli_end_to_end(orc, tmp_path):
     r = subprocess.run(args + ["--index_type", "roar"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
     assert (work / "evaluation" / "search" / "roar_syn_l2_32.csv").exists()
+    assert "traversal: rounds" in r.stdout  # the reference's choice for an index of this size
     rprob = orc.Problem(base, roar, np.array([123], np.int32))
     oi, _, os_, _ = orc.search_B(rprob, q, k, 64, start_order=WAVE64, nbr_order=WAVE64)
     row = [l for l in r.stdout.splitlines() if l.startswith("64\t")][0].split()
@@ -321,7 +322,7 @@ def test_cli_end_to_end(orc, tmp_path):
     # best-first policy through the same driver
     r = subprocess.run(args + ["--policy", "best_first"], cwd=work / "cwd", capture_output=True, text=True,
                        timeout=120)
-    assert r.returncode == 0
+    assert r.returncode == 0 and "traversal: best_first" in r.stdout
     oi, _, os_, _ = orc.search_A(prob, q, k, 32, order=WAVE64)
     row = [l for l in r.stdout.splitlines() if l.startswith("32\t")][0].split()
     assert abs(float(row[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
