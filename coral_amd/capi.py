@@ -40,7 +40,8 @@ class Stats(C.Structure):
 
 class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
-                ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("reserved", C.c_int32 * 3)]
+                ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("best_first_packed", C.c_int32),
+                ("reserved", C.c_int32 * 2)]
 
 
 class BuildParams(C.Structure):
@@ -192,8 +193,10 @@ class Index:
         _check(lib().coral_index_get_deleted(self._h, _ptr(m)))
         return m
 
-    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False):
-        t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)))
+    def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False,
+                best_first_packed=False):
+        t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)),
+                   int(bool(best_first_packed)))
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

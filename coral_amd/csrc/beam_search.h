@@ -40,17 +40,18 @@ struct SearchArgs {
 struct BestFirstArgs {
     uint8_t* visited;   // [slots][stride]: the epoch of the query that last visited the node, 0 = never
     uint32_t* epochs;   // [slots]: last epoch used by the slot (kept across launches)
-    size_t stride;      // bytes per slot: n rounded up to a multiple of 16
+    size_t stride;      // bytes per slot, a multiple of 16: n, or 4 * ceil(n / 24) when packed
     int32_t slots;      // wavefronts = queries in flight
     int32_t rows_in_flight;  // 8 or 16: float4 registers of vector data a lane requests before it adds them up
     int32_t rows_unique;     // no graph row lists an id twice (checked by launch_find_repeated_ids)
+    int32_t packed;          // visited is [slots][stride] of 32-bit words, 8 bits of epoch over 24 node flags each
 };
 
 // LDS bytes of one wavefront: a beam of L keys, 64 candidate keys, 64 ids, L byte counters
 __host__ __device__ inline size_t best_first_wave_lds_bytes(int L) {
     return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + 15) & ~(size_t)15;
 }
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, int* max_wg_per_cu);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int* max_wg_per_cu);
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice
 hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream);

@@ -12,6 +12,8 @@
 // query that last visited the node, so nothing is cleared between queries (every 255th query of a slot wipes its
 // array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a million nodes); each test costs a
 // 128-byte line of HBM traffic and each mark a 32-byte write, together about a quarter of what the vectors cost.
+// For indexes too large for a byte per node and slot the same state is packed into 32-bit words of 8 epoch bits
+// over 24 node flags (template parameter PACKED).
 //
 // The arithmetic is that of beam_search.hip (same lane-strided accumulation, same butterfly, same 64-bit keys), so
 // results and counters are identical bit for bit; a wavefront needs no workgroup barrier anywhere.
@@ -46,7 +48,9 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
     return v;
 }
 
-template <int G, int CPL, int RIF>
+// PACKED: the visited state of a slot is one 32-bit word per 24 nodes (8 bits of epoch, 24 flags) instead of one
+// byte per node: a sixth of the memory, the same one line per test.
+template <int G, int CPL, int RIF, bool PACKED>
 __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -83,6 +87,24 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             epoch = 1u;
         }
         const uint8_t tag = (uint8_t)epoch;
+        uint32_t* visw = reinterpret_cast<uint32_t*>(vis);
+        // first visit?  (every lane passes its own id; ids of one call are distinct, or told apart by the caller)
+        auto unvisited = [&](uint32_t id) -> bool {
+            if (!PACKED) return __hip_atomic_load(vis + id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != tag;
+            const uint32_t w = __hip_atomic_load(visw + id / 24u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return (w >> 24) != epoch || ((w >> (id % 24u)) & 1u) == 0u;
+        };
+        // Mark a visit.  Packed: bring the word to this epoch (a maximum: words of older epochs lose their flags, a
+        // word of this epoch keeps them), then set the flag; both without a return value, and any interleaving of the
+        // two operations of several lanes on one word ends with all their flags set.
+        auto mark = [&](uint32_t id) {
+            if (!PACKED) {
+                __hip_atomic_store(vis + id, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                __hip_atomic_fetch_max(visw + id / 24u, epoch << 24, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_or(visw + id / 24u, 1u << (id % 24u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        };
 
         float4 qreg[CPL];
         {
@@ -209,7 +231,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             const int T = M - s0 < kBatch ? M - s0 : kBatch;
             if (lane < T) {
                 const uint32_t id = (uint32_t)a.start_ids[s0 + lane];
-                __hip_atomic_store(vis + id, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                mark(id);
                 todo[lane] = id;
             }
             wave_sync();
@@ -241,7 +263,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             int v = -1;
             if (lane < R) v = a.nbrs[(size_t)eid * R + lane];
             bool isnew = false;
-            if (v >= 0) isnew = __hip_atomic_load(vis + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != tag;
+            if (v >= 0) isnew = unvisited((uint32_t)v);
             if (!b.rows_unique && __ballot(isnew)) {
                 // an id listed twice in the row counts once (the first listing)
                 for (int k = 0; k < R; ++k) {
@@ -249,7 +271,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                     if (k < lane && vk == v) isnew = false;
                 }
             }
-            if (isnew) __hip_atomic_store(vis + v, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (isnew) mark((uint32_t)v);
             const uint64_t m = __ballot(isnew);
             const int T = __popcll(m);
             if (isnew) todo[prefix_popc(m)] = (uint32_t)v;
@@ -327,25 +349,26 @@ using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 
 // RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
 // dependent memory waits of a step against 8 and needs 128 registers
-template <int RIF>
+template <int RIF, bool PACKED>
 bf_kernel_fn pick_bf_kernel_rif(int chunks) {
-    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF>;
-    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF>;
-    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF>;
-    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF>;
-    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF>;
-    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF>;
+    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED>;
+    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED>;
+    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED>;
+    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED>;
+    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED>;
+    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED>;
     return nullptr;
 }
 
-bf_kernel_fn pick_bf_kernel(int dim, int rif) {
-    return rif >= 16 ? pick_bf_kernel_rif<16>(dim / 4) : pick_bf_kernel_rif<8>(dim / 4);
+bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed) {
+    if (packed) return rif >= 16 ? pick_bf_kernel_rif<16, true>(dim / 4) : pick_bf_kernel_rif<8, true>(dim / 4);
+    return rif >= 16 ? pick_bf_kernel_rif<16, false>(dim / 4) : pick_bf_kernel_rif<8, false>(dim / 4);
 }
 
 }  // namespace
 
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, int* max_wg_per_cu) {
-    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int* max_wg_per_cu) {
+    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed);
     if (!fn) return hipErrorInvalidValue;
     const size_t lds = best_first_wave_lds_bytes(L) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -359,7 +382,7 @@ hipError_t best_first_prepare(int dim, int L, int rows_in_flight, int* max_wg_pe
 }
 
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream) {
-    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight);
+    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_wave_lds_bytes(a.L) * kWavesPerWg, stream, a, b);

@@ -304,7 +304,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         idx->counters_alloc = need_counters;
     }
     // Best-first: one wavefront per query with the visited state in HBM (best_first.hip), when the memory for it
-    // is there: n bytes per wavefront, up to a third of what is free and 64 GiB.
+    // is there: n bytes per wavefront (n / 6 in the packed form), up to a third of what is free and 64 GiB.
     idx->bf_ready = false;
     if (best_first && !t.best_first_in_lds) {
         int bf_wg_per_cu = 0;
@@ -312,14 +312,21 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const int chunks = idx->dim / 4;
         const int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
         idx->bf_rows_in_flight = rif;
-        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, &bf_wg_per_cu));
-        const size_t stride = ((size_t)idx->n + 15) & ~(size_t)15;
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, &bf_wg_per_cu));
         size_t free_b = 0, total_b = 0;
         HIP_TRY(hipMemGetInfo(&free_b, &total_b));
         const size_t budget = std::min<size_t>((free_b + idx->bf_alloc_bytes) / 3, (size_t)64 << 30);
-        int64_t want = t.workgroups > 0 ? (int64_t)t.workgroups * 4 : (int64_t)bf_wg_per_cu * idx->num_cu * 4;
-        int slots = (int)std::min<int64_t>(want, (int64_t)Q);
-        slots = (int)std::min<size_t>((size_t)slots, budget / stride);
+        const int64_t want = t.workgroups > 0 ? (int64_t)t.workgroups * 4 : (int64_t)bf_wg_per_cu * idx->num_cu * 4;
+        const size_t stride_bytes = ((size_t)idx->n + 15) & ~(size_t)15;
+        const size_t stride_packed = ((((size_t)idx->n + 23) / 24 * 4) + 15) & ~(size_t)15;
+        // a byte per node while that leaves every wavefront its slot, else the packed words
+        const int64_t need = std::min<int64_t>(want, (int64_t)Q);
+        const int packed = t.best_first_packed || (int64_t)(budget / stride_bytes) < need ? 1 : 0;
+        const size_t stride = packed ? stride_packed : stride_bytes;
+        if (packed != idx->bf_packed) idx->bf_stride = 0;  // forces a fresh, zeroed allocation
+        idx->bf_packed = packed;
+        if (packed) HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, true, &bf_wg_per_cu));
+        int slots = (int)std::min<size_t>((size_t)need, budget / stride);
         // below about four wavefronts per CU the workgroup-per-query kernel is the faster one
         if (bf_wg_per_cu > 0 && (slots >= 4 * idx->num_cu || slots >= Q || t.workgroups > 0) && slots > 0) {
             bool have = stride == idx->bf_stride && slots <= idx->bf_alloc_slots;
@@ -410,6 +417,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     if (wave_kernel) {
         coral::BestFirstArgs b;
         b.rows_unique = idx->rows_unique == 1;
+        b.packed = idx->bf_packed;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;

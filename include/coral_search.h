@@ -101,7 +101,10 @@ typedef struct {
                                    per node and query slot in HBM (n bytes x up to 4096 slots); 1 keeps it on the
                                    workgroup-per-query kernel with the visited set in LDS, as it also does by
                                    itself when that memory is not to be had */
-    int32_t reserved[3];
+    int32_t best_first_packed;  /* that visited state is a byte per node while n bytes x query slots fit a third of
+                                   the free memory (and 64 GiB), else a 32-bit word per 24 nodes (8 bits of epoch,
+                                   24 flags: n / 6 bytes per slot, about 5 % slower); 1 = the packed form always */
+    int32_t reserved[2];
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);

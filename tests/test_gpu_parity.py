@@ -82,10 +82,11 @@ def test_exact_against_same_order_oracle(orc, case):
     else:
         oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=m, order=WAVE64)
     idx = capi.Index(base, nbrs, starts, m)
-    # best-first has two kernels: a wavefront per query (visited bytes in HBM) and a workgroup per query (LDS table)
-    for in_lds in ((False, True) if policy == 1 else (False,)):
+    # best-first has two kernels: a wavefront per query (visited state in HBM, a byte per node or packed words) and a
+    # workgroup per query (LDS table)
+    for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
         idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy,
-                    best_first_in_lds=in_lds)
+                    best_first_in_lds=in_lds, best_first_packed=packed)
         ids, dists, st = idx.search(q, k, L, policy=policy)
         cnt = idx.query_counters(q.shape[0])
         assert np.array_equal(ids, oi)
@@ -115,13 +116,14 @@ def test_best_first_query_slots_are_reused(orc):
     oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
     idx = capi.Index(base, nbrs, starts)
     idx.set_deleted(mask)
-    idx.prepare(q.shape[0], L, workgroups=2, policy=1)
-    for rep in range(2):
-        print("slot reuse pass", rep, flush=True)
-        ids, dists, st = idx.search(q, k, L, policy=1, have_delete=True)
-        cnt = idx.query_counters(q.shape[0])
-        assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(cnt, os_)
-        assert st.spills == 0
+    for packed in (False, True):
+        idx.prepare(q.shape[0], L, workgroups=2, policy=1, best_first_packed=packed)
+        for rep in range(2):
+            print("slot reuse pass", rep, "packed" if packed else "bytes", flush=True)
+            ids, dists, st = idx.search(q, k, L, policy=1, have_delete=True)
+            cnt = idx.query_counters(q.shape[0])
+            assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(cnt, os_)
+            assert st.spills == 0
     # fewer queries than slots, and the other kernel on the same index afterwards
     ids, dists, _ = idx.search(q[:3], k, L, policy=1, have_delete=True)
     assert np.array_equal(ids, oi[:3])
