@@ -109,6 +109,8 @@ SIGNATURES = {
     "coral_build_graph_from_clusters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "coral_index_get_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_start_ids_fps": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "coral_bruteforce_set_exact_only": (C.c_int, [C.c_void_p, C.c_int32]),
+    "coral_bruteforce_last_redone": (C.c_int64, [C.c_void_p]),
     "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                        C.c_void_p, C.POINTER(C.c_double)]),
 }
@@ -233,6 +235,13 @@ class Index:
         _check(lib().coral_bruteforce_knn(self._h, _ptr(q), Q, k, int(have_delete), _ptr(ids), _ptr(dists),
                                           C.byref(t)))
         return ids, dists, t.value
+
+    def bruteforce_exact_only(self, on=True):
+        """Skip (or restore) the matrix-core screening pass of the exact kNN."""
+        _check(lib().coral_bruteforce_set_exact_only(self._h, int(bool(on))))
+
+    def bruteforce_last_redone(self):
+        return int(lib().coral_bruteforce_last_redone(self._h))
 
     def bruteforce_device(self, d_queries, d_ids, d_dists, Q, k, have_delete=False, stream=None):
         t = C.c_double()

@@ -12,4 +12,18 @@ hipError_t launch_row_select(const float* D, int64_t ldD, int nq, int64_t n, int
                              unsigned long long* out, int64_t out_stride, int* redo, hipStream_t stream);
 hipError_t launch_merge_segments(const unsigned long long* part, int nq, int nseg, int k, int metric,
                                  int32_t* ids, float* dists, hipStream_t stream);
+// --- the screening pass on the matrix cores (bruteforce_mfma.hip) ---
+// out[r] = |x_r|^2; *max_bits (optional, zero before) = bit pattern of the largest of them
+hipError_t launch_row_norms(const float* x, int64_t n, int dim, float* out, uint32_t* max_bits, hipStream_t stream);
+// as launch_distance_tile, with D[q][b] = |q|^2 + |b|^2 - 2 q.b (L2) or -q.b (IP) from fp32 MFMA inner products
+hipError_t launch_approx_tile(const float* queries, const float* base, int nq, int64_t nb, int dim, int metric,
+                              const float* qn, const float* bn, const uint32_t* deleted, int64_t base_id0, float* D,
+                              int64_t ldD, hipStream_t stream);
+// cand_ids / cand_d [nq][kc] (ascending approximate signed distance, -1 = none) -> the exact k best per query in the
+// reference's summation order; redo[q] = 1 where the candidates cannot vouch for the result
+hipError_t launch_rerank(const float* queries, const float* base, int nq, int dim, int metric, const int32_t* cand_ids,
+                         const float* cand_d, int kc, int k, const float* qn, const uint32_t* bn_max_bits, int32_t* ids,
+                         float* dists, int* redo, hipStream_t stream);
+hipError_t launch_scatter_results(const int32_t* rows, int count, int k, const int32_t* src_ids, const float* src_d,
+                                  int32_t* dst_ids, float* dst_d, hipStream_t stream);
 }  // namespace coral

@@ -1,9 +1,12 @@
 // bruteforce_api.cpp -- coral_bruteforce_knn*: exact k nearest neighbours of a batch of
-// queries among the index's resident vectors (kernels in bruteforce.hip).
+// queries among the index's resident vectors (kernels in bruteforce.hip, bruteforce_mfma.hip).
 #include <algorithm>
 #include <cstring>
+#include <vector>
 
+#include "beam_search.h"
 #include "bruteforce.h"
+#include "graph_build.h"
 #include "index_internal.h"
 
 using coral::fail;
@@ -11,20 +14,12 @@ using coral::fail;
 namespace {
 constexpr int64_t kSegment = (int64_t)1 << 22;   // base points per pass
 constexpr int64_t kBufferFloats = (int64_t)1 << 29;  // 2 GiB distance buffer
-}  // namespace
 
-extern "C" {
-
-int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q, int32_t k,
-                             int32_t have_delete, int32_t* d_ids, float* d_dists, void* stream_,
-                             double* time_s) {
-    if (!idx || !d_queries || !d_ids) return fail(CORAL_ERR_ARG, "null argument");
-    if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
-    if (k <= 0 || k > 2048) return fail(CORAL_ERR_ARG, "k must be in 1..2048 (got %d)", k);
-    if (have_delete && !idx->d_deleted)
-        return fail(CORAL_ERR_STATE, "have_delete set but no tombstone mask was given");
-    HIP_TRY(hipSetDevice(idx->device));
-    hipStream_t stream = stream_ ? (hipStream_t)stream_ : idx->stream;
+// the passes over the base: distances of a block of queries to a segment of the base into D, the k best of every row
+// of D, and at the end the k best of the per-segment winners.  screen: approximate distances from the matrix cores
+// (qn, bn: squared norms) instead of the reference-order ones.
+int knn_passes(coral_index* idx, const float* d_queries, int32_t Q, int32_t k, int32_t have_delete, bool screen,
+               const float* d_qn, int metric_out, int32_t* d_ids, float* d_dists, hipStream_t stream) {
     const int64_t n = idx->n;
     int64_t seg = std::min(n, kSegment);
     int64_t nseg = (n + seg - 1) / seg;
@@ -55,33 +50,131 @@ int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q
     HIP_TRY_R(hipMalloc(&D, (size_t)qc * ld * sizeof(float)));
     HIP_TRY_R(hipMalloc(&part, (size_t)Q * nseg * k * sizeof(unsigned long long)));
     HIP_TRY_R(hipMalloc(&redo, (size_t)qc * sizeof(int)));
-    hipEvent_t ev0, ev1;
-    HIP_TRY_R(hipEventCreate(&ev0));
-    HIP_TRY_R(hipEventCreate(&ev1));
-    HIP_TRY_R(hipEventRecord(ev0, stream));
     for (int64_t q0 = 0; q0 < Q; q0 += qc) {
         const int nq = (int)std::min<int64_t>(qc, Q - q0);
         for (int64_t s = 0; s < nseg; ++s) {
             const int64_t b0 = s * seg, nb = std::min(seg, n - b0);
-            HIP_TRY_R(coral::launch_distance_tile(d_queries + (size_t)q0 * idx->dim,
-                                                  idx->d_vec + (size_t)b0 * idx->dim, nq, nb, idx->dim,
-                                                  idx->metric, have_delete ? idx->d_deleted : nullptr, b0, D, ld,
-                                                  stream));
-            HIP_TRY_R(coral::launch_row_select(D, ld, nq, nb, k, b0, part + ((size_t)q0 * nseg + s) * k,
-                                               nseg * k, redo, stream));
+            const float* qp = d_queries + (size_t)q0 * idx->dim;
+            const float* bp = idx->d_vec + (size_t)b0 * idx->dim;
+            const uint32_t* del = have_delete ? idx->d_deleted : nullptr;
+            if (screen)
+                HIP_TRY_R(coral::launch_approx_tile(qp, bp, nq, nb, idx->dim, idx->metric, d_qn + q0, idx->d_bnorm + b0, del,
+                                                    b0, D, ld, stream));
+            else
+                HIP_TRY_R(coral::launch_distance_tile(qp, bp, nq, nb, idx->dim, idx->metric, del, b0, D, ld, stream));
+            HIP_TRY_R(coral::launch_row_select(D, ld, nq, nb, k, b0, part + ((size_t)q0 * nseg + s) * k, nseg * k, redo,
+                                               stream));
         }
     }
-    HIP_TRY_R(coral::launch_merge_segments(part, Q, (int)nseg, k, idx->metric, d_ids, d_dists, stream));
-    HIP_TRY_R(hipEventRecord(ev1, stream));
-    HIP_TRY_R(hipEventSynchronize(ev1));
-    float ms = 0.f;
-    HIP_TRY_R(hipEventElapsedTime(&ms, ev0, ev1));
+    HIP_TRY_R(coral::launch_merge_segments(part, Q, (int)nseg, k, metric_out, d_ids, d_dists, stream));
+    HIP_TRY_R(hipStreamSynchronize(stream));
 #undef HIP_TRY_R
+    release();
+    return CORAL_OK;
+}
+
+// |b|^2 of the base, once per index
+int ensure_base_norms(coral_index* idx, hipStream_t stream) {
+    if (idx->d_bnorm) return CORAL_OK;
+    HIP_TRY(hipMalloc(&idx->d_bnorm_max, sizeof(uint32_t)));
+    HIP_TRY(hipMalloc(&idx->d_bnorm, (size_t)idx->n * sizeof(float)));
+    HIP_TRY(coral::launch_fill_u32(idx->d_bnorm_max, 1, 0u, stream));
+    HIP_TRY(coral::launch_row_norms(idx->d_vec, idx->n, idx->dim, idx->d_bnorm, idx->d_bnorm_max, stream));
+    return CORAL_OK;
+}
+
+constexpr int kScreenSlack = 32;  // candidates kept beyond k
+
+}  // namespace
+
+extern "C" {
+
+int coral_bruteforce_set_exact_only(coral_index* idx, int32_t on) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    idx->knn_exact_only = on != 0;
+    return CORAL_OK;
+}
+
+int64_t coral_bruteforce_last_redone(coral_index* idx) { return idx ? idx->knn_last_redone : -1; }
+
+int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q, int32_t k,
+                             int32_t have_delete, int32_t* d_ids, float* d_dists, void* stream_,
+                             double* time_s) {
+    if (!idx || !d_queries || !d_ids) return fail(CORAL_ERR_ARG, "null argument");
+    if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
+    if (k <= 0 || k > 2048) return fail(CORAL_ERR_ARG, "k must be in 1..2048 (got %d)", k);
+    if (have_delete && !idx->d_deleted)
+        return fail(CORAL_ERR_STATE, "have_delete set but no tombstone mask was given");
+    HIP_TRY(hipSetDevice(idx->device));
+    hipStream_t stream = stream_ ? (hipStream_t)stream_ : idx->stream;
+    hipEvent_t ev0, ev1;
+    HIP_TRY(hipEventCreate(&ev0));
+    HIP_TRY(hipEventCreate(&ev1));
+    HIP_TRY(hipEventRecord(ev0, stream));
+    int rc = CORAL_OK;
+    const int kc = k + kScreenSlack;
+    idx->knn_last_redone = 0;
+    if (idx->knn_exact_only || kc > 2048 || idx->n <= kc) {
+        rc = knn_passes(idx, d_queries, Q, k, have_delete, false, nullptr, idx->metric, d_ids, d_dists, stream);
+    } else {
+        // screening on the matrix cores, exact distances for the kc candidates of each query, the exact passes for
+        // the queries whose candidates cannot vouch for the result (bruteforce_mfma.hip)
+        float *d_qn = nullptr, *d_cd = nullptr, *d_rq = nullptr, *d_rd = nullptr;
+        int32_t *d_cid = nullptr, *d_rows = nullptr, *d_rid = nullptr;
+        int* d_redo = nullptr;
+        std::vector<int> redo((size_t)Q);
+        std::vector<int32_t> rows;
+        auto release = [&]() {
+            (void)hipFree(d_qn), (void)hipFree(d_cd), (void)hipFree(d_cid), (void)hipFree(d_redo);
+            (void)hipFree(d_rows), (void)hipFree(d_rq), (void)hipFree(d_rid), (void)hipFree(d_rd);
+        };
+        auto ok = [&](hipError_t e, const char* what) {
+            if (e == hipSuccess) return true;
+            rc = fail(e == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE, "%s failed: %s", what,
+                      hipGetErrorString(e));
+            return false;
+        };
+        if ((rc = ensure_base_norms(idx, stream)) == CORAL_OK &&
+            ok(hipMalloc(&d_qn, (size_t)Q * sizeof(float)), "hipMalloc") &&
+            ok(hipMalloc(&d_cid, (size_t)Q * kc * sizeof(int32_t)), "hipMalloc") &&
+            ok(hipMalloc(&d_cd, (size_t)Q * kc * sizeof(float)), "hipMalloc") &&
+            ok(hipMalloc(&d_redo, (size_t)Q * sizeof(int)), "hipMalloc") &&
+            ok(coral::launch_row_norms(d_queries, Q, idx->dim, d_qn, nullptr, stream), "query norms"))
+            rc = knn_passes(idx, d_queries, Q, kc, have_delete, true, d_qn, /*signed distances*/ 0, d_cid, d_cd, stream);
+        if (rc == CORAL_OK &&
+            ok(coral::launch_rerank(d_queries, idx->d_vec, Q, idx->dim, idx->metric, d_cid, d_cd, kc, k, d_qn,
+                                    idx->d_bnorm_max, d_ids, d_dists, d_redo, stream), "rerank") &&
+            ok(hipMemcpyAsync(redo.data(), d_redo, (size_t)Q * sizeof(int), hipMemcpyDeviceToHost, stream), "hipMemcpy") &&
+            ok(hipStreamSynchronize(stream), "synchronize")) {
+            for (int32_t q = 0; q < Q; ++q)
+                if (redo[(size_t)q]) rows.push_back(q);
+        }
+        if (rc == CORAL_OK && !rows.empty()) {
+            const int m = (int)rows.size();
+            if (ok(hipMalloc(&d_rows, (size_t)m * sizeof(int32_t)), "hipMalloc") &&
+                ok(hipMalloc(&d_rq, (size_t)m * idx->dim * sizeof(float)), "hipMalloc") &&
+                ok(hipMalloc(&d_rid, (size_t)m * k * sizeof(int32_t)), "hipMalloc") &&
+                ok(hipMalloc(&d_rd, (size_t)m * k * sizeof(float)), "hipMalloc") &&
+                ok(hipMemcpyAsync(d_rows, rows.data(), (size_t)m * sizeof(int32_t), hipMemcpyHostToDevice, stream), "hipMemcpy") &&
+                ok(coral::launch_gather_rows(d_queries, idx->dim, d_rows, m, d_rq, stream), "gather"))
+                rc = knn_passes(idx, d_rq, m, k, have_delete, false, nullptr, idx->metric, d_rid, d_rd, stream);
+            if (rc == CORAL_OK &&
+                ok(coral::launch_scatter_results(d_rows, m, k, d_rid, d_rd, d_ids, d_dists, stream), "scatter"))
+                ok(hipStreamSynchronize(stream), "synchronize");
+        }
+        idx->knn_last_redone = (int64_t)rows.size();
+        release();
+    }
+    if (rc == CORAL_OK) {
+        HIP_TRY(hipEventRecord(ev1, stream));
+        HIP_TRY(hipEventSynchronize(ev1));
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
+        if (time_s) *time_s = ms / 1000.0;
+    }
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
-    release();
-    if (time_s) *time_s = ms / 1000.0;
-    return CORAL_OK;
+    return rc;
 }
 
 int coral_bruteforce_knn(coral_index* idx, const float* h_queries, int32_t Q, int32_t k, int32_t have_delete,

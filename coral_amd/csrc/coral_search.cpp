@@ -157,6 +157,8 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_phase);
     (void)hipFree(idx->d_bf_visited);
     (void)hipFree(idx->d_bf_epochs);
+    (void)hipFree(idx->d_bnorm);
+    (void)hipFree(idx->d_bnorm_max);
     (void)hipFree(idx->d_io_q);
     (void)hipFree(idx->d_io_ids);
     (void)hipFree(idx->d_io_dists);

@@ -51,6 +51,13 @@ struct coral_index {
     float* d_io_dists = nullptr;
     size_t io_q_bytes = 0, io_ids_bytes = 0, io_dists_bytes = 0;
 
+    // exact kNN: |b|^2 of every base vector and the bit pattern of the largest (made on first use), and whether the
+    // matrix-core screening pass is skipped
+    float* d_bnorm = nullptr;
+    uint32_t* d_bnorm_max = nullptr;
+    bool knn_exact_only = false;
+    int64_t knn_last_redone = 0;  // queries of the last call that went through the exact passes after screening
+
     // best-first on one wavefront per query: per-slot visited epochs in global memory
     bool bf_ready = false;
     uint8_t* d_bf_visited = nullptr;

@@ -175,6 +175,14 @@ CORAL_API int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries,
                                        double* time_s);
 CORAL_API int coral_bruteforce_knn(coral_index* idx, const float* h_queries, int32_t Q, int32_t k,
                                    int32_t have_delete, int32_t* h_ids, float* h_dists, double* time_s);
+/* The search first screens all pairs with approximate distances from the matrix cores, keeps k + 32 candidates per
+ * query, measures those in the reference's summation order and sends the rare query whose candidates cannot vouch
+ * for the result through the plain passes: same ids and distance bits either way.  on = 1 skips the screening
+ * (every pair in the reference's order on the vector units).  No counterpart in the reference (faiss does this work
+ * there). */
+CORAL_API int coral_bruteforce_set_exact_only(coral_index* idx, int32_t on);
+/* queries of the last coral_bruteforce_knn* call that went through the plain passes after the screening */
+CORAL_API int64_t coral_bruteforce_last_redone(coral_index* idx);
 
 /* Entry points by farthest-point sampling in hop distance, Graph::FPS (src/start.cu:74-145): out_ids[0] =
  * first_id; each further id is the node whose smallest hop count from the ids chosen so far is largest

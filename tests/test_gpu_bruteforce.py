@@ -70,11 +70,19 @@ def test_bruteforce_exact_against_oracle(orc, n, dim, Q, k, metric, tomb):
     idx = capi.Index(base, ring(n), np.array([0], np.int32), m)
     if tomb:
         idx.set_deleted(mask)
-    ids, dists, _ = idx.bruteforce(q, k, have_delete=tomb)
+    ids, dists, _ = idx.bruteforce(q, k, have_delete=tomb)  # matrix-core screening + exact re-ranking
+    redone = idx.bruteforce_last_redone()
+    idx.bruteforce_exact_only(True)                         # every pair in the reference's order
+    ids2, dists2, _ = idx.bruteforce(q, k, have_delete=tomb)
+    assert idx.bruteforce_last_redone() == 0
     idx.close()
+    print("queries that the screening could not vouch for: %d of %d" % (redone, Q), flush=True)
     oi, od = orc.bruteforce(base, q, k, m, deleted=mask, order=SEQ)
     assert np.array_equal(ids, oi)
     assert dists.tobytes() == od.tobytes()
+    assert np.array_equal(ids2, oi) and dists2.tobytes() == od.tobytes()
+    if n > 2 * (k + 32) and dim >= 20:
+        assert redone <= Q // 4  # independent data: the candidates nearly always suffice
     # against the fp64 closed form: same ids except where fp32 rounding reorders near-ties
     ti, td = orc.bruteforce(base, q, k, m, deleted=mask)
     live = ti >= 0
@@ -88,8 +96,10 @@ def test_bruteforce_ties_are_ordered_by_id(orc):
     grid = np.stack(np.meshgrid(*[np.arange(side)] * 4, indexing="ij"), -1).reshape(-1, 4).astype(np.float32)
     q = np.array([[3, 3, 3, 3], [0, 0, 0, 0], [2.5, 3, 1, 6]], np.float32)
     idx = capi.Index(grid, ring(grid.shape[0]), np.array([0], np.int32))
+    redone = 0
     for k in (1, 9, 33, 81, 200):
         ids, dists, _ = idx.bruteforce(q, k)
+        redone += idx.bruteforce_last_redone()
         oi, od = orc.bruteforce(grid, q, k, order=SEQ)
         assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
         d2 = ((grid[ids] - q[:, None, :]) ** 2).sum(-1)
@@ -98,6 +108,7 @@ def test_bruteforce_ties_are_ordered_by_id(orc):
         for r in range(q.shape[0]):
             same = np.diff(dists[r]) == 0
             assert (np.diff(ids[r])[same] > 0).all()
+    assert redone > 0  # ties across the last candidate's place: the screening hands those queries over
     idx.close()
 
 
