@@ -5,7 +5,9 @@
 // (src/knn.cu:174-193).  Output order and file layout are the gt file's
 // (uint32 nq, uint32 k, int32 ids[nq*k], include/efanna2e/util.h:81-103).
 //
-// Three kernels:
+// The search screens all pairs on the matrix cores first and re-ranks a few candidates per query exactly
+// (bruteforce_mfma.hip); the kernels here are the selection both ways share, and the plain distance pass that
+// defines the result and takes over where the screening cannot vouch for it:
 //   distance_tile_kernel  a 128 x 128 tile of (query, base) pairs per workgroup, 8 x 8 pairs per
 //                         thread, operands staged through LDS.  Every pair is accumulated by ONE
 //                         thread walking the dimensions in order with one fused multiply-add per
