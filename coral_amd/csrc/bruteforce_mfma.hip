@@ -25,7 +25,11 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int MT = 128, NT = 128, BK = 8;  // tile of queries x base points per workgroup, dimensions per LDS stage
+#ifndef CORAL_MFMA_BK
+#define CORAL_MFMA_BK 8
+#endif
+constexpr int MT = 128, NT = 128, BK = CORAL_MFMA_BK;  // tile of queries x base points per workgroup, dimensions per LDS stage
+constexpr int NLD = BK / 8;                             // float4 loads per thread, operand and stage
 
 __device__ __forceinline__ uint32_t mf_ord32(float s) {
     const uint32_t u = __float_as_uint(s);
@@ -73,18 +77,25 @@ __global__ __launch_bounds__(256) void approx_tile_mfma_kernel(const float* __re
     const int64_t b0 = (int64_t)blockIdx.x * NT;
     const int q0 = blockIdx.y * MT;
     const int lrow = tid >> 1, lk = (tid & 1) * 4;  // staging: thread t loads row t/2, dimensions (t&1)*4 .. +4
-    float4 va, vb;
+    float4 va[NLD], vb[NLD];
     auto fetch = [&](int k0) {
-        va = make_float4(0, 0, 0, 0), vb = make_float4(0, 0, 0, 0);
-        const int kd = k0 + lk;
-        if (kd < dim) {
-            if (q0 + lrow < nq) va = *reinterpret_cast<const float4*>(queries + (size_t)(q0 + lrow) * dim + kd);
-            if (b0 + lrow < nb) vb = *reinterpret_cast<const float4*>(base + (size_t)(b0 + lrow) * dim + kd);
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            va[u] = make_float4(0, 0, 0, 0), vb[u] = make_float4(0, 0, 0, 0);
+            const int kd = k0 + lk + 8 * u;
+            if (kd < dim) {
+                if (q0 + lrow < nq) va[u] = *reinterpret_cast<const float4*>(queries + (size_t)(q0 + lrow) * dim + kd);
+                if (b0 + lrow < nb) vb[u] = *reinterpret_cast<const float4*>(base + (size_t)(b0 + lrow) * dim + kd);
+            }
         }
     };
     auto park = [&](int buf) {
-        sa[buf][lk + 0][lrow] = va.x, sa[buf][lk + 1][lrow] = va.y, sa[buf][lk + 2][lrow] = va.z, sa[buf][lk + 3][lrow] = va.w;
-        sb[buf][lk + 0][lrow] = vb.x, sb[buf][lk + 1][lrow] = vb.y, sb[buf][lk + 2][lrow] = vb.z, sb[buf][lk + 3][lrow] = vb.w;
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const int r = lk + 8 * u;
+            sa[buf][r + 0][lrow] = va[u].x, sa[buf][r + 1][lrow] = va[u].y, sa[buf][r + 2][lrow] = va[u].z, sa[buf][r + 3][lrow] = va[u].w;
+            sb[buf][r + 0][lrow] = vb[u].x, sb[buf][r + 1][lrow] = vb[u].y, sb[buf][r + 2][lrow] = vb[u].z, sb[buf][r + 3][lrow] = vb[u].w;
+        }
     };
     v16f acc[2][2];
 #pragma unroll
