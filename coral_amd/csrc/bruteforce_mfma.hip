@@ -64,7 +64,10 @@ __global__ __launch_bounds__(256) void row_norms_kernel(const float* __restrict_
 // ids.  grid = (ceil(nb/NT), ceil(nq/MT)), 256 threads = 4 wavefronts in 2 x 2, each 64 x 64 of the tile as 2 x 2
 // MFMA blocks of 32 x 32.  Operands go through LDS dimension-major, so that the 32 lanes of an MFMA operand read
 // consecutive words.
-__global__ __launch_bounds__(256) void approx_tile_mfma_kernel(const float* __restrict__ queries,
+#ifndef CORAL_MFMA_WAVES
+#define CORAL_MFMA_WAVES 4
+#endif
+__global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel(const float* __restrict__ queries,
                                                               const float* __restrict__ base, int nq, int64_t nb,
                                                               int dim, int metric, const float* __restrict__ qn,
                                                               const float* __restrict__ bn,
