@@ -45,13 +45,24 @@ struct BestFirstArgs {
     int32_t rows_in_flight;  // 8 or 16: float4 registers of vector data a lane requests before it adds them up
     int32_t rows_unique;     // no graph row lists an id twice (checked by launch_find_repeated_ids)
     int32_t packed;          // visited is [slots][stride] of 32-bit words, 8 bits of epoch over 24 node flags each
+    int32_t bloom_log2;      // log2 of the bits of the per-wavefront Bloom filter in LDS, 0 = none
 };
 
-// LDS bytes of one wavefront: a beam of L keys, 64 candidate keys, 64 ids, L byte counters
-__host__ __device__ inline size_t best_first_wave_lds_bytes(int L) {
-    return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + 15) & ~(size_t)15;
+// LDS bytes of one wavefront: a beam of L keys, 64 candidate keys, 64 ids, L byte counters, and a Bloom filter of
+// 2^bloom_log2 bits over the visited ids (bloom_log2 = 0: none)
+__host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2) {
+    const size_t bloom = bloom_log2 ? ((size_t)1 << bloom_log2) / 8 : 0;
+    return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + bloom + 15) & ~(size_t)15;
 }
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int* max_wg_per_cu);
+// the filter size for a beam of L: 64 bits per beam entry rounded up to a power of two, halved while that would leave
+// a CU fewer than sixteen wavefronts; none below 4096 bits
+__host__ inline int best_first_bloom_log2(int L) {
+    int lg = 12;
+    while (((size_t)1 << lg) < (size_t)64 * L && lg < 17) ++lg;
+    while (lg >= 12 && best_first_wave_lds_bytes(L, lg) > (size_t)10 * 1024) --lg;
+    return lg >= 12 ? lg : 0;
+}
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int* max_wg_per_cu);
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice
 hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream);

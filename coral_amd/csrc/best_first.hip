@@ -13,7 +13,8 @@
 // array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a million nodes); each test costs a
 // 128-byte line of HBM traffic and each mark a 32-byte write, together about a quarter of what the vectors cost.
 // For indexes too large for a byte per node and slot the same state is packed into 32-bit words of 8 epoch bits
-// over 24 node flags (template parameter PACKED).
+// over 24 node flags (template parameter PACKED).  A Bloom filter over the query's visited ids in LDS (4 KB at
+// L = 512) answers most tests without that line: an id it does not know is new for certain.
 //
 // The arithmetic is that of beam_search.hip (same lane-strided accumulation, same butterfly, same 64-bit keys), so
 // results and counters are identical bit for bit; a wavefront needs no workgroup barrier anywhere.
@@ -58,12 +59,33 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
     if (slot >= b.slots) return;  // the whole wavefront; no workgroup barrier is used below
     const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2, M = a.M;
     const int Lp = (L + 3) & ~3;
-    unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L);
+    unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L, b.bloom_log2);
     uint64_t* beam = reinterpret_cast<uint64_t*>(mine_lds);      // L keys, sorted
     uint64_t* cand = beam + Lp;                                   // kBatch keys
     uint32_t* todo = reinterpret_cast<uint32_t*>(cand + kBatch);  // kBatch ids
     uint32_t* marks = todo + kBatch;                              // Lp byte counters, zero between merges
+    uint32_t* bloom = marks + (Lp >> 2);                          // 2^bloom_log2 bits, or none
     for (int i = lane; i < (Lp >> 2); i += 64) marks[i] = 0u;
+    // The Bloom filter holds every id the query has visited.  An id it does not know is new for certain and needs no
+    // look at the visited state in HBM (most tests: a query sees far more new ids than old ones); an id it may know
+    // is looked up as before.  Two multiplicative hashes.
+    const int bl = b.bloom_log2;
+    const int bloom_words = bl ? (1 << bl) >> 5 : 0;
+    auto bloom_bits = [&](uint32_t id, uint32_t& h1, uint32_t& h2) {
+        h1 = (id * 0x9E3779B1u) >> (32 - bl);
+        h2 = (id * 0x85EBCA77u + 0x3C6EF372u) >> (32 - bl);
+    };
+    auto bloom_may_hold = [&](uint32_t id) -> bool {
+        uint32_t h1, h2;
+        bloom_bits(id, h1, h2);
+        return ((bloom[h1 >> 5] >> (h1 & 31)) & (bloom[h2 >> 5] >> (h2 & 31)) & 1u) != 0u;
+    };
+    auto bloom_add = [&](uint32_t id) {
+        uint32_t h1, h2;
+        bloom_bits(id, h1, h2);
+        atomicOr(&bloom[h1 >> 5], 1u << (h1 & 31));
+        atomicOr(&bloom[h2 >> 5], 1u << (h2 & 31));
+    };
 
     uint8_t* vis = b.visited + (size_t)slot * b.stride;
     uint32_t epoch = b.epochs[slot];
@@ -87,6 +109,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             epoch = 1u;
         }
         const uint8_t tag = (uint8_t)epoch;
+        for (int i = lane; i < bloom_words; i += 64) bloom[i] = 0u;
         uint32_t* visw = reinterpret_cast<uint32_t*>(vis);
         // first visit?  (every lane passes its own id; ids of one call are distinct, or told apart by the caller)
         auto unvisited = [&](uint32_t id) -> bool {
@@ -232,6 +255,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             if (lane < T) {
                 const uint32_t id = (uint32_t)a.start_ids[s0 + lane];
                 mark(id);
+                if (bl) bloom_add(id);
                 todo[lane] = id;
             }
             wave_sync();
@@ -263,7 +287,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             int v = -1;
             if (lane < R) v = a.nbrs[(size_t)eid * R + lane];
             bool isnew = false;
-            if (v >= 0) isnew = unvisited((uint32_t)v);
+            if (v >= 0) isnew = (bl && !bloom_may_hold((uint32_t)v)) || unvisited((uint32_t)v);
             if (!b.rows_unique && __ballot(isnew)) {
                 // an id listed twice in the row counts once (the first listing)
                 for (int k = 0; k < R; ++k) {
@@ -271,7 +295,10 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                     if (k < lane && vk == v) isnew = false;
                 }
             }
-            if (isnew) mark((uint32_t)v);
+            if (isnew) {
+                mark((uint32_t)v);
+                if (bl) bloom_add((uint32_t)v);
+            }
             const uint64_t m = __ballot(isnew);
             const int T = __popcll(m);
             if (isnew) todo[prefix_popc(m)] = (uint32_t)v;
@@ -367,10 +394,10 @@ bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed) {
 
 }  // namespace
 
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int* max_wg_per_cu) {
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int* max_wg_per_cu) {
     bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed);
     if (!fn) return hipErrorInvalidValue;
-    const size_t lds = best_first_wave_lds_bytes(L) * kWavesPerWg;
+    const size_t lds = best_first_wave_lds_bytes(L, bloom_log2) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -385,7 +412,7 @@ hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStr
     bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
-    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_wave_lds_bytes(a.L) * kWavesPerWg, stream, a, b);
+    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_wave_lds_bytes(a.L, b.bloom_log2) * kWavesPerWg, stream, a, b);
     return hipGetLastError();
 }
 

@@ -314,7 +314,9 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const int chunks = idx->dim / 4;
         const int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
         idx->bf_rows_in_flight = rif;
-        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, &bf_wg_per_cu));
+        const int bloom_log2 = coral::best_first_bloom_log2(L);
+        idx->bf_bloom_log2 = bloom_log2;
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, bloom_log2, &bf_wg_per_cu));
         size_t free_b = 0, total_b = 0;
         HIP_TRY(hipMemGetInfo(&free_b, &total_b));
         const size_t budget = std::min<size_t>((free_b + idx->bf_alloc_bytes) / 3, (size_t)64 << 30);
@@ -327,7 +329,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const size_t stride = packed ? stride_packed : stride_bytes;
         if (packed != idx->bf_packed) idx->bf_stride = 0;  // forces a fresh, zeroed allocation
         idx->bf_packed = packed;
-        if (packed) HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, true, &bf_wg_per_cu));
+        if (packed) HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, true, bloom_log2, &bf_wg_per_cu));
         int slots = (int)std::min<size_t>((size_t)need, budget / stride);
         // below about four wavefronts per CU the workgroup-per-query kernel is the faster one
         if (bf_wg_per_cu > 0 && (slots >= 4 * idx->num_cu || slots >= Q || t.workgroups > 0) && slots > 0) {
@@ -420,6 +422,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         coral::BestFirstArgs b;
         b.rows_unique = idx->rows_unique == 1;
         b.packed = idx->bf_packed;
+        b.bloom_log2 = idx->bf_bloom_log2;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;
