@@ -54,11 +54,11 @@ __host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log
     const size_t bloom = bloom_log2 ? ((size_t)1 << bloom_log2) / 8 : 0;
     return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + bloom + 15) & ~(size_t)15;
 }
-// the filter size for a beam of L: 64 bits per beam entry rounded up to a power of two, halved while that would leave
+// the filter size for a beam of L: 128 bits per beam entry rounded up to a power of two, halved while that would leave
 // a CU fewer than sixteen wavefronts; none below 4096 bits
 __host__ inline int best_first_bloom_log2(int L) {
     int lg = 12;
-    while (((size_t)1 << lg) < (size_t)64 * L && lg < 17) ++lg;
+    while (((size_t)1 << lg) < (size_t)128 * L && lg < 17) ++lg;
     while (lg >= 12 && best_first_wave_lds_bytes(L, lg) > (size_t)10 * 1024) --lg;
     return lg >= 12 ? lg : 0;
 }
