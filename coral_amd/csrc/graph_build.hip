@@ -392,6 +392,7 @@ __global__ void enh_reverse_kernel(const float* __restrict__ vec, int dim, int m
     const int half = gtid >> 5, nhalf = (gridDim.x * blockDim.x) >> 5;
     const int total = batch * kn;
     const int rounds = (total + nhalf - 1) / nhalf;  // the same trip count for both halves of a wavefront
+    unsigned int n_in = 0u, n_out = 0u;
     for (int rd_i = 0; rd_i < rounds; ++rd_i) {
         const int pair = half + rd_i * nhalf;
         bool active = pair < total;
@@ -445,8 +446,19 @@ __global__ void enh_reverse_kernel(const float* __restrict__ vec, int dim, int m
         if (active && l == 0) {
             if (accept) deg[v] = newdeg;
             owner[v] = INT_MAX;
-            if (stats) atomicAdd(stats + (accept ? 0 : 1), 1ull);
+            n_in += accept ? 1 : 0, n_out += accept ? 0 : 1;
         }
+    }
+    // the two counts of the whole workgroup in one atomic each (millions of pairs would otherwise queue on two words)
+    __shared__ unsigned int s_in, s_out;
+    if (threadIdx.x == 0) s_in = 0u, s_out = 0u;
+    __syncthreads();
+    if (n_in) atomicAdd(&s_in, n_in);
+    if (n_out) atomicAdd(&s_out, n_out);
+    __syncthreads();
+    if (stats && threadIdx.x == 0) {
+        if (s_in) atomicAdd(stats + 0, (unsigned long long)s_in);
+        if (s_out) atomicAdd(stats + 1, (unsigned long long)s_out);
     }
 }
 

@@ -4,9 +4,10 @@
 #include <stdint.h>
 
 namespace coral {
-hipError_t launch_bfs_init(int* hops, int* frontier, int start, int64_t n, hipStream_t st);
+// seen: uint32[ceil(n/32)], one bit per node that has its hop count
+hipError_t launch_bfs_init(int* hops, uint32_t* seen, int* frontier, int start, int64_t n, hipStream_t st);
 hipError_t launch_bfs_expand(const int32_t* nbrs, int R, const int* frontier, int fsize, int* next, int* nsize,
-                             int* hops, int level, hipStream_t st);
+                             int* hops, uint32_t* seen, int level, hipStream_t st);
 hipError_t launch_update_min_hop(const int* hops, int* min_hops, int64_t n, hipStream_t st);
 hipError_t launch_argmax(const int* v, int64_t n, unsigned long long* partial, int nblocks, hipStream_t st);
 hipError_t launch_mark_deleted(const int32_t* ids, int count, int64_t n, uint32_t* deleted, int* bad, hipStream_t st);

@@ -13,20 +13,42 @@
 
 namespace coral {
 
-__global__ void bfs_init_kernel(int* hops, int* frontier, int start, int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+// seen: one bit per node, set when the node gets its hop count.  A frontier node's 32 neighbours are mostly nodes that
+// have theirs already (only the first of a node's many in-edges to arrive sets it), and the bitmap is 32 times
+// smaller than the hop array: it stays in L2 where the hop array does not.
+__global__ void bfs_init_kernel(int* hops, uint32_t* seen, int* frontier, int start, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
         hops[i] = i == start ? 0 : -1;
+        if ((i & 31) == 0) seen[i >> 5] = (start >> 5) == (i >> 5) ? 1u << (start & 31) : 0u;
+    }
     if (blockIdx.x == 0 && threadIdx.x == 0) frontier[0] = start;
 }
 
-// half a wavefront per frontier node: lane = neighbour slot of its 128-byte row
-__global__ void bfs_expand_kernel(const int32_t* __restrict__ nbrs, int R, const int* __restrict__ frontier,
-                                  int frontier_size, int* __restrict__ next_frontier, int* __restrict__ next_size,
-                                  int* __restrict__ hops, int level) {
+// half a wavefront per frontier node: lane = neighbour slot of its 128-byte row.  Newly reached nodes are collected
+// in LDS and handed to the next frontier a few thousand at a time: one atomic on the frontier's counter per flush
+// instead of one per wavefront and step (millions on one address per search otherwise).
+constexpr int kBfsStage = 4096;
+__global__ __launch_bounds__(256) void bfs_expand_kernel(const int32_t* __restrict__ nbrs, int R,
+                                                        const int* __restrict__ frontier, int frontier_size,
+                                                        int* __restrict__ next_frontier, int* __restrict__ next_size,
+                                                        int* __restrict__ hops, uint32_t* __restrict__ seen, int level) {
+    __shared__ int s_buf[kBfsStage];
+    __shared__ int s_cnt, s_base;
     const int gtid = blockIdx.x * blockDim.x + threadIdx.x;
     const int group = gtid >> 5, lane32 = gtid & 31, ngroups = (gridDim.x * blockDim.x) >> 5;
     const int lane = threadIdx.x & 63;
-    const int rounds = (frontier_size + ngroups - 1) / ngroups;  // uniform trip count for the ballots
+    const int rounds = (frontier_size + ngroups - 1) / ngroups;  // uniform trip count for ballots and barriers
+    if (threadIdx.x == 0) s_cnt = 0;
+    __syncthreads();
+    auto flush = [&]() {  // all threads
+        const int cnt = s_cnt;
+        if (threadIdx.x == 0 && cnt > 0) s_base = atomicAdd(next_size, cnt);
+        __syncthreads();
+        for (int i = threadIdx.x; i < cnt; i += 256) next_frontier[s_base + i] = s_buf[i];
+        __syncthreads();
+        if (threadIdx.x == 0) s_cnt = 0;
+        __syncthreads();
+    };
     for (int r = 0; r < rounds; ++r) {
         const int i = group + r * ngroups;
         bool valid = false;
@@ -34,15 +56,23 @@ __global__ void bfs_expand_kernel(const int32_t* __restrict__ nbrs, int R, const
         if (i < frontier_size && lane32 < R) v = nbrs[(size_t)frontier[i] * R + lane32];
         // a row ends at its first negative entry: only the lanes below it hold neighbours
         const unsigned int ends = (unsigned int)(__ballot(v < 0) >> (lane & 32));
-        if (lane32 < __ffs((int)ends) - 1 || ends == 0u) valid = atomicCAS(hops + v, -1, level) == -1;
+        if (lane32 < __ffs((int)ends) - 1 || ends == 0u) {
+            const uint32_t bit = 1u << (v & 31);
+            // look before the atomic: a set bit stays set
+            if ((seen[v >> 5] & bit) == 0u) valid = (atomicOr(seen + (v >> 5), bit) & bit) == 0u;
+            if (valid) hops[v] = level;
+        }
         const unsigned long long m = __ballot(valid);
         if (m) {
             int base = 0;
-            if (lane == __ffsll((long long)m) - 1) base = atomicAdd(next_size, __popcll(m));
+            if (lane == __ffsll((long long)m) - 1) base = atomicAdd(&s_cnt, __popcll(m));
             base = __shfl(base, __ffsll((long long)m) - 1, 64);
-            if (valid) next_frontier[base + __popcll(m & ((1ull << lane) - 1ull))] = v;
+            if (valid) s_buf[base + __popcll(m & ((1ull << lane) - 1ull))] = v;
         }
+        __syncthreads();
+        if (s_cnt > kBfsStage - 256) flush();  // a step adds at most 256
     }
+    flush();
 }
 
 // src/start.cu:20-30
@@ -93,16 +123,16 @@ hipError_t launch_mark_deleted(const int32_t* ids, int count, int64_t n, uint32_
     hipLaunchKernelGGL(mark_deleted_kernel, dim3((count + 255) / 256), dim3(256), 0, st, ids, count, n, deleted, bad);
     return hipGetLastError();
 }
-hipError_t launch_bfs_init(int* hops, int* frontier, int start, int64_t n, hipStream_t st) {
-    hipLaunchKernelGGL(bfs_init_kernel, dim3(1024), dim3(256), 0, st, hops, frontier, start, n);
+hipError_t launch_bfs_init(int* hops, uint32_t* seen, int* frontier, int start, int64_t n, hipStream_t st) {
+    hipLaunchKernelGGL(bfs_init_kernel, dim3(1024), dim3(256), 0, st, hops, seen, frontier, start, n);
     return hipGetLastError();
 }
 hipError_t launch_bfs_expand(const int32_t* nbrs, int R, const int* frontier, int fsize, int* next, int* nsize,
-                             int* hops, int level, hipStream_t st) {
+                             int* hops, uint32_t* seen, int level, hipStream_t st) {
     int blocks = (fsize * 32 + 255) / 256;
     blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
     hipLaunchKernelGGL(bfs_expand_kernel, dim3(blocks), dim3(256), 0, st, nbrs, R, frontier, fsize, next, nsize, hops,
-                       level);
+                       seen, level);
     return hipGetLastError();
 }
 hipError_t launch_update_min_hop(const int* hops, int* min_hops, int64_t n, hipStream_t st) {

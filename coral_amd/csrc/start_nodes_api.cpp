@@ -18,10 +18,11 @@ extern "C" int coral_start_ids_fps(coral_index* idx, int32_t first_id, int32_t M
     const int64_t n = idx->n;
     const int nblocks = 512;
     int *hops = nullptr, *min_hops = nullptr, *fa = nullptr, *fb = nullptr, *sizes = nullptr;
+    uint32_t* seen = nullptr;
     unsigned long long* partial = nullptr;
     auto release = [&]() {
         (void)hipFree(hops), (void)hipFree(min_hops), (void)hipFree(fa), (void)hipFree(fb);
-        (void)hipFree(sizes), (void)hipFree(partial);
+        (void)hipFree(sizes), (void)hipFree(partial), (void)hipFree(seen);
     };
 #define TRY_R(expr)                                                                      \
     do {                                                                                 \
@@ -36,6 +37,7 @@ extern "C" int coral_start_ids_fps(coral_index* idx, int32_t first_id, int32_t M
     TRY_R(hipMalloc(&min_hops, n * sizeof(int)));
     TRY_R(hipMalloc(&fa, n * sizeof(int)));
     TRY_R(hipMalloc(&fb, n * sizeof(int)));
+    TRY_R(hipMalloc(&seen, (((size_t)n + 31) / 32 + 1) * sizeof(uint32_t)));
     TRY_R(hipMalloc(&sizes, 2 * sizeof(int)));
     TRY_R(hipMalloc(&partial, nblocks * sizeof(unsigned long long)));
     TRY_R(coral::launch_fill_u32((uint32_t*)min_hops, (size_t)n, (uint32_t)INT_MAX, st));
@@ -44,12 +46,12 @@ extern "C" int coral_start_ids_fps(coral_index* idx, int32_t first_id, int32_t M
     out_ids[count++] = start;
     while (count < M) {
         // one breadth-first search from the id selected last (src/start.cu:53-72)
-        TRY_R(coral::launch_bfs_init(hops, fa, start, n, st));
+        TRY_R(coral::launch_bfs_init(hops, seen, fa, start, n, st));
         int fsize = 1, level = 1;
         int *cur = fa, *next = fb;
         while (fsize > 0) {
             TRY_R(coral::launch_fill_u32((uint32_t*)sizes, 1, 0u, st));
-            TRY_R(coral::launch_bfs_expand(idx->d_nbrs, idx->R, cur, fsize, next, sizes, hops, level++, st));
+            TRY_R(coral::launch_bfs_expand(idx->d_nbrs, idx->R, cur, fsize, next, sizes, hops, seen, level++, st));
             TRY_R(hipMemcpyAsync(&fsize, sizes, sizeof(int), hipMemcpyDeviceToHost, st));
             TRY_R(hipStreamSynchronize(st));
             std::swap(cur, next);
