@@ -5,9 +5,9 @@
 // measure the new ones, insert them, pick the closest entry not yet expanded.  Every step is a chain of dependent
 // memory accesses; what makes it fast on this GPU is how many such chains run side by side.  A workgroup per query
 // with the visited set in LDS (the form beam_search.hip gives this policy) holds two queries per CU.  Here a query
-// needs one wavefront and 5.4 KB of LDS at L = 512 (its sorted beam, merged in place): sixteen queries per CU, as
-// many as 128 registers per lane allow, enough to keep HBM busy (2.6 times the throughput of the other form at a
-// million nodes; more wavefronts add nothing).  The visited set moves to global memory in the form the CPU path
+// needs one wavefront and 9.5 KB of LDS at L = 512 (its sorted beam, merged in place, and a filter over its visited
+// ids): sixteen queries per CU, as many as 128 registers per lane allow, enough to keep HBM busy (2.8 times the
+// throughput of the other form at a million nodes; more wavefronts add nothing).  The visited set moves to global memory in the form the CPU path
 // itself uses (src/search_in_cpu.cpp:44-48, 68-71): one byte per node and query slot holding the epoch of the
 // query that last visited the node, so nothing is cleared between queries (every 255th query of a slot wipes its
 // array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a million nodes); each test costs a
