@@ -264,14 +264,15 @@ Test_Result IndexGPU::Search_and_Verify(const float* queries, const int* gts, in
         release();
         throw std::runtime_error("Search_and_Verify: device allocation or upload failed");
     }
-    // the reference prepares once per process (a function-local static, src/index_gpu.cpp:101-108)
-    // and breaks if a later call is larger; here a change of (num, L) prepares again
-    if (!verify_prepared_ || verify_Q_ < num || verify_L_ != L) {
-        if (coral_search_prepare(index_, num, L, nullptr)) {
-            release();
-            raise("search_prepare");
-        }
-        verify_prepared_ = true, verify_Q_ = num, verify_L_ = L;
+    // the reference prepares once per process (a function-local static, src/index_gpu.cpp:101-108) and breaks if a
+    // later call is larger; here every call states its batch, beam and traversal (other calls on this index may
+    // have prepared it differently in between, and preparing what is already there costs next to nothing)
+    coral_tuning tuning;
+    std::memset(&tuning, 0, sizeof tuning);
+    tuning.policy = GetPolicy();
+    if (coral_search_prepare(index_, num, L, &tuning)) {
+        release();
+        raise("search_prepare");
     }
     coral_stats st;
     int64_t hits = 0;

@@ -151,8 +151,6 @@ class CORAL_API IndexGPU {
     std::vector<int32_t> nbrs_;
     std::string graph_dir_;
     coral_index* index_ = nullptr;
-    bool verify_prepared_ = false;
-    int verify_Q_ = 0, verify_L_ = 0;
 };
 
 }  // namespace efanna2e
