@@ -29,6 +29,8 @@ HBM_PEAK_GBPS = 8000.0
 # measured offline (profiles/beam_search_kernel_1Mx200_L*.md; FETCH_SIZE reads half the bytes of a
 # 1 GiB copy on this GPU, so its factor is 2.0; WRITE_SIZE's is 1.0).  None = not measured.
 MEASURED_TRAFFIC_BYTES = {256: 1.3825e+11, 512: 2.6955e+11}
+# the same for the best-first kernel at L = 512 (profiles/best_first_wave_kernel_1Mx200_L512.md)
+BEST_FIRST_TRAFFIC_BYTES = {512: 1.314e+11}
 
 
 def algorithmic_bytes(expansions, dist_evals, Q, dim, k, R=32):
@@ -194,6 +196,7 @@ def main():
                                                            "dist_evals_per_query", "expansions_per_query")}
         out["best_first"]["kernel"] = "best_first_wave_kernel"
         out["best_first"]["frac"] = best_first["gbps"] / HBM_PEAK_GBPS
+        out["best_first"]["traffic"] = BEST_FIRST_TRAFFIC_BYTES.get(best_first["L"])
 
     # the IndexGPU::Search shape: host buffers in and out (query upload to the index's staging buffers,
     # search, id download); reported beside the headline, never as the headline
