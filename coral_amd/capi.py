@@ -103,6 +103,7 @@ SIGNATURES = {
                                             C.c_void_p, C.c_void_p]),
     "coral_build_enhance_top_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                                 C.c_void_p, C.c_void_p]),
+    "coral_build_resume": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_build_top_hit_ids": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "coral_build_connect_enhance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_build_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
@@ -262,6 +263,20 @@ class Index:
 
     def build_end(self):
         _check(lib().coral_build_end(self._h))
+
+    def build_resume(self, nbrs, dists, hits=None):
+        """construction state from the rows [n][R], distances and hit counts of an earlier build"""
+        nbrs = np.ascontiguousarray(nbrs, np.int32)
+        dists = np.ascontiguousarray(dists, np.float32)
+        if nbrs.ndim != 2 or nbrs.shape[0] != self.n or dists.shape != nbrs.shape:
+            raise ValueError("nbrs and dists must both be [n][R]")
+        if hits is not None:
+            hits = np.ascontiguousarray(hits, np.uint32)
+            if hits.shape != (self.n,):
+                raise ValueError("hits must be [n]")
+        _check(lib().coral_build_resume(self._h, nbrs.shape[1], _ptr(nbrs), _ptr(dists),
+                                        _ptr(hits) if hits is not None else None))
+        self.R = nbrs.shape[1]
 
     def build_nap_batch(self, d_knn_ids, batch, k_b, need_discard=True):
         """d_knn_ids: device pointer (int) to int32 [batch][k_b]."""

@@ -451,6 +451,32 @@ int coral_start_ids_write(const char* dir, const int32_t* ids, int32_t count) {
     return CORAL_OK;
 }
 
+// ----------------------------------------------------------------- hit counts
+int coral_hits_read(const char* dir, uint32_t* hits, int64_t n) {
+    if (!dir || !hits || n <= 0) return fail(CORAL_ERR_ARG, "bad argument");
+    const std::string path = std::string(dir) + "/hits.bin";
+    File f(path.c_str(), "rb");
+    if (!f.f) return fail(CORAL_ERR_IO, "open file error: %s", path.c_str());
+    int64_t stored = 0;
+    if (std::fread(&stored, sizeof stored, 1, f.f) != 1) return fail(CORAL_ERR_IO, "%s: short header", path.c_str());
+    if (stored < n)
+        return fail(CORAL_ERR_IO, "%s holds %lld counts, the index has %lld nodes", path.c_str(), (long long)stored,
+                    (long long)n);
+    if (std::fread(hits, sizeof(uint32_t), (size_t)n, f.f) != (size_t)n)
+        return fail(CORAL_ERR_IO, "%s: truncated", path.c_str());
+    return CORAL_OK;
+}
+
+int coral_hits_write(const char* dir, const uint32_t* hits, int64_t n) {
+    if (!dir || !hits || n <= 0) return fail(CORAL_ERR_ARG, "bad argument");
+    const std::string path = std::string(dir) + "/hits.bin";
+    File f(path.c_str(), "wb");
+    if (!f.f) return fail(CORAL_ERR_IO, "cannot create %s", path.c_str());
+    if (std::fwrite(&n, sizeof n, 1, f.f) != 1 || std::fwrite(hits, sizeof(uint32_t), (size_t)n, f.f) != (size_t)n)
+        return fail(CORAL_ERR_IO, "%s: short write", path.c_str());
+    return CORAL_OK;
+}
+
 // ----------------------------------------------------------------- RoarGraph
 int coral_roargraph_read(const char* path, int64_t n, int32_t R, int32_t* nbrs, int32_t* ep) {
     if (!path || !nbrs || !ep || n <= 0 || R <= 0) return fail(CORAL_ERR_ARG, "bad argument");

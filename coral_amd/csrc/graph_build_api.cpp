@@ -130,6 +130,37 @@ int coral_build_end(coral_index* idx) {
     return CORAL_OK;
 }
 
+int coral_build_resume(coral_index* idx, int32_t R, const int32_t* h_nbrs, const float* h_dists,
+                       const uint32_t* h_hits) {
+    if (!idx || !h_nbrs || !h_dists) return fail(CORAL_ERR_ARG, "null argument");
+    const int64_t n = idx->n;
+    if (R <= 0 || R > coral::kBuildMaxR) return fail(CORAL_ERR_ARG, "R must be in 1..%d (got %d)", coral::kBuildMaxR, R);
+    // a row is its first deg cells: every id in range, nothing after the first -1
+    std::vector<int32_t> deg((size_t)n);
+    int64_t bad = -1;
+#pragma omp parallel for schedule(static) reduction(max : bad)
+    for (int64_t i = 0; i < n; ++i) {
+        const int32_t* row = h_nbrs + (size_t)i * R;
+        int d = 0;
+        while (d < R && row[d] >= 0) ++d;
+        bool ok = true;
+        for (int j = 0; j < R; ++j)
+            if (j < d ? row[j] >= n : row[j] != -1) ok = false;
+        deg[(size_t)i] = d;
+        if (!ok) bad = std::max(bad, i);
+    }
+    if (bad >= 0)
+        return fail(CORAL_ERR_GRAPH, "row %lld is not a row of a build (ids in range, -1 only at the end)",
+                    (long long)bad);
+    if (int rc = coral_build_begin(idx, R)) return rc;
+    const size_t cells = (size_t)n * R;
+    HIP_TRY(hipMemcpy(idx->d_nbrs, h_nbrs, cells * sizeof(int32_t), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(idx->d_nbr_dists, h_dists, cells * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(idx->d_deg, deg.data(), (size_t)n * sizeof(int32_t), hipMemcpyHostToDevice));
+    if (h_hits) HIP_TRY(hipMemcpy(idx->d_hits, h_hits, (size_t)n * sizeof(uint32_t), hipMemcpyHostToDevice));
+    return CORAL_OK;
+}
+
 int coral_build_nap_batch(coral_index* idx, const int32_t* d_knn_ids, int32_t batch, int32_t k_b, int32_t need_discard) {
     if (!idx || !d_knn_ids) return fail(CORAL_ERR_ARG, "null argument");
     if (!idx->building) return fail(CORAL_ERR_STATE, "coral_build_begin has not been called");

@@ -153,7 +153,7 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     SetParameters(parameters);
     load_config(parameters.Get<std::string>("config_file", std::string("default")));
     const int CE = parameters.Get<int>("CE");
-    if (CE != 0 && CE != 1) throw std::runtime_error("BuildGPU: CE must be 0 or 1 (2, enhancement only, is not provided)");
+    if (CE < 0 || CE > 2) throw std::runtime_error("BuildGPU: CE must be 0 (none), 1 (after the build) or 2 (only)");
     max_degree_ = parameters.Get<int>("max_degree");
     k_ = parameters.Get<int>("k");
     metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
@@ -180,18 +180,34 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     p.enhance_search_batch = PC.enhance_search_batch, p.enhance_nap_batch = PC.enhance_nap_batch;
     p.top_hit_num = PC.top_hit_num;
     p.n_start = PC.search_start_nodes_num;
-    const std::string train_gt = parameters.Get<std::string>("train_gt_file", std::string("None"));
-    if (train_gt != "None" && !train_gt.empty()) {
-        // clusters from a ground-truth file of the sampled queries (src/index_gpu.cpp:505-515: nq, k, ids)
-        int32_t nq = 0, gk = 0;
-        if (coral_gt_read_meta(train_gt.c_str(), &nq, &gk)) raise("train_gt_file");
-        if (gk != k_) throw std::runtime_error("BuildGPU: train_gt_file holds k=" + std::to_string(gk) + ", expected " +
-                                               std::to_string(k_));
-        std::vector<int32_t> clusters((size_t)nq * gk);
-        if (coral_gt_read(train_gt.c_str(), clusters.data(), nq, gk)) raise("train_gt_file");
-        if (coral_build_graph_from_clusters(index_, clusters.data(), nq, &p, &last_build)) raise("BuildGPU");
-    } else if (coral_build_graph(index_, sq_data, (int64_t)n_sq, &p, &last_build)) {
-        raise("BuildGPU");
+    std::vector<uint32_t> hits(nd_);
+    if (CE == 2) {
+        // enhancement only (src/index_gpu.cpp:332-333, 367-373): the rows, their distances and the hit counts of an
+        // earlier BuildGPU with CE 0 come back from graph_file
+        nbrs_.assign(nd_ * (size_t)max_degree_, -1);
+        std::vector<float> saved(nd_ * (size_t)max_degree_);
+        if (coral_graph_dir_read(graph_dir_.c_str(), (int64_t)nd_, max_degree_, nbrs_.data(), saved.data()))
+            raise("BuildGPU: load graph");
+        if (coral_hits_read(graph_dir_.c_str(), hits.data(), (int64_t)nd_)) raise("BuildGPU: load hits");
+        if (coral_build_resume(index_, max_degree_, nbrs_.data(), saved.data(), hits.data())) raise("BuildGPU");
+        p.connect_enhance = 1;
+        if (coral_build_connect_enhance(index_, &p, &last_build)) raise("BuildGPU");
+    } else {
+        const std::string train_gt = parameters.Get<std::string>("train_gt_file", std::string("None"));
+        if (train_gt != "None" && !train_gt.empty()) {
+            // clusters from a ground-truth file of the sampled queries (src/index_gpu.cpp:505-515: nq, k, ids)
+            int32_t nq = 0, gk = 0;
+            if (coral_gt_read_meta(train_gt.c_str(), &nq, &gk)) raise("train_gt_file");
+            if (gk != k_) throw std::runtime_error("BuildGPU: train_gt_file holds k=" + std::to_string(gk) + ", expected " +
+                                                   std::to_string(k_));
+            std::vector<int32_t> clusters((size_t)nq * gk);
+            if (coral_gt_read(train_gt.c_str(), clusters.data(), nq, gk)) raise("train_gt_file");
+            if (coral_build_graph_from_clusters(index_, clusters.data(), nq, &p, &last_build)) raise("BuildGPU");
+        } else if (coral_build_graph(index_, sq_data, (int64_t)n_sq, &p, &last_build)) {
+            raise("BuildGPU");
+        }
+        // gpufuncs->save_hits() (src/index_gpu.cpp:362): the counts are complete once the clusters are through
+        if (coral_build_top_hit_ids(index_, 0, nullptr, hits.data())) raise("BuildGPU");
     }
     // Graph::save_build (include/graph.cuh:481-484): start ids, then every row with its distances
     nbrs_.assign(nd_ * (size_t)max_degree_, -1);
@@ -204,6 +220,7 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     if (coral_graph_dir_write(graph_dir_.c_str(), (int64_t)nd_, max_degree_, nbrs_.data(), dists.data()))
         raise("save graph");
     if (coral_start_ids_write(graph_dir_.c_str(), start_ids_.data(), (int32_t)start_ids_.size())) raise("save start ids");
+    if (coral_hits_write(graph_dir_.c_str(), hits.data(), (int64_t)nd_)) raise("save hits");
 }
 
 void IndexGPU::LoadRoarGraph(std::string filename) {

@@ -18,6 +18,8 @@ SIGNATURES = {
     "coral_graph_dir_write": (C.c_int, [C.c_char_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),
     "coral_start_ids_read": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int32, C.POINTER(C.c_int32)]),
     "coral_start_ids_write": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int32]),
+    "coral_hits_read": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int64]),
+    "coral_hits_write": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int64]),
     "coral_roargraph_read": (C.c_int, [C.c_char_p, C.c_int64, C.c_int32, C.c_void_p, C.POINTER(C.c_int32)]),
     "coral_roargraph_write": (C.c_int, [C.c_char_p, C.c_int64, C.c_int32, C.c_void_p, C.c_int32]),
     "coral_lz4_compress_bound": (C.c_int, [C.c_int]),
@@ -114,6 +116,18 @@ def start_ids_read(path, capacity=4096):
 def start_ids_write(path, ids):
     ids = np.ascontiguousarray(ids, dtype=np.int32)
     _check(_L().coral_start_ids_write(_s(path), _p(ids), ids.size))
+
+
+def hits_read(path, n):
+    """<path>/hits.bin -> uint32 [n] (include/ivf.cuh:647-656)"""
+    hits = np.empty(n, dtype=np.uint32)
+    _check(_L().coral_hits_read(_s(path), _p(hits), n))
+    return hits
+
+
+def hits_write(path, hits):
+    hits = np.ascontiguousarray(hits, dtype=np.uint32)
+    _check(_L().coral_hits_write(_s(path), _p(hits), hits.size))
 
 
 def roargraph_read(path, n, R=32):

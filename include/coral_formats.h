@@ -60,6 +60,11 @@ CORAL_API int coral_graph_dir_write(const char* dir, int64_t n, int32_t R, const
 CORAL_API int coral_start_ids_read(const char* dir, int32_t* ids, int32_t capacity, int32_t* count);
 CORAL_API int coral_start_ids_write(const char* dir, const int32_t* ids, int32_t count);
 
+/* IVFBuilder::save_hits / load_hits (include/ivf.cuh:639-656): <dir>/hits.bin = int64 n, then uint32[n], how many
+ * clusters of the build contained each node.  read fails when the file holds fewer than n counts. */
+CORAL_API int coral_hits_read(const char* dir, uint32_t* hits, int64_t n);
+CORAL_API int coral_hits_write(const char* dir, const uint32_t* hits, int64_t n);
+
 /* Graph::LoadRoarGraph: degrees above R are truncated to R as the reference does */
 CORAL_API int coral_roargraph_read(const char* path, int64_t n, int32_t R, int32_t* nbrs, int32_t* ep);
 CORAL_API int coral_roargraph_write(const char* path, int64_t n, int32_t R, const int32_t* nbrs,

@@ -235,6 +235,13 @@ CORAL_API int coral_build_begin(coral_index* idx, int32_t R);
 /* frees the per-neighbour distances and the staging; the rows and start ids stay */
 CORAL_API int coral_build_end(coral_index* idx);
 
+/* Graph ctor in Mode::CE (include/graph.cuh:252-256, DS.load_batch_slots of every node): construction state from
+ * rows of an earlier build, as coral_index_get_graph handed them out before coral_build_end (h_nbrs [n][R] with -1
+ * after the last neighbour, h_dists [n][R] the neighbours' distances), and the per-node cluster counts (h_hits [n], or
+ * NULL for zeros; IVFBuilder::load_hits, include/ivf.cuh:647-656).  coral_build_connect_enhance can follow. */
+CORAL_API int coral_build_resume(coral_index* idx, int32_t R, const int32_t* h_nbrs, const float* h_dists,
+                                 const uint32_t* h_hits);
+
 /* GPUFuncs::graph_update -> gpu_neibor_aware (src/upd_disk.cu:218-224, src/upd_gpu.cu:260-303): one batch of
  * clusters, d_knn_ids int32 [batch][k_b] on the device, distinct ids per row.  Every member becomes a pivot:
  * candidates = the other members (pairs where both sides already have neighbours are left out) + its current row;

@@ -221,6 +221,27 @@ def test_start_ids_text(tmp_path):
     assert F.start_ids_read(tmp_path / "idx").size == 0
 
 
+def test_hits_file(tmp_path):
+    """hits.bin = int64 n + uint32[n] (include/ivf.cuh:639-656); a file of more counts serves a smaller index"""
+    os.makedirs(tmp_path / "idx")
+    hits = np.array([3, 0, 7, 4000000000, 1], np.uint32)
+    F.hits_write(tmp_path / "idx", hits)
+    raw = (tmp_path / "idx" / "hits.bin").read_bytes()
+    assert raw == struct.pack("<q", 5) + hits.tobytes()
+    assert F.hits_read(tmp_path / "idx", 5).tolist() == hits.tolist()
+    assert F.hits_read(tmp_path / "idx", 3).tolist() == hits[:3].tolist()
+    with pytest.raises(Exception) as e:
+        F.hits_read(tmp_path / "idx", 6)
+    assert "holds 5 counts" in str(e.value)
+    (tmp_path / "idx" / "hits.bin").write_bytes(raw[:-2])
+    with pytest.raises(Exception) as e:
+        F.hits_read(tmp_path / "idx", 5)
+    assert "truncated" in str(e.value)
+    with pytest.raises(Exception) as e:
+        F.hits_read(tmp_path / "elsewhere", 5)
+    assert "elsewhere" in str(e.value)
+
+
 def test_roargraph_file(tmp_path):
     g, _, deg = _graph(12, 6, 4)
     p = tmp_path / "roar.index"

@@ -224,6 +224,49 @@ def test_whole_construction_equals_the_oracle_pipeline(orc, metric, ce, seed, to
     assert np.array_equal(ids, ids2) and dd.tobytes() == dd2.tobytes()
 
 
+def test_enhancement_alone_on_a_resumed_build_equals_the_whole_construction():
+    """rows, distances and hit counts of a construction without enhancement, handed to a new index
+    (coral_build_resume), then coral_build_connect_enhance: the state a construction with enhancement ends in."""
+    n, dim, A = 12000, 48, 900
+    base = base_of(n, dim, 310, capi.L2)
+    aux = make_queries(A, dim, 410)
+    kw = dict(R=16, k_b=24, batch=128, enhance_search_batch=5000, enhance_nap_batch=700, enhance_L=64, n_start=8,
+              top_hit_num=9000)
+    idx = capi.Index(base, None, None)
+    idx.build_graph(aux, capi.build_params(connect_enhance=1, **kw))
+    want = idx.get_graph(with_build_state=True)
+    idx.close()
+    idx = capi.Index(base, None, None)
+    idx.build_graph(aux, capi.build_params(connect_enhance=0, **kw))
+    nbrs, dists, deg, _ = idx.get_graph(with_build_state=True)
+    _, hits = idx.build_top_hit_ids(0)
+    idx.close()
+    assert (deg == 0).sum() > 1000 and hits.sum() == A * 24
+    idx = capi.Index(base, None, None)
+    idx.build_resume(nbrs, dists, hits)
+    got = idx.get_graph(with_build_state=True)
+    assert np.array_equal(got[0], nbrs) and got[1].tobytes() == dists.tobytes() and np.array_equal(got[2], deg)
+    stats = idx.build_connect_enhance(capi.build_params(connect_enhance=1, **kw))
+    got = idx.get_graph(with_build_state=True)
+    assert stats.isolated == (deg == 0).sum() and stats.top_hit_nodes == 9000 - stats.isolated
+    for g, w in zip(got, want):
+        assert g.tobytes() == w.tobytes()
+    # rows that no build could have left are turned away, and the index stays as it was
+    broken = nbrs.copy()
+    broken[5, 3] = n
+    with pytest.raises(capi.CoralError) as e:
+        idx.build_resume(broken, dists, hits)
+    assert e.value.code == 2 and "row 5" in str(e.value)
+    broken = nbrs.copy()
+    row = int(np.where(deg == 0)[0][0])
+    broken[row, 1] = 7  # a neighbour after the end of the row
+    with pytest.raises(capi.CoralError) as e:
+        idx.build_resume(broken, dists, None)
+    assert e.value.code == 2 and "row %d" % row in str(e.value)
+    assert np.array_equal(idx.get_graph(with_build_state=True)[0], want[0])
+    idx.close()
+
+
 def test_builder_argument_errors():
     base = synth.gaussian_matrix(1, 100, 8)
     idx = capi.Index(base, None, None)
@@ -274,6 +317,7 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
             "--query_test_file", str(work / "query.fbin"), "--gt_test_file", str(work / "gt24.bin")]
     gt24, _ = orc.bruteforce(base, q, 24)
     formats.gt_write(work / "gt24.bin", gt24)
+    build_args = args
     r = subprocess.run(args, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr + r.stdout
     index_dir = work / "indexes" / "syn_l2_16_1.0_1"  # ../indexes/<dataset>_<dist>_<R>_<thres>_<CE>
@@ -322,6 +366,25 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     r = subprocess.run(args2[:-4] + ["--k", "25", "--train_gt_file", str(work / "clusters.bin")], cwd=work / "cwd",
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 1 and "expected 25" in r.stderr
+    # --CE 0, then --CE 2 (enhancement only) on what it saved: the directory of the --CE 1 run
+    staged = ["--index_dir", str(work / "staged")]
+    ce_at = build_args.index("--CE") + 1
+    for ce in ("0", "2"):
+        a = build_args[:ce_at] + [ce] + build_args[ce_at + 1:] + staged
+        r = subprocess.run(a, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stderr + r.stdout
+        if ce == "0":
+            nbrs0, _ = formats.graph_dir_read(work / "staged", n, 16, want_dists=True)
+            assert (nbrs0[:, 0] < 0).sum() > 1000 and not np.array_equal(nbrs0, nbrs)
+            hits = formats.hits_read(work / "staged", n)
+            assert hits.sum() == A * 24
+    nbrs3, dists3 = formats.graph_dir_read(work / "staged", n, 16, want_dists=True)
+    assert np.array_equal(nbrs3, nbrs) and dists3.tobytes() == dists.tobytes()
+    assert formats.start_ids_read(work / "staged").tolist() == starts.tolist()
+    assert np.array_equal(formats.hits_read(work / "staged", n), hits)
+    r = subprocess.run(build_args[:ce_at] + ["2"] + build_args[ce_at + 1:] + ["--index_dir", str(work / "nothing_here")],
+                       cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1 and "nothing_here" in r.stderr
 
 
 def test_fewer_reachable_nodes_than_entry_points(orc):
