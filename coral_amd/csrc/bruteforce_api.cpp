@@ -76,10 +76,16 @@ int knn_passes(coral_index* idx, const float* d_queries, int32_t Q, int32_t k, i
 // |b|^2 of the base, once per index
 int ensure_base_norms(coral_index* idx, hipStream_t stream) {
     if (idx->d_bnorm) return CORAL_OK;
-    HIP_TRY(hipMalloc(&idx->d_bnorm_max, sizeof(uint32_t)));
-    HIP_TRY(hipMalloc(&idx->d_bnorm, (size_t)idx->n * sizeof(float)));
-    HIP_TRY(coral::launch_fill_u32(idx->d_bnorm_max, 1, 0u, stream));
-    HIP_TRY(coral::launch_row_norms(idx->d_vec, idx->n, idx->dim, idx->d_bnorm, idx->d_bnorm_max, stream));
+    if (!idx->d_bnorm_max) HIP_TRY(hipMalloc(&idx->d_bnorm_max, sizeof(uint32_t)));
+    float* norms = nullptr;
+    HIP_TRY(hipMalloc(&norms, (size_t)idx->n * sizeof(float)));
+    hipError_t e = coral::launch_fill_u32(idx->d_bnorm_max, 1, 0u, stream);
+    if (e == hipSuccess) e = coral::launch_row_norms(idx->d_vec, idx->n, idx->dim, norms, idx->d_bnorm_max, stream);
+    if (e != hipSuccess) {
+        (void)hipFree(norms);
+        HIP_TRY(e);
+    }
+    idx->d_bnorm = norms;  // kept only once its kernel is on the stream
     return CORAL_OK;
 }
 

@@ -287,6 +287,8 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     int workgroups = t.workgroups > 0 ? t.workgroups : wg_per_cu * idx->num_cu;
     workgroups = std::min(workgroups, (int)Q);
 
+    // from here on buffers are replaced: a failure part-way leaves the index unprepared, not half-prepared
+    idx->prepared = false;
     const size_t spill_words = ((size_t)idx->n + 31) / 32;
     const size_t need_words = spill_words * (size_t)workgroups;
     if (need_words > idx->spill_alloc_words) {

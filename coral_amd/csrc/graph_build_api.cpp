@@ -3,6 +3,8 @@
 //   coral_build_nap_batch        GPUFuncs::graph_update        src/upd_disk.cu:218-224 -> gpu_neibor_aware, src/upd_gpu.cu:260-303
 //   coral_build_connect_enhance  GPUFuncs::gpu_connect_enhance src/enhance.cu:728-861 (enhance_mode 0, isolated nodes)
 //   coral_build_enhance_batch    GPUFuncs::enhance_neibor_aware_gpu src/enhance.cu:660-689
+//   coral_build_enhance_top_batch  its five-argument form      src/enhance.cu:632-658 (most-hit nodes, :819-856)
+//   coral_build_resume           Graph ctor in Mode::CE        include/graph.cuh:252-256 (rows of a saved build)
 #include <algorithm>
 #include <chrono>
 #include <climits>
