@@ -424,7 +424,12 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             __syncthreads();
             const int nexp = s_nexp;
             PHASE_MARK(2);
-            if (nexp == 0) break;
+            if (nexp == 0) {
+                // a round that finds every entry expanded still counts: the candidates of the round that first
+                // overfilled the beam can all have fallen behind its L entries
+                if (a.policy == 0) ++rounds;
+                break;
+            }
 
             // The round's rows are taken in chunks of `ech` beam entries (what the todo
             // list holds).  Requesting graph rows ahead of time (the next chunk's, or for

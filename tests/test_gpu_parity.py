@@ -98,6 +98,25 @@ def test_exact_against_same_order_oracle(orc, case):
     idx.close()
 
 
+def test_tiny_beams_count_their_last_round(orc):
+    """L = 1 and 2: the round that first overfills the beam can leave only expanded entries in it; the round after,
+    which finds nothing to expand, is counted like the oracle's."""
+    n, dim, R = 300, 20, 16
+    base, nbrs, starts = problem(n, dim, R, seed=13, n_start=1, ragged_seed=181)
+    q = make_queries(3000, dim, 313)
+    idx = capi.Index(base, nbrs, starts)
+    seen = 0
+    for L in (1, 2):
+        oi, od, os_, _ = orc.search_B(orc.Problem(base, nbrs, starts), q, L, L, start_order=WAVE64, nbr_order=WAVE64)
+        idx.prepare(q.shape[0], L)
+        ids, dists, _ = idx.search(q, L, L)
+        assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+        assert np.array_equal(idx.query_counters(q.shape[0]), os_)
+        seen += int(((os_[:, 1] == 1) & (os_[:, 3] == 2)).sum())
+    assert seen > 0  # one row read, two rounds: the case above
+    idx.close()
+
+
 def test_best_first_query_slots_are_reused(orc):
     """The wavefront-per-query kernel keeps one byte of visited state per node and query slot and tells queries
     apart by an epoch that wraps at 256: eight slots serve 2400 queries (300 each), twice, on a graph whose rows
