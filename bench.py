@@ -86,10 +86,11 @@ def shipped_config_leg(w):
     return out
 
 
-def structured_leg():
+def structured_leg(with_cpu=True):
     """The same path on data that has neighbourhood structure (workloads.structured: 1M x 200 near a 16-dimensional
     subspace, same construction, same k): recall@100 >= 0.90 exists there, and the line reports the best rate at or
-    above it for each policy.  Beside the headline, never the headline."""
+    above it for each policy, with the reference's CPU search at the beam capacity that gets its traversal
+    (best-first) there.  Beside the headline, never the headline."""
     import torch
     from coral_amd import capi, workloads
     w = workloads.structured()
@@ -101,13 +102,18 @@ def structured_leg():
     d_ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
     d_gt = torch.from_numpy(gt).cuda()
     out = {"workload": w["name"], "graph_total_s": w["build"]["total_s"]}
-    for name, policy, Ls in (("rounds", capi.POLICY_ROUNDS, (128, 192, 256)),
-                             ("best_first", capi.POLICY_BEST_FIRST, (256, 384, 512))):
+    for name, policy, Ls in (("rounds", capi.POLICY_ROUNDS, (128, 144, 160, 192, 256)),
+                             ("best_first", capi.POLICY_BEST_FIRST, (256, 288, 320, 384, 512))):
         rows = [measure(idx, d_q, d_ids, d_gt, Q, k, dim, L, 3, 1, policy) for L in Ls]
         out[name] = [{"L": r["L"], "qps": r["qps"], "recall": r["recall"], "frac": r["gbps"] / HBM_PEAK_GBPS,
                       "dist_evals_per_query": r["dist_evals_per_query"]} for r in rows]
         ok = [r for r in rows if r["recall"] >= 0.90]
         out[name + "_qps_at_recall_0.90"] = max(r["qps"] for r in ok) if ok else None
+        if ok and name == "best_first" and with_cpu:
+            fastest = max(ok, key=lambda r: r["qps"])
+            cpu = cpu_baseline(w, gt, fastest["L"], k)
+            out["cpu_at_recall_0.90"] = cpu
+            out["gpu_over_cpu_at_recall_0.90"] = fastest["qps"] / cpu["value"]
     idx.close()
     return out
 
@@ -222,7 +228,7 @@ def main():
     idx.close()
     if not (args.no_structured or args.only_L):
         out["shipped_config_graph"] = optional(shipped_config_leg, w)
-        out["structured"] = optional(structured_leg)
+        out["structured"] = optional(structured_leg, with_cpu=not args.no_cpu)
     print(json.dumps(out), flush=True)
     return 0
 

@@ -224,6 +224,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
     if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
     if (L <= 0 || L > kMaxL) return fail(CORAL_ERR_ARG, "L must be in 1..%d (got %d)", kMaxL, L);
+    if (idx->M <= 0) return fail(CORAL_ERR_STATE, "the graph has no start ids yet (rows under construction)");
     if (idx->M > L)
         return fail(CORAL_ERR_ARG, "%d start ids do not fit a beam of capacity %d", idx->M, L);
     coral_tuning t;

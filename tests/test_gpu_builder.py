@@ -285,6 +285,9 @@ def test_builder_argument_errors():
     idx.build_nap_batch(knn.data_ptr(), 2, 10)
     nbrs, dists, deg, _ = idx.get_graph(with_build_state=True)
     assert (deg[:20] > 0).all() and (deg[20:] == 0).all()
+    with pytest.raises(capi.CoralError) as e:  # rows exist, entry points do not yet
+        idx.search(base[:3], 2, 8)
+    assert e.value.code == capi.ERR_STATE and "no start ids" in str(e.value)
     idx.build_end()
     with pytest.raises(capi.CoralError):
         idx.get_graph(with_build_state=True)
