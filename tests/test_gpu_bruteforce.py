@@ -90,6 +90,52 @@ def test_bruteforce_exact_against_oracle(orc, n, dim, Q, k, metric, tomb):
     assert np.allclose(dists[live], td[live], rtol=1e-5, atol=1e-6)
 
 
+def test_randomised_knn_problems_equal_the_oracle(orc):
+    """Seeded random sizes, k, metrics, tombstones and laws of the data (ties on a lattice, repeated vectors, large
+    and small magnitudes, a common offset that makes the screening's error bound bite): the screened path and the
+    exact-only path both return the oracle's ids and distance bits."""
+    redone = 0
+    for c in range(80):
+        rng = np.random.RandomState(7000 + c)
+        n = int(rng.choice([50, 129, 300, 1000, 4097, 10000, 30000]))
+        dim = int(rng.choice([4, 8, 12, 20, 32, 64, 100, 128, 200, 256, 512]))
+        Q = int(rng.choice([1, 5, 37, 128, 129, 300]))
+        k = int(rng.choice([1, 2, 10, 32, 64, 100, 129, 300]))
+        metric = capi.IP if rng.rand() < 0.35 else capi.L2
+        tomb = rng.rand() < 0.3
+        kind = str(rng.choice(["gauss", "lattice", "dups", "big", "tiny", "offset"]))
+        while n * dim * Q > 1e9:
+            Q = max(1, Q // 2)
+        print("case", dict(c=c, n=n, dim=dim, Q=Q, k=k, metric=metric, tomb=tomb, kind=kind), flush=True)
+        base = synth.gaussian_matrix(2000 + c, n, dim)
+        q = synth.shifted_queries(Q, dim, 3 + c, 4 + c, 5 + c)
+        if kind == "lattice":
+            base, q = np.round(base), np.round(q)
+        elif kind == "dups":
+            base[n // 2:] = base[:n - n // 2]
+        elif kind == "big":
+            base, q = base * 1000.0, q * 1000.0
+        elif kind == "tiny":
+            base, q = base * 1e-3, q * 1e-3
+        elif kind == "offset":
+            base, q = base + 50.0, q + 50.0
+        base, q = base.astype(np.float32), q.astype(np.float32)
+        if metric == capi.IP and kind in ("gauss", "dups"):
+            base, q = synth.normalize_rows(base), synth.normalize_rows(q)
+        mask = synth.tombstone_mask(n, 77 + c, int(rng.choice([2, 3, 10]))) if tomb else None
+        oi, od = orc.bruteforce(base, q, k, metric, deleted=mask, order=SEQ)
+        idx = capi.Index(base, None, None, metric)
+        if tomb:
+            idx.set_deleted(mask)
+        for exact_only in (False, True):
+            idx.bruteforce_exact_only(exact_only)
+            ids, dists, _ = idx.bruteforce(q, k, have_delete=tomb)
+            redone += 0 if exact_only else idx.bruteforce_last_redone()
+            assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+        idx.close()
+    assert redone > 0  # some of these queries went through the exact passes after the screening
+
+
 def test_bruteforce_ties_are_ordered_by_id(orc):
     # integer lattice: many exactly equal distances, including across the k-th place
     side = 7

@@ -98,6 +98,60 @@ def test_exact_against_same_order_oracle(orc, case):
     idx.close()
 
 
+def test_randomised_search_problems_equal_the_oracle(orc):
+    """Seeded random sizes, widths, degrees, beam lengths, k, start ids, batch sizes, table sizes, workgroup
+    shapes, ragged rows, repeated ids, tombstones, both metrics, both traversals (best-first in its three kernel
+    forms): ids, distance bits and per-query counters equal the oracle's in the kernel's summation order."""
+    for c in range(120):
+        rng = np.random.RandomState(5000 + c)
+        n = int(rng.choice([300, 700, 2000, 5000, 12000]))
+        dim = int(rng.choice([4, 8, 12, 16, 20, 32, 48, 64, 100, 128, 200, 256, 384, 512, 768, 1024]))
+        R = int(rng.choice([1, 2, 3, 5, 8, 13, 16, 24, 31, 32]))
+        metric = "ip" if rng.rand() < 0.3 else "l2"
+        policy = int(rng.rand() < 0.5)
+        L = min(n, int(rng.choice([1, 2, 5, 16, 33, 64, 100, 128, 200, 256, 300, 512, 700, 1024, 1500, 2048])))
+        k = int(rng.randint(1, L + 1)) if rng.rand() < 0.7 else L
+        M = int(min(L, n, rng.choice([1, 2, 3, 8, 16, 40, 64, 65, 130])))
+        Q = int(rng.choice([1, 3, 17, 64, 150, 400, 1000]))
+        Q = max(1, min(Q, 60000 // max(L, 16)))
+        slots = int(rng.choice([0, 0, 0, 10, 11, 12, 13]))
+        threads = int(rng.choice([0, 0, 128, 256, 512, 1024]))
+        rg = int(rng.randint(1, 1000)) if rng.rand() < 0.4 else None
+        dele, dup = rng.rand() < 0.35, rng.rand() < 0.3
+        wgs = int(rng.choice([0, 0, 1, 2, 7]))
+        print("case", dict(c=c, n=n, dim=dim, R=R, metric=metric, policy=policy, L=L, k=k, M=M, Q=Q, slots=slots,
+                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs), flush=True)
+        m = capi.IP if metric == "ip" else capi.L2
+        base = synth.gaussian_matrix(1000 + c, n, dim)
+        if metric == "ip":
+            base = synth.normalize_rows(base)
+        nbrs = gpu_graph(base, R, metric)
+        if rg is not None:
+            nbrs = ragged(nbrs, rg)
+        if dup and R >= 3:
+            rows = rng.choice(n, n // 3, replace=False)
+            rows = rows[nbrs[rows, R - 1] >= 0]
+            nbrs[rows, R - 1] = nbrs[rows, 0]
+        starts = rng.choice(n, M, replace=False).astype(np.int32)
+        mask = synth.tombstone_mask(n, 50 + c, modulo=int(rng.choice([2, 5, 10]))) if dele else None
+        q = make_queries(Q, dim, 300 + c, metric)
+        prob = orc.Problem(base, nbrs, starts, mask)
+        if policy == 0:
+            oi, od, os_, _ = orc.search_B(prob, q, k, L, metric=m, start_order=WAVE64, nbr_order=WAVE64)
+        else:
+            oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=m, order=WAVE64)
+        idx = capi.Index(base, nbrs, starts, m)
+        if dele:
+            idx.set_deleted(mask)
+        for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
+            idx.prepare(Q, L, visited_slots_log2=slots, threads=threads, workgroups=wgs, policy=policy,
+                        best_first_in_lds=in_lds, best_first_packed=packed)
+            ids, dists, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
+            assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+            assert np.array_equal(idx.query_counters(Q), os_)
+        idx.close()
+
+
 def test_tiny_beams_count_their_last_round(orc):
     """L = 1 and 2: the round that first overfills the beam can leave only expanded entries in it; the round after,
     which finds nothing to expand, is counted like the oracle's."""
