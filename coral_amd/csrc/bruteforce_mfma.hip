@@ -115,46 +115,71 @@ __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel
     for (int k0 = 0; k0 < dim; k0 += BK) {
         const bool more = k0 + BK < dim;
         if (more) fetch(k0 + BK);
+        // the operands of a pair of dimensions are read while the pair before is multiplied
+        float a0 = sa[cur][kh][wr * 64 + m], a1 = sa[cur][kh][wr * 64 + 32 + m];
+        float c0 = sb[cur][kh][wc * 64 + m], c1 = sb[cur][kh][wc * 64 + 32 + m];
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
-            const float a0 = sa[cur][kk + kh][wr * 64 + m], a1 = sa[cur][kk + kh][wr * 64 + 32 + m];
-            const float c0 = sb[cur][kk + kh][wc * 64 + m], c1 = sb[cur][kk + kh][wc * 64 + 32 + m];
+            float a0n = 0.0f, a1n = 0.0f, c0n = 0.0f, c1n = 0.0f;
+            if (kk + 2 < BK) {
+                a0n = sa[cur][kk + 2 + kh][wr * 64 + m], a1n = sa[cur][kk + 2 + kh][wr * 64 + 32 + m];
+                c0n = sb[cur][kk + 2 + kh][wc * 64 + m], c1n = sb[cur][kk + 2 + kh][wc * 64 + 32 + m];
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keeps the reads above ahead of the multiplications below
             acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, c0, acc[0][0], 0, 0, 0);
             acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, c1, acc[0][1], 0, 0, 0);
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, c0, acc[1][0], 0, 0, 0);
             acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, c1, acc[1][1], 0, 0, 0);
+            a0 = a0n, a1 = a1n, c0 = c0n, c1 = c1n;
         }
         if (more) park(cur ^ 1);
         __syncthreads();
         cur ^= 1;
     }
-    // a 32 x 32 block's 16 registers: register v of lane l holds row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32
+    // a 32 x 32 block's 16 registers: register v of lane l holds row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32.
+    // The norms of the tile's rows and columns (+inf for a tombstoned column) come through LDS, fetched once per
+    // workgroup instead of by 64 dependent global loads per lane.
+    float* srow = &sa[0][0][0];  // the operand buffers are free after the last barrier of the loop
+    float* scol = &sb[0][0][0];
     const float inf = __int_as_float(0x7f800000);
+    if (tid < MT) {
+        const int r = q0 + tid;
+        srow[tid] = (metric == 0 && r < nq) ? qn[r] : 0.0f;
+    } else if (tid < MT + NT) {
+        const int64_t c = b0 + (tid - MT);
+        float v = 0.0f;
+        if (c < nb) {
+            if (metric == 0) v = bn[c];
+            if (deleted) {
+                const int64_t id = base_id0 + c;
+                if ((deleted[id >> 5] >> (id & 31)) & 1u) v = inf;
+            }
+        }
+        scol[tid - MT] = v;
+    }
+    __syncthreads();
 #pragma unroll
-    for (int ti = 0; ti < 2; ++ti)
+    for (int ti = 0; ti < 2; ++ti) {
+        float4 rown[4];  // |q|^2 of the 16 rows this lane holds of a block: four runs of four
+#pragma unroll
+        for (int g = 0; g < 4; ++g) rown[g] = *reinterpret_cast<const float4*>(srow + wr * 64 + ti * 32 + 8 * g + 4 * kh);
 #pragma unroll
         for (int tj = 0; tj < 2; ++tj) {
-            const int64_t c = b0 + wc * 64 + tj * 32 + m;
-            bool dead = false;
-            float bnc = 0.0f;
-            if (c < nb) {
-                if (metric == 0) bnc = bn[c];
-                if (deleted) {
-                    const int64_t id = base_id0 + c;
-                    dead = ((deleted[id >> 5] >> (id & 31)) & 1u) != 0;
-                }
-            }
+            const int cl = wc * 64 + tj * 32 + m;
+            const int64_t c = b0 + cl;
+            const float bnc = scol[cl];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = q0 + wr * 64 + ti * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
-                if (r < nq && c < nb) {
-                    const float dot = acc[ti][tj][v];
-                    float s = metric == 0 ? (qn[r] + bnc) - 2.0f * dot : 0.0f - dot;
-                    if (dead) s = inf;
-                    D[(size_t)(r - q0 + (int64_t)blockIdx.y * MT) * ldD + c] = s;
-                }
+                const float4 rn4 = rown[v >> 2];
+                const float rn = (v & 3) == 0 ? rn4.x : (v & 3) == 1 ? rn4.y : (v & 3) == 2 ? rn4.z : rn4.w;
+                const float dot = acc[ti][tj][v];
+                // (|q|^2 + |b|^2) - 2 q.b; a tombstoned column's +inf survives both forms
+                const float s = metric == 0 ? (rn + bnc) - 2.0f * dot : (bnc == inf ? inf : 0.0f - dot);
+                if (r < nq && c < nb) D[(size_t)r * ldD + c] = s;
             }
         }
+    }
 }
 
 // One workgroup per query: the kc candidates (ids, -1 = none; approximate signed distances, ascending) are measured
