@@ -61,9 +61,9 @@ __global__ __launch_bounds__(256) void row_norms_kernel(const float* __restrict_
 }
 
 // D[q][b] ~ signed distance (smaller is closer): |q|^2 + |b|^2 - 2 q.b for L2, -q.b for IP; +inf for tombstoned
-// ids.  grid = (ceil(nb/NT), ceil(nq/MT)), 256 threads = 4 wavefronts in 2 x 2, each 64 x 64 of the tile as 2 x 2
-// MFMA blocks of 32 x 32.  Operands go through LDS dimension-major, so that the 32 lanes of an MFMA operand read
-// consecutive words.
+// ids.  One workgroup per 128 x 128 tile (the mapping of blockIdx to tiles is at the head of the kernel), 256
+// threads = 4 wavefronts in 2 x 2, each 64 x 64 of the tile as 2 x 2 MFMA blocks of 32 x 32.  Operands go through
+// LDS dimension-major, so that the 32 lanes of an MFMA operand read consecutive words.
 #ifndef CORAL_MFMA_WAVES
 #define CORAL_MFMA_WAVES 4
 #endif
@@ -77,8 +77,15 @@ __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel
     __shared__ float sb[2][BK][NT + 4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1;
-    const int64_t b0 = (int64_t)blockIdx.x * NT;
-    const int q0 = blockIdx.y * MT;
+    // Workgroups go to the eight XCDs in turn, each with an L2 of its own: the workgroups that share a tile of
+    // base points (one per tile of queries) are given consecutive places on one XCD, so that the base tile comes
+    // from memory once and from that L2 afterwards.  grid.x = 8 x ceil(base tiles / 8) x query tiles.
+    const int nqt = (nq + MT - 1) / MT;
+    const unsigned xcd = blockIdx.x & 7u, place = blockIdx.x >> 3;
+    const int64_t bt = (int64_t)(place / (unsigned)nqt) * 8 + xcd;
+    const int64_t b0 = bt * NT;
+    const int q0 = (int)(place % (unsigned)nqt) * MT;
+    if (b0 >= nb) return;  // the padding of the last group of eight base tiles
     const int lrow = tid >> 1, lk = (tid & 1) * 4;  // staging: thread t loads row t/2, dimensions (t&1)*4 .. +4
     float4 va[NLD], vb[NLD];
     auto fetch = [&](int k0) {
@@ -284,7 +291,10 @@ hipError_t launch_row_norms(const float* x, int64_t n, int dim, float* out, uint
 hipError_t launch_approx_tile(const float* queries, const float* base, int nq, int64_t nb, int dim, int metric,
                               const float* qn, const float* bn, const uint32_t* deleted, int64_t base_id0, float* D,
                               int64_t ldD, hipStream_t stream) {
-    dim3 grid((unsigned)((nb + NT - 1) / NT), (unsigned)((nq + MT - 1) / MT));
+    const int64_t nbt = (nb + NT - 1) / NT, nqt = (nq + MT - 1) / MT;
+    const int64_t wgs = (nbt + 7) / 8 * 8 * nqt;
+    if (wgs <= 0 || wgs > 0x7fffffff) return hipErrorInvalidValue;
+    dim3 grid((unsigned)wgs);
     hipLaunchKernelGGL(approx_tile_mfma_kernel, grid, dim3(256), 0, stream, queries, base, nq, nb, dim, metric, qn, bn,
                        deleted, base_id0, D, ldD);
     return hipGetLastError();
