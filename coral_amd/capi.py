@@ -41,7 +41,7 @@ class Stats(C.Structure):
 class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
                 ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("best_first_packed", C.c_int32),
-                ("reserved", C.c_int32 * 2)]
+                ("best_first_table_log2", C.c_int32), ("reserved", C.c_int32 * 1)]
 
 
 class BuildParams(C.Structure):
@@ -197,9 +197,9 @@ class Index:
         return m
 
     def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False,
-                best_first_packed=False):
+                best_first_packed=False, best_first_table_log2=0):
         t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)),
-                   int(bool(best_first_packed)))
+                   int(bool(best_first_packed)), best_first_table_log2)
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

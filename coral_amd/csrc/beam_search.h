@@ -46,13 +46,19 @@ struct BestFirstArgs {
     int32_t rows_unique;     // no graph row lists an id twice (checked by launch_find_repeated_ids)
     int32_t packed;          // visited is [slots][stride] of 32-bit words, 8 bits of epoch over 24 node flags each
     int32_t bloom_log2;      // log2 of the bits of the per-wavefront Bloom filter in LDS, 0 = none
+    // first level of the visited set: an exact table of 2^table_log2 16-bit cells per wavefront in LDS (0 = none) in
+    // buckets of four; rem_bits = the bits of the mixed id (id_bits wide) that a cell stores, at most 14; after
+    // table_limit first visits the table takes no more, and what it cannot take goes to the state in HBM
+    int32_t table_log2, table_limit, id_bits, rem_bits;
 };
 
-// LDS bytes of one wavefront: a beam of L keys, 64 candidate keys, 64 ids, L byte counters, and a Bloom filter of
-// 2^bloom_log2 bits over the visited ids (bloom_log2 = 0: none)
-__host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2) {
+// LDS bytes of one wavefront: a beam of L keys, 64 candidate keys, 64 ids, L byte counters, a Bloom filter of
+// 2^bloom_log2 bits over the visited ids in HBM (bloom_log2 = 0: none) and a table of 2^table_log2 16-bit cells
+// (table_log2 = 0: none)
+__host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2, int table_log2 = 0) {
     const size_t bloom = bloom_log2 ? ((size_t)1 << bloom_log2) / 8 : 0;
-    return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + bloom + 15) & ~(size_t)15;
+    const size_t table = table_log2 ? (size_t)2 << table_log2 : 0;
+    return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + bloom + table + 15) & ~(size_t)15;
 }
 // the filter size for a beam of L: 128 bits per beam entry rounded up to a power of two, halved while that would leave
 // a CU fewer than sixteen wavefronts; none below 4096 bits
@@ -62,7 +68,8 @@ __host__ inline int best_first_bloom_log2(int L) {
     while (lg >= 12 && best_first_wave_lds_bytes(L, lg) > (size_t)10 * 1024) --lg;
     return lg >= 12 ? lg : 0;
 }
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int* max_wg_per_cu);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int table_log2,
+                              int* max_wg_per_cu);
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice
 hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream);

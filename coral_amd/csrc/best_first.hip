@@ -7,14 +7,20 @@
 // with the visited set in LDS (the form beam_search.hip gives this policy) holds two queries per CU.  Here a query
 // needs one wavefront and 9.5 KB of LDS at L = 512 (its sorted beam, merged in place, and a filter over its visited
 // ids): sixteen queries per CU, as many as 128 registers per lane allow, enough to keep HBM busy (2.8 times the
-// throughput of the other form at a million nodes; more wavefronts add nothing).  The visited set moves to global memory in the form the CPU path
-// itself uses (src/search_in_cpu.cpp:44-48, 68-71): one byte per node and query slot holding the epoch of the
-// query that last visited the node, so nothing is cleared between queries (every 255th query of a slot wipes its
-// array).  With 288 GB of HBM four thousand such arrays are cheap (4 GB at a million nodes); each test costs a
-// 128-byte line of HBM traffic and each mark a 32-byte write, together about a quarter of what the vectors cost.
-// For indexes too large for a byte per node and slot the same state is packed into 32-bit words of 8 epoch bits
-// over 24 node flags (template parameter PACKED).  A Bloom filter over the query's visited ids in LDS (4 KB at
-// L = 512) answers most tests without that line: an id it does not know is new for certain.
+// throughput of the other form at a million nodes; more wavefronts add nothing).
+//
+// The visited set has two levels.  In global memory, the form the CPU path itself uses (src/search_in_cpu.cpp:44-48,
+// 68-71): one byte per node and query slot holding the epoch of the query that last visited the node, so nothing
+// is cleared between queries (every 255th query of a slot wipes its array).  With 288 GB of HBM four thousand such
+// arrays are cheap (4 GB at a million nodes); each test costs a 128-byte line of HBM traffic and each mark a
+// 32-byte write.  For indexes too large for a byte per node and slot the same state is packed into 32-bit words of
+// 8 epoch bits over 24 node flags (template parameter PACKED).  A Bloom filter over the query's visited ids in LDS
+// (4 KB at L = 512) answers most tests without that line: an id it does not know is new for certain.
+// Those single-line requests cost the memory system more than their bytes say (a launch without them moves its
+// vectors 1.4 times as fast on data whose neighbourhoods overlap), so where the beam leaves room -- L <= 368 -- the
+// first level is an exact table of 16-bit cells in LDS, in buckets of four with two candidate buckets per id: a
+// test is two 8-byte LDS reads whatever the load, and only ids that find both buckets full go to the state in HBM.
+// 8192 cells (16 KB) per query leave a CU eight wavefronts, which this kernel needs anyway to saturate memory.
 //
 // The arithmetic is that of beam_search.hip (same lane-strided accumulation, same butterfly, same 64-bit keys), so
 // results and counters are identical bit for bit; a wavefront needs no workgroup barrier anywhere.
@@ -59,11 +65,12 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
     if (slot >= b.slots) return;  // the whole wavefront; no workgroup barrier is used below
     const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2, M = a.M;
     const int Lp = (L + 3) & ~3;
-    unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L, b.bloom_log2);
+    unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L, b.bloom_log2, b.table_log2);
     uint64_t* beam = reinterpret_cast<uint64_t*>(mine_lds);      // L keys, sorted
     uint64_t* cand = beam + Lp;                                   // kBatch keys
     uint32_t* todo = reinterpret_cast<uint32_t*>(cand + kBatch);  // kBatch ids
-    uint32_t* marks = todo + kBatch;                              // Lp byte counters, zero between merges
+    uint32_t* table = todo + kBatch;                              // 2^table_log2 16-bit cells, or none (8-byte aligned)
+    uint32_t* marks = table + (b.table_log2 ? (1 << b.table_log2) >> 1 : 0);  // Lp byte counters, zero between merges
     uint32_t* bloom = marks + (Lp >> 2);                          // 2^bloom_log2 bits, or none
     for (int i = lane; i < (Lp >> 2); i += 64) marks[i] = 0u;
     // The Bloom filter holds every id the query has visited.  An id it does not know is new for certain and needs no
@@ -85,6 +92,54 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
         bloom_bits(id, h1, h2);
         atomicOr(&bloom[h1 >> 5], 1u << (h1 & 31));
         atomicOr(&bloom[h2 >> 5], 1u << (h2 & 31));
+    };
+
+    // First level of the visited set, when the launch has one: an exact table of 16-bit cells in LDS, in buckets of
+    // four.  A bijection mixes the id; the high bits of the result pick a bucket, a second bucket follows from that
+    // one and the remaining bits (the remainder), and a cell stores the remainder and which of the two buckets it is
+    // in: cell = 1 + ((second << rb) | remainder), 0 = empty.  (bucket, cell) determine the mixed value and hence the
+    // id, so the table is exact.  A test reads the two buckets (two 8-byte reads, whatever the load); an id goes to
+    // the emptier one.  0: the id was there; 1: it is now; 2: it is not and cannot be (the table takes no more
+    // inserts, or both buckets are full): such ids are settled against the state in HBM.
+    // One call handles distinct ids in its lanes (the caller has removed repeats).
+    const int tl = b.table_log2;
+    const uint32_t t_bkmask = tl ? (1u << (tl - 2)) - 1u : 0u;
+    const uint32_t t_bmask = b.id_bits >= 32 ? 0xffffffffu : (1u << b.id_bits) - 1u;
+    const int t_rb = b.rem_bits, t_xs = b.id_bits > 1 ? b.id_bits / 2 : 1;
+    const uint32_t t_rmask = (1u << t_rb) - 1u;
+    auto table_test_and_set = [&](uint32_t id, bool frozen) -> int {
+        uint32_t h = (id * 0x9E3779B1u) & t_bmask;
+        h ^= h >> t_xs;
+        h = (h * 0x85EBCA6Bu) & t_bmask;
+        h ^= h >> t_xs;
+        const uint32_t rem = h & t_rmask;
+        const uint32_t b1 = (h >> t_rb) & t_bkmask;
+        const uint32_t b2 = (b1 ^ (((rem + 1u) * 0x5BD1E995u) >> 15)) & t_bkmask;
+        const uint32_t want1 = 1u + rem, want2 = 1u + ((1u << t_rb) | rem);
+        const uint2* buckets = reinterpret_cast<const uint2*>(table);
+        for (int attempt = 0; attempt < 8; ++attempt) {
+            const uint2 w1 = buckets[b1], w2 = buckets[b2];
+            const uint32_t c1[4] = {w1.x & 0xffffu, w1.x >> 16, w1.y & 0xffffu, w1.y >> 16};
+            const uint32_t c2[4] = {w2.x & 0xffffu, w2.x >> 16, w2.y & 0xffffu, w2.y >> 16};
+            int e1 = 0, e2 = 0, f1 = -1, f2 = -1;  // empty cells and the first of them, per bucket
+            bool present = false;
+#pragma unroll
+            for (int i = 3; i >= 0; --i) {
+                present |= c1[i] == want1 || c2[i] == want2;
+                if (c1[i] == 0u) ++e1, f1 = i;
+                if (c2[i] == 0u) ++e2, f2 = i;
+            }
+            if (present) return 0;
+            if (frozen || (e1 == 0 && e2 == 0)) return 2;
+            const bool second = e2 > e1;
+            const uint32_t bk = second ? b2 : b1, want = second ? want2 : want1;
+            const int cell = second ? f2 : f1;
+            const uint32_t oldw = second ? (cell < 2 ? w2.x : w2.y) : (cell < 2 ? w1.x : w1.y);
+            const int sh = (cell & 1) * 16;
+            if (atomicCAS(table + bk * 2u + (uint32_t)(cell >> 1), oldw, oldw | (want << sh)) == oldw) return 1;
+            // another lane took a cell of that word: look again
+        }
+        return 2;
     };
 
     uint8_t* vis = b.visited + (size_t)slot * b.stride;
@@ -110,6 +165,9 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
         }
         const uint8_t tag = (uint8_t)epoch;
         for (int i = lane; i < bloom_words; i += 64) bloom[i] = 0u;
+        for (int i = lane; i < (tl ? (1 << tl) >> 1 : 0); i += 64) table[i] = 0u;
+        int in_table = 0;         // first visits the table holds
+        bool any_over = tl == 0;  // has an id of this query gone to the state in HBM?
         uint32_t* visw = reinterpret_cast<uint32_t*>(vis);
         // first visit?  (every lane passes its own id; ids of one call are distinct, or told apart by the caller)
         auto unvisited = [&](uint32_t id) -> bool {
@@ -252,12 +310,19 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
         // ---- seeds: every start id is visited and measured (src/search_in_cpu.cpp:74-79)
         for (int s0 = 0; s0 < M; s0 += kBatch) {
             const int T = M - s0 < kBatch ? M - s0 : kBatch;
+            bool over = false;
             if (lane < T) {
                 const uint32_t id = (uint32_t)a.start_ids[s0 + lane];
-                mark(id);
-                if (bl) bloom_add(id);
+                over = tl == 0 || table_test_and_set(id, in_table >= b.table_limit) == 2;
+                if (over) {
+                    mark(id);
+                    if (bl) bloom_add(id);
+                }
                 todo[lane] = id;
             }
+            const int n_over = __popcll(__ballot(over));
+            in_table += T - n_over;
+            any_over = any_over || n_over > 0;
             wave_sync();
             measure_and_merge(T);
         }
@@ -286,20 +351,34 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
 
             int v = -1;
             if (lane < R) v = a.nbrs[(size_t)eid * R + lane];
-            bool isnew = false;
-            if (v >= 0) isnew = (bl && !bloom_may_hold((uint32_t)v)) || unvisited((uint32_t)v);
-            if (!b.rows_unique && __ballot(isnew)) {
+            if (!b.rows_unique) {
                 // an id listed twice in the row counts once (the first listing)
+                const int v0 = v;
                 for (int k = 0; k < R; ++k) {
-                    const int vk = __builtin_amdgcn_readlane(v, k);
-                    if (k < lane && vk == v) isnew = false;
+                    const int vk = __builtin_amdgcn_readlane(v0, k);
+                    if (k < lane && vk == v0) v = -1;
                 }
             }
-            if (isnew) {
+            // the table first; what it has no room for is settled against the state in HBM, which holds nothing
+            // before the first id went there, and whose filter knows every id that did
+            bool isnew = false, over = false;
+            if (v >= 0) {
+                if (tl) {
+                    const int r = table_test_and_set((uint32_t)v, in_table >= b.table_limit);
+                    isnew = r == 1, over = r == 2;
+                } else {
+                    over = true;
+                }
+                if (over) isnew = !any_over || (bl && !bloom_may_hold((uint32_t)v)) || unvisited((uint32_t)v);
+            }
+            if (isnew && over) {
                 mark((uint32_t)v);
                 if (bl) bloom_add((uint32_t)v);
             }
+            const uint64_t m_over = __ballot(isnew && over);
             const uint64_t m = __ballot(isnew);
+            in_table += __popcll(m & ~m_over);
+            any_over = any_over || m_over != 0ull;
             const int T = __popcll(m);
             if (isnew) todo[prefix_popc(m)] = (uint32_t)v;
             nd += T;
@@ -394,10 +473,11 @@ bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed) {
 
 }  // namespace
 
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int* max_wg_per_cu) {
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int table_log2,
+                              int* max_wg_per_cu) {
     bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed);
     if (!fn) return hipErrorInvalidValue;
-    const size_t lds = best_first_wave_lds_bytes(L, bloom_log2) * kWavesPerWg;
+    const size_t lds = best_first_wave_lds_bytes(L, bloom_log2, table_log2) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -412,7 +492,8 @@ hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStr
     bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
-    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_wave_lds_bytes(a.L, b.bloom_log2) * kWavesPerWg, stream, a, b);
+    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64),
+                       best_first_wave_lds_bytes(a.L, b.bloom_log2, b.table_log2) * kWavesPerWg, stream, a, b);
     return hipGetLastError();
 }
 

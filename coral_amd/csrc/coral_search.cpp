@@ -317,9 +317,40 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const int chunks = idx->dim / 4;
         const int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
         idx->bf_rows_in_flight = rif;
-        const int bloom_log2 = coral::best_first_bloom_log2(L);
+        // First level of the visited set: an exact table of 16-bit cells per wavefront in LDS, where one that holds
+        // most of a query's first visits (20 to 30 per beam entry) still leaves a CU eight wavefronts -- what the
+        // HBM-resident state costs in requests is worth more than the wavefronts given up.  Sixteen wavefronts if
+        // 24 cells per entry fit with them, else twelve, else eight with 20 cells per entry; no table for longer
+        // beams, or when the ids are wider than a cell can tell apart (14 bits beyond the bucket index).
+        int table_log2 = 0;
+        auto table_rem_bits = [&](int lg) { return std::max(0, id_bits - (lg - 2)); };
+        if (t.best_first_table_log2 > 0) {
+            if (t.best_first_table_log2 < 8 || t.best_first_table_log2 > 14 ||
+                coral::best_first_wave_lds_bytes(L, 0, t.best_first_table_log2) * 4 > (size_t)kMaxLdsBytes)
+                return fail(CORAL_ERR_ARG, "best_first_table_log2 must be in 8..14 and fit LDS with the beam");
+            if (table_rem_bits(t.best_first_table_log2) > 14)
+                return fail(CORAL_ERR_ARG, "ids of %d bits do not fit the cells of a 2^%d table", id_bits,
+                            t.best_first_table_log2);
+            table_log2 = t.best_first_table_log2;
+        } else if (t.best_first_table_log2 == 0) {
+            const struct { int waves, cells_per_entry; } plans[] = {{16, 24}, {12, 24}, {8, 20}};
+            for (const auto& pl : plans) {
+                for (int lg = 14; lg >= 10 && !table_log2; --lg)
+                    if (coral::best_first_wave_lds_bytes(L, 0, lg) * pl.waves <= (size_t)kMaxLdsBytes &&
+                        (1 << lg) >= pl.cells_per_entry * L && table_rem_bits(lg) <= 14)
+                        table_log2 = lg;
+                if (table_log2) break;
+            }
+        }
+        idx->bf_table_log2 = table_log2;
+        // no limit below the number of cells: a test costs two reads whatever the load, so the table takes ids until
+        // both buckets of one are full, and goes on taking the others
+        idx->bf_table_limit = table_log2 ? 1 << table_log2 : 0;
+        idx->bf_table_rem_bits = table_log2 ? table_rem_bits(table_log2) : 0;
+        // with a table the filter would only cover what outgrew it, and its LDS is worth more as cells
+        const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L);
         idx->bf_bloom_log2 = bloom_log2;
-        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, bloom_log2, &bf_wg_per_cu));
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, bloom_log2, table_log2, &bf_wg_per_cu));
         size_t free_b = 0, total_b = 0;
         HIP_TRY(hipMemGetInfo(&free_b, &total_b));
         const size_t budget = std::min<size_t>((free_b + idx->bf_alloc_bytes) / 3, (size_t)64 << 30);
@@ -332,7 +363,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const size_t stride = packed ? stride_packed : stride_bytes;
         if (packed != idx->bf_packed) idx->bf_stride = 0;  // forces a fresh, zeroed allocation
         idx->bf_packed = packed;
-        if (packed) HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, true, bloom_log2, &bf_wg_per_cu));
+        if (packed) HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, true, bloom_log2, table_log2, &bf_wg_per_cu));
         int slots = (int)std::min<size_t>((size_t)need, budget / stride);
         // below about four wavefronts per CU the workgroup-per-query kernel is the faster one
         if (bf_wg_per_cu > 0 && (slots >= 4 * idx->num_cu || slots >= Q || t.workgroups > 0) && slots > 0) {
@@ -426,6 +457,8 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         b.rows_unique = idx->rows_unique == 1;
         b.packed = idx->bf_packed;
         b.bloom_log2 = idx->bf_bloom_log2;
+        b.table_log2 = idx->bf_table_log2, b.table_limit = idx->bf_table_limit;
+        b.id_bits = idx->id_bits, b.rem_bits = idx->bf_table_rem_bits;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;

@@ -104,7 +104,12 @@ typedef struct {
     int32_t best_first_packed;  /* that visited state is a byte per node while n bytes x query slots fit a third of
                                    the free memory (and 64 GiB), else a 32-bit word per 24 nodes (8 bits of epoch,
                                    24 flags: n / 6 bytes per slot, about 5 % slower); 1 = the packed form always */
-    int32_t reserved[2];
+    int32_t best_first_table_log2; /* the wavefront-per-query kernel keeps the first visits of a query in an exact
+                                   table of 16-bit cells in LDS (the cells of the ROUNDS kernel's table) and only
+                                   what outgrows it in HBM: log2 of the cells per query, 8..14; 0 = chosen from L
+                                   where 8192 cells hold most of a query's visits (L <= 368 at up to 2^25 nodes),
+                                   none otherwise; -1 = none */
+    int32_t reserved[1];
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);

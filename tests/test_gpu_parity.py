@@ -84,9 +84,13 @@ def test_exact_against_same_order_oracle(orc, case):
     idx = capi.Index(base, nbrs, starts, m)
     # best-first has two kernels: a wavefront per query (visited state in HBM, a byte per node or packed words) and a
     # workgroup per query (LDS table)
-    for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
+    # workgroup per query (LDS table); the wavefront form keeps the first visits in an exact table in LDS where the
+    # beam leaves room (chosen by the library, none, or a small one that overflows into the state in HBM)
+    forms = ((False, False, 0), (False, True, 0), (True, False, 0), (False, False, -1), (False, True, 8),
+             (False, False, 9)) if policy == 1 else ((False, False, 0),)
+    for in_lds, packed, table in forms:
         idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy,
-                    best_first_in_lds=in_lds, best_first_packed=packed)
+                    best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=table)
         ids, dists, st = idx.search(q, k, L, policy=policy)
         cnt = idx.query_counters(q.shape[0])
         assert np.array_equal(ids, oi)
@@ -119,8 +123,9 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         rg = int(rng.randint(1, 1000)) if rng.rand() < 0.4 else None
         dele, dup = rng.rand() < 0.35, rng.rand() < 0.3
         wgs = int(rng.choice([0, 0, 1, 2, 7]))
+        tbl = int(rng.choice([0, 0, -1, 8, 9, 10, 12]))
         print("case", dict(c=c, n=n, dim=dim, R=R, metric=metric, policy=policy, L=L, k=k, M=M, Q=Q, slots=slots,
-                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs), flush=True)
+                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl), flush=True)
         m = capi.IP if metric == "ip" else capi.L2
         base = synth.gaussian_matrix(1000 + c, n, dim)
         if metric == "ip":
@@ -145,7 +150,7 @@ def test_randomised_search_problems_equal_the_oracle(orc):
             idx.set_deleted(mask)
         for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
             idx.prepare(Q, L, visited_slots_log2=slots, threads=threads, workgroups=wgs, policy=policy,
-                        best_first_in_lds=in_lds, best_first_packed=packed)
+                        best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=tbl)
             ids, dists, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
             assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
             assert np.array_equal(idx.query_counters(Q), os_)
@@ -189,10 +194,11 @@ def test_best_first_query_slots_are_reused(orc):
     oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
     idx = capi.Index(base, nbrs, starts)
     idx.set_deleted(mask)
-    for packed in (False, True):
-        idx.prepare(q.shape[0], L, workgroups=2, policy=1, best_first_packed=packed)
+    # without the table in LDS every visit goes through the state in HBM; with a table of 256 cells most do
+    for packed, table in ((False, -1), (True, -1), (False, 8), (True, 8)):
+        idx.prepare(q.shape[0], L, workgroups=2, policy=1, best_first_packed=packed, best_first_table_log2=table)
         for rep in range(2):
-            print("slot reuse pass", rep, "packed" if packed else "bytes", flush=True)
+            print("slot reuse pass", rep, "packed" if packed else "bytes", "table", table, flush=True)
             ids, dists, st = idx.search(q, k, L, policy=1, have_delete=True)
             cnt = idx.query_counters(q.shape[0])
             assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(cnt, os_)
