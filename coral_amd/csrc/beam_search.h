@@ -52,13 +52,13 @@ struct BestFirstArgs {
     int32_t table_log2, table_limit, id_bits, rem_bits;
 };
 
-// LDS bytes of one wavefront: a beam of L keys, 64 candidate keys, 64 ids, L byte counters, a Bloom filter of
+// LDS bytes of one wavefront: a beam of L keys, 32 candidate keys, 32 ids, L byte counters, a Bloom filter of
 // 2^bloom_log2 bits over the visited ids in HBM (bloom_log2 = 0: none) and a table of 2^table_log2 16-bit cells
 // (table_log2 = 0: none)
 __host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2, int table_log2 = 0) {
     const size_t bloom = bloom_log2 ? ((size_t)1 << bloom_log2) / 8 : 0;
     const size_t table = table_log2 ? (size_t)2 << table_log2 : 0;
-    return ((size_t)((L + 3) & ~3) * 9 + 64 * 8 + 64 * 4 + bloom + table + 15) & ~(size_t)15;
+    return ((size_t)((L + 3) & ~3) * 9 + 32 * 8 + 32 * 4 + bloom + table + 15) & ~(size_t)15;
 }
 // the filter size for a beam of L: 128 bits per beam entry rounded up to a power of two, halved while that would leave
 // a CU fewer than sixteen wavefronts; none below 4096 bits

@@ -5,7 +5,7 @@
 // measure the new ones, insert them, pick the closest entry not yet expanded.  Every step is a chain of dependent
 // memory accesses; what makes it fast on this GPU is how many such chains run side by side.  A workgroup per query
 // with the visited set in LDS (the form beam_search.hip gives this policy) holds two queries per CU.  Here a query
-// needs one wavefront and 9.5 KB of LDS at L = 512 (its sorted beam, merged in place, and a filter over its visited
+// needs one wavefront and 9.1 KB of LDS at L = 512 (its sorted beam, merged in place, and a filter over its visited
 // ids): sixteen queries per CU, as many as 128 registers per lane allow, enough to keep HBM busy (2.8 times the
 // throughput of the other form at a million nodes; more wavefronts add nothing).
 //
@@ -17,7 +17,7 @@
 // 8 epoch bits over 24 node flags (template parameter PACKED).  A Bloom filter over the query's visited ids in LDS
 // (4 KB at L = 512) answers most tests without that line: an id it does not know is new for certain.
 // Those single-line requests cost the memory system more than their bytes say (a launch without them moves its
-// vectors 1.4 times as fast on data whose neighbourhoods overlap), so where the beam leaves room -- L <= 368 -- the
+// vectors 1.4 times as fast on data whose neighbourhoods overlap), so where the beam leaves room -- L <= 409 -- the
 // first level is an exact table of 16-bit cells in LDS, in buckets of four with two candidate buckets per id: a
 // test is two 8-byte LDS reads whatever the load, and only ids that find both buckets full go to the state in HBM.
 // 8192 cells (16 KB) per query leave a CU eight wavefronts, which this kernel needs anyway to saturate memory.
@@ -35,7 +35,7 @@ namespace coral {
 namespace {
 
 constexpr int kWavesPerWg = 4;
-constexpr int kBatch = 64;  // ids measured and merged at a time (a graph row has at most 32)
+constexpr int kBatch = 32;  // ids measured and merged at a time (a graph row has at most 32)
 
 __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

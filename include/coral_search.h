@@ -107,7 +107,7 @@ typedef struct {
     int32_t best_first_table_log2; /* the wavefront-per-query kernel keeps the first visits of a query in an exact
                                    table of 16-bit cells in LDS (the cells of the ROUNDS kernel's table) and only
                                    what outgrows it in HBM: log2 of the cells per query, 8..14; 0 = chosen from L
-                                   where 8192 cells hold most of a query's visits (L <= 368 at up to 2^25 nodes),
+                                   where 8192 cells hold most of a query's visits (L <= 409 at up to 2^25 nodes),
                                    none otherwise; -1 = none */
     int32_t reserved[1];
 } coral_tuning;
