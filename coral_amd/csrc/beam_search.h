@@ -42,7 +42,7 @@ struct BestFirstArgs {
     uint32_t* epochs;   // [slots]: last epoch used by the slot (kept across launches)
     size_t stride;      // bytes per slot, a multiple of 16: n, or 4 * ceil(n / 24) when packed
     int32_t slots;      // wavefronts = queries in flight
-    int32_t rows_in_flight;  // 8 or 16: float4 registers of vector data a lane requests before it adds them up
+    int32_t rows_in_flight;  // 8, 16 or 32: float4 registers of vector data a lane requests before it adds them up
     int32_t rows_unique;     // no graph row lists an id twice (checked by launch_find_repeated_ids)
     int32_t packed;          // visited is [slots][stride] of 32-bit words, 8 bits of epoch over 24 node flags each
     int32_t bloom_log2;      // log2 of the bits of the per-wavefront Bloom filter in LDS, 0 = none

@@ -58,7 +58,7 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
 // PACKED: the visited state of a slot is one 32-bit word per 24 nodes (8 bits of epoch, 24 flags) instead of one
 // byte per node: a sixth of the memory, the same one line per test.
 template <int G, int CPL, int RIF, bool PACKED>
-__global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
+__global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = blockIdx.x * kWavesPerWg + wave;
@@ -249,22 +249,28 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                     acc[u] = acc[u] + dpp_mov<0x141>(acc[u]);  // row_half_mirror
                     acc[u] = acc[u] + dpp_mov<0x140>(acc[u]);  // row_mirror
                 }
-                float mine = acc[0];
-                int myid = vid[0];
+                // lane l of a group takes the sum of row l: the levels across the 16-lane rows add lanes 16 and 32
+                // apart, which have chosen the same row as long as at most 16 rows are dealt out at a time
+                constexpr int UH = U > 16 ? 16 : U;
 #pragma unroll
-                for (int u = 1; u < U; ++u)
-                    if ((lane & (U - 1)) == u) mine = acc[u], myid = vid[u];
-                if (G >= 32) mine = mine + __shfl_xor(mine, 16, 64);
-                if (G >= 64) mine = mine + __shfl_xor(mine, 32, 64);
-                const bool valid = gl < U && myid >= 0;
-                const float s = a.metric == 0 ? mine : 0.0f - mine;
-                const uint64_t key = make_key(s, myid, 0u);
-                // the queue turns away what is not better than its worst entry once it is full
-                // (include/efanna2e/neighbor.h:162-166)
-                const bool app = valid && s < 3.402823466e+38f && key < live;
-                const uint64_t m = __ballot(app);
-                if (app) cand[nc + prefix_popc(m)] = key;
-                nc += __popcll(m);
+                for (int h = 0; h < U; h += UH) {
+                    float mine = acc[h];
+                    int myid = vid[h];
+#pragma unroll
+                    for (int u = 1; u < UH; ++u)
+                        if ((lane & (UH - 1)) == u) mine = acc[h + u], myid = vid[h + u];
+                    if (G >= 32) mine = mine + __shfl_xor(mine, 16, 64);
+                    if (G >= 64) mine = mine + __shfl_xor(mine, 32, 64);
+                    const bool valid = gl < UH && myid >= 0;
+                    const float s = a.metric == 0 ? mine : 0.0f - mine;
+                    const uint64_t key = make_key(s, myid, 0u);
+                    // the queue turns away what is not better than its worst entry once it is full
+                    // (include/efanna2e/neighbor.h:162-166)
+                    const bool app = valid && s < 3.402823466e+38f && key < live;
+                    const uint64_t m = __ballot(app);
+                    if (app) cand[nc + prefix_popc(m)] = key;
+                    nc += __popcll(m);
+                }
             }
             wave_sync();
             if (nc == 0) return;
@@ -454,7 +460,8 @@ __global__ __launch_bounds__(256) void find_repeated_ids_kernel(const int32_t* _
 using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 
 // RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
-// dependent memory waits of a step against 8 and needs 128 registers
+// dependent memory waits of a step against 8 and needs 128 registers; 32 (a whole step at once, 212 registers) is
+// for launches whose LDS holds a CU to eight wavefronts anyway (+2..3 %)
 template <int RIF, bool PACKED>
 bf_kernel_fn pick_bf_kernel_rif(int chunks) {
     if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED>;
@@ -467,6 +474,9 @@ bf_kernel_fn pick_bf_kernel_rif(int chunks) {
 }
 
 bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed) {
+    // 32: for launches that hold eight wavefronts per CU or fewer (256 registers per lane); rows of 17..64 chunks
+    if (rif >= 32 && dim / 4 > 16 && dim / 4 <= 64)
+        return packed ? pick_bf_kernel_rif<32, true>(dim / 4) : pick_bf_kernel_rif<32, false>(dim / 4);
     if (packed) return rif >= 16 ? pick_bf_kernel_rif<16, true>(dim / 4) : pick_bf_kernel_rif<8, true>(dim / 4);
     return rif >= 16 ? pick_bf_kernel_rif<16, false>(dim / 4) : pick_bf_kernel_rif<8, false>(dim / 4);
 }

@@ -315,8 +315,6 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         int bf_wg_per_cu = 0;
         // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling
         const int chunks = idx->dim / 4;
-        const int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
-        idx->bf_rows_in_flight = rif;
         // First level of the visited set: an exact table of 16-bit cells per wavefront in LDS, where one that holds
         // most of a query's first visits (20 to 30 per beam entry) still leaves a CU eight wavefronts -- what the
         // HBM-resident state costs in requests is worth more than the wavefronts given up.  Sixteen wavefronts if
@@ -347,6 +345,13 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         // both buckets of one are full, and goes on taking the others
         idx->bf_table_limit = table_log2 ? 1 << table_log2 : 0;
         idx->bf_table_rem_bits = table_log2 ? table_rem_bits(table_log2) : 0;
+        // a launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a
+        // step requested before any is added up
+        int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
+        if (table_log2 && coral::best_first_wave_lds_bytes(L, 0, table_log2) * 12 > (size_t)kMaxLdsBytes && chunks > 16 &&
+            chunks <= 64)
+            rif = 32;
+        idx->bf_rows_in_flight = rif;
         // with a table the filter would only cover what outgrew it, and its LDS is worth more as cells
         const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L);
         idx->bf_bloom_log2 = bloom_log2;
