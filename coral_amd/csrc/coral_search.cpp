@@ -40,6 +40,35 @@ using coral::fail;
 constexpr int kMaxL = 2048;
 constexpr int kMaxLdsBytes = 160 * 1024;
 
+// bits of a mixed id that a cell of the wavefront kernel's table stores: what the bucket index (a quarter of the
+// cells) does not imply; a cell has room for 14
+int bf_table_rem_bits(int id_bits, int table_log2) { return std::max(0, id_bits - (table_log2 - 2)); }
+
+// First level of the visited set of the wavefront-per-query best-first kernel: an exact table of 16-bit cells per
+// wavefront in LDS, where one that holds most of a query's first visits (20 to 30 per beam entry) still leaves a CU
+// eight wavefronts -- what the HBM-resident state costs in requests is worth more than the wavefronts given up.
+// Sixteen wavefronts if 24 cells per entry fit with them, else twelve, else eight with 20 cells per entry; no table
+// (0) for longer beams, or when the ids are wider than a cell can tell apart.  wanted: the caller's
+// coral_tuning.best_first_table_log2.
+int choose_bf_table(int L, int id_bits, int wanted, int* table_log2) {
+    *table_log2 = 0;
+    if (wanted > 0) {
+        if (wanted < 8 || wanted > 14 || coral::best_first_wave_lds_bytes(L, 0, wanted) * 4 > (size_t)kMaxLdsBytes)
+            return fail(CORAL_ERR_ARG, "best_first_table_log2 must be in 8..14 and fit LDS with the beam");
+        if (bf_table_rem_bits(id_bits, wanted) > 14)
+            return fail(CORAL_ERR_ARG, "ids of %d bits do not fit the cells of a 2^%d table", id_bits, wanted);
+        *table_log2 = wanted;
+    } else if (wanted == 0) {
+        const struct { int waves, cells_per_entry; } plans[] = {{16, 24}, {12, 24}, {8, 20}};
+        for (const auto& pl : plans)
+            for (int lg = 14; lg >= 10 && !*table_log2; --lg)
+                if (coral::best_first_wave_lds_bytes(L, 0, lg) * pl.waves <= (size_t)kMaxLdsBytes &&
+                    (1 << lg) >= pl.cells_per_entry * L && bf_table_rem_bits(id_bits, lg) <= 14)
+                    *table_log2 = lg;
+    }
+    return CORAL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -288,6 +317,9 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     int workgroups = t.workgroups > 0 ? t.workgroups : wg_per_cu * idx->num_cu;
     workgroups = std::min(workgroups, (int)Q);
 
+    int table_log2 = 0;  // of the wavefront-per-query best-first kernel
+    if (best_first && !t.best_first_in_lds)
+        if (int rc = choose_bf_table(L, id_bits, t.best_first_table_log2, &table_log2)) return rc;
     // from here on buffers are replaced: a failure part-way leaves the index unprepared, not half-prepared
     idx->prepared = false;
     const size_t spill_words = ((size_t)idx->n + 31) / 32;
@@ -313,40 +345,14 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     idx->bf_ready = false;
     if (best_first && !t.best_first_in_lds) {
         int bf_wg_per_cu = 0;
-        // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling
         const int chunks = idx->dim / 4;
-        // First level of the visited set: an exact table of 16-bit cells per wavefront in LDS, where one that holds
-        // most of a query's first visits (20 to 30 per beam entry) still leaves a CU eight wavefronts -- what the
-        // HBM-resident state costs in requests is worth more than the wavefronts given up.  Sixteen wavefronts if
-        // 24 cells per entry fit with them, else twelve, else eight with 20 cells per entry; no table for longer
-        // beams, or when the ids are wider than a cell can tell apart (14 bits beyond the bucket index).
-        int table_log2 = 0;
-        auto table_rem_bits = [&](int lg) { return std::max(0, id_bits - (lg - 2)); };
-        if (t.best_first_table_log2 > 0) {
-            if (t.best_first_table_log2 < 8 || t.best_first_table_log2 > 14 ||
-                coral::best_first_wave_lds_bytes(L, 0, t.best_first_table_log2) * 4 > (size_t)kMaxLdsBytes)
-                return fail(CORAL_ERR_ARG, "best_first_table_log2 must be in 8..14 and fit LDS with the beam");
-            if (table_rem_bits(t.best_first_table_log2) > 14)
-                return fail(CORAL_ERR_ARG, "ids of %d bits do not fit the cells of a 2^%d table", id_bits,
-                            t.best_first_table_log2);
-            table_log2 = t.best_first_table_log2;
-        } else if (t.best_first_table_log2 == 0) {
-            const struct { int waves, cells_per_entry; } plans[] = {{16, 24}, {12, 24}, {8, 20}};
-            for (const auto& pl : plans) {
-                for (int lg = 14; lg >= 10 && !table_log2; --lg)
-                    if (coral::best_first_wave_lds_bytes(L, 0, lg) * pl.waves <= (size_t)kMaxLdsBytes &&
-                        (1 << lg) >= pl.cells_per_entry * L && table_rem_bits(lg) <= 14)
-                        table_log2 = lg;
-                if (table_log2) break;
-            }
-        }
         idx->bf_table_log2 = table_log2;
         // no limit below the number of cells: a test costs two reads whatever the load, so the table takes ids until
         // both buckets of one are full, and goes on taking the others
         idx->bf_table_limit = table_log2 ? 1 << table_log2 : 0;
-        idx->bf_table_rem_bits = table_log2 ? table_rem_bits(table_log2) : 0;
-        // a launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a
-        // step requested before any is added up
+        idx->bf_table_rem_bits = table_log2 ? bf_table_rem_bits(id_bits, table_log2) : 0;
+        // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling; a
+        // launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a step
         int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
         if (table_log2 && coral::best_first_wave_lds_bytes(L, 0, table_log2) * 12 > (size_t)kMaxLdsBytes && chunks > 16 &&
             chunks <= 64)
