@@ -47,9 +47,9 @@ struct BestFirstArgs {
     int32_t packed;          // visited is [slots][stride] of 32-bit words, 8 bits of epoch over 24 node flags each
     int32_t bloom_log2;      // log2 of the bits of the per-wavefront Bloom filter in LDS, 0 = none
     // first level of the visited set: an exact table of 2^table_log2 16-bit cells per wavefront in LDS (0 = none) in
-    // buckets of four; rem_bits = the bits of the mixed id (id_bits wide) that a cell stores, at most 14; after
-    // table_limit first visits the table takes no more, and what it cannot take goes to the state in HBM
-    int32_t table_log2, table_limit, id_bits, rem_bits;
+    // buckets of four; rem_bits = the bits of the mixed id (id_bits wide) that a cell stores, at most 14; what
+    // finds its two buckets full goes to the state in HBM
+    int32_t table_log2, id_bits, rem_bits;
 };
 
 // LDS bytes of one wavefront: a beam of L keys, 32 candidate keys, 32 ids, L byte counters, a Bloom filter of

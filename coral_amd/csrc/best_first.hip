@@ -99,15 +99,15 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
     // one and the remaining bits (the remainder), and a cell stores the remainder and which of the two buckets it is
     // in: cell = 1 + ((second << rb) | remainder), 0 = empty.  (bucket, cell) determine the mixed value and hence the
     // id, so the table is exact.  A test reads the two buckets (two 8-byte reads, whatever the load); an id goes to
-    // the emptier one.  0: the id was there; 1: it is now; 2: it is not and cannot be (the table takes no more
-    // inserts, or both buckets are full): such ids are settled against the state in HBM.
+    // the emptier one.  0: the id was there; 1: it is now; 2: it is not and cannot be (both buckets are full): such
+    // ids are settled against the state in HBM.
     // One call handles distinct ids in its lanes (the caller has removed repeats).
     const int tl = b.table_log2;
     const uint32_t t_bkmask = tl ? (1u << (tl - 2)) - 1u : 0u;
     const uint32_t t_bmask = b.id_bits >= 32 ? 0xffffffffu : (1u << b.id_bits) - 1u;
     const int t_rb = b.rem_bits, t_xs = b.id_bits > 1 ? b.id_bits / 2 : 1;
     const uint32_t t_rmask = (1u << t_rb) - 1u;
-    auto table_test_and_set = [&](uint32_t id, bool frozen) -> int {
+    auto table_test_and_set = [&](uint32_t id) -> int {
         uint32_t h = (id * 0x9E3779B1u) & t_bmask;
         h ^= h >> t_xs;
         h = (h * 0x85EBCA6Bu) & t_bmask;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 if (c2[i] == 0u) ++e2, f2 = i;
             }
             if (present) return 0;
-            if (frozen || (e1 == 0 && e2 == 0)) return 2;
+            if (e1 == 0 && e2 == 0) return 2;
             const bool second = e2 > e1;
             const uint32_t bk = second ? b2 : b1, want = second ? want2 : want1;
             const int cell = second ? f2 : f1;
@@ -166,7 +166,6 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
         const uint8_t tag = (uint8_t)epoch;
         for (int i = lane; i < bloom_words; i += 64) bloom[i] = 0u;
         for (int i = lane; i < (tl ? (1 << tl) >> 1 : 0); i += 64) table[i] = 0u;
-        int in_table = 0;         // first visits the table holds
         bool any_over = tl == 0;  // has an id of this query gone to the state in HBM?
         uint32_t* visw = reinterpret_cast<uint32_t*>(vis);
         // first visit?  (every lane passes its own id; ids of one call are distinct, or told apart by the caller)
@@ -319,16 +318,14 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             bool over = false;
             if (lane < T) {
                 const uint32_t id = (uint32_t)a.start_ids[s0 + lane];
-                over = tl == 0 || table_test_and_set(id, in_table >= b.table_limit) == 2;
+                over = tl == 0 || table_test_and_set(id) == 2;
                 if (over) {
                     mark(id);
                     if (bl) bloom_add(id);
                 }
                 todo[lane] = id;
             }
-            const int n_over = __popcll(__ballot(over));
-            in_table += T - n_over;
-            any_over = any_over || n_over > 0;
+            any_over = any_over || __ballot(over) != 0ull;
             wave_sync();
             measure_and_merge(T);
         }
@@ -370,7 +367,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             bool isnew = false, over = false;
             if (v >= 0) {
                 if (tl) {
-                    const int r = table_test_and_set((uint32_t)v, in_table >= b.table_limit);
+                    const int r = table_test_and_set((uint32_t)v);
                     isnew = r == 1, over = r == 2;
                 } else {
                     over = true;
@@ -381,10 +378,8 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 mark((uint32_t)v);
                 if (bl) bloom_add((uint32_t)v);
             }
-            const uint64_t m_over = __ballot(isnew && over);
             const uint64_t m = __ballot(isnew);
-            in_table += __popcll(m & ~m_over);
-            any_over = any_over || m_over != 0ull;
+            any_over = any_over || __ballot(isnew && over) != 0ull;
             const int T = __popcll(m);
             if (isnew) todo[prefix_popc(m)] = (uint32_t)v;
             nd += T;

@@ -347,9 +347,6 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         int bf_wg_per_cu = 0;
         const int chunks = idx->dim / 4;
         idx->bf_table_log2 = table_log2;
-        // no limit below the number of cells: a test costs two reads whatever the load, so the table takes ids until
-        // both buckets of one are full, and goes on taking the others
-        idx->bf_table_limit = table_log2 ? 1 << table_log2 : 0;
         idx->bf_table_rem_bits = table_log2 ? bf_table_rem_bits(id_bits, table_log2) : 0;
         // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling; a
         // launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a step
@@ -468,7 +465,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         b.rows_unique = idx->rows_unique == 1;
         b.packed = idx->bf_packed;
         b.bloom_log2 = idx->bf_bloom_log2;
-        b.table_log2 = idx->bf_table_log2, b.table_limit = idx->bf_table_limit;
+        b.table_log2 = idx->bf_table_log2;
         b.id_bits = idx->id_bits, b.rem_bits = idx->bf_table_rem_bits;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);

@@ -64,7 +64,7 @@ struct coral_index {
     uint32_t* d_bf_epochs = nullptr;
     size_t bf_stride = 0, bf_alloc_bytes = 0;
     int bf_slots = 0, bf_alloc_slots = 0, bf_rows_in_flight = 8, bf_packed = 0, bf_bloom_log2 = 0;
-    int bf_table_log2 = 0, bf_table_limit = 0, bf_table_rem_bits = 0;
+    int bf_table_log2 = 0, bf_table_rem_bits = 0;
     int rows_unique = -1;  // 1: no graph row lists an id twice, 0: some do, -1: not looked at since the rows changed
     // the tuning of the last prepare, and what the searches since have taught about the visited table:
     // at beam capacity bump_L the library's own choice of table size is raised by bump_log2
