@@ -249,12 +249,19 @@ def cpu_baseline(w, gt, L, k):
     probe = min(256, q.shape[0])
     _, _, _, t = fn(prob, q[:probe], k, L, nthreads=threads)
     n = int(min(q.shape[0], max(probe, 20.0 / max(t / probe, 1e-9))))
-    ids, _, stats, t = fn(prob, q[:n], k, L, nthreads=threads)
+    # a sample that short of 10 s is timed again (at most 9 passes in all) and the median pass is
+    # quoted: a single pass of under a second on a shared host varies by a third from run to run
+    times = []
+    while not times or (sum(times) < 10.0 and len(times) < 9):
+        ids, _, stats, t = fn(prob, q[:n], k, L, nthreads=threads)
+        times.append(t)
+    t = sorted(times)[len(times) // 2]
     hits = oracle.recall_hits(ids, gt[:n], k)
     return {"value": n / t, "unit": "queries/s", "cores": threads, "kind": "reference" if use_ref else "port",
-            "sample": "first %d of %d queries, L=%d, k=%d, M=%d start ids, policy best-first" %
-                      (n, q.shape[0], L, k, w["starts"].size),
-            "recall": hits / float(n * k), "time_s": t, "dist_evals_per_query": float(stats[:, 2].mean()),
+            "sample": "first %d of %d queries, L=%d, k=%d, M=%d start ids, policy best-first; median of %d passes" %
+                      (n, q.shape[0], L, k, w["starts"].size, len(times)),
+            "recall": hits / float(n * k), "time_s": t, "passes_s": [round(x, 4) for x in times],
+            "dist_evals_per_query": float(stats[:, 2].mean()),
             "expansions_per_query": float(stats[:, 1].mean())}
 
 
