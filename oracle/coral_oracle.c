@@ -36,8 +36,11 @@
  *     be built or run here).  Pinned by code reading plus invariants: result ==
  *     top-k of top-L(visited) under (distance,id); every beam entry expanded at
  *     exit; equality with exact kNN on complete graphs and when L >= N;
- *     hand-computed traversals on path/ring graphs; an independent
- *     set-based pure-Python simulator on tiny inputs.
+ *     hand-computed traversals on path/ring graphs, one of them with every
+ *     counter worked out by hand so that each rule of the policy (threshold
+ *     kept when an append fills the beam exactly, frozen inside a round,
+ *     strict comparison, start ids not counted) decides the hop count; an
+ *     independent set-based pure-Python simulator on tiny inputs.
  *   - oracle_bruteforce*: fp64 closed form, exact lattice cases with ties, top-k of a full sort.
  *   - oracle_fps, oracle_nap_batch, oracle_enhance_batch, oracle_enhance_top_batch: no executable reference (CUDA, faiss, outcomes that
  *     depend on thread timing).  Pinned by code reading, hand-computed cases, the invariants of the occlusion

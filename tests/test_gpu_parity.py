@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 
 from coral_amd import capi, formats, synth
-from util import make_queries, near_tie_equal, ragged
+from util import make_queries, near_tie_equal, ragged, rounds_hand_case
 
 pytestmark = pytest.mark.gpu
 
@@ -99,6 +99,28 @@ def test_exact_against_same_order_oracle(orc, case):
         assert st.hops == int(os_[:, 0].sum()) and st.dist_evals == int(os_[:, 2].sum())
         if slots == 11 and (policy == 0 or in_lds):
             assert st.spills > 0
+    idx.close()
+
+
+def test_hand_computed_traversals_through_the_c_abi():
+    """The traversal worked out by hand in util.rounds_hand_case, with no oracle in between: ids, distances and all
+    four counters of the rounds policy (each rule of the policy decides one of them), and the best-first answer on
+    the same points, in every kernel form."""
+    base, nbrs, starts, q, L, k, want = rounds_hand_case()
+    idx = capi.Index(base, nbrs, starts, capi.L2)
+    for threads in (0, 128, 1024):
+        idx.prepare(1, L, threads=threads, policy=0)
+        ids, dists, st = idx.search(q, k, L, policy=0)
+        assert ids[0].tolist() == want["ids"] and dists[0].tolist() == want["dists"]
+        assert idx.query_counters(1)[0].tolist() == [want["hops"], want["expansions"], want["dist_evals"],
+                                                      want["rounds"]]
+        assert (st.hops, st.expansions, st.dist_evals) == (want["hops"], want["expansions"], want["dist_evals"])
+    for in_lds, packed, table in ((False, False, 0), (False, True, 0), (True, False, 0), (False, False, -1),
+                                  (False, False, 8)):
+        idx.prepare(1, L, policy=1, best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=table)
+        ids, dists, st = idx.search(q, k, L, policy=1)
+        assert ids[0].tolist() == [10, 5, 6] and dists[0].tolist() == [1.0, 36.0, 56.25]
+        assert idx.query_counters(1)[0, :3].tolist() == [1 + 5, 5, 7]
     idx.close()
 
 

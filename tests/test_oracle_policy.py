@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 
 import pysim
-from util import digest, make_problem, make_queries, ragged
+from util import digest, make_problem, make_queries, ragged, rounds_hand_case
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
@@ -40,6 +40,15 @@ def test_policy_a_equals_reference_harness(orc, ref, L, k, M):
     assert np.array_equal(a[0], b[0])
     assert a[1].tobytes() == b[1].tobytes()
     assert np.array_equal(a[2], b[2])
+
+
+def test_best_first_hand_case_on_the_reference_queue(orc, ref):
+    """The hand-worked line of util.rounds_hand_case under the reference's own queue and distance: the answer
+    that differs from the rounds policy's (6 instead of 4) is the reference's, not a slip of the restatement."""
+    base, nbrs, starts, q, L, k, _ = rounds_hand_case()
+    ids, dists, stats, _ = orc.ref_search_in_cpu(orc.Problem(base, nbrs, starts), q, k, L)
+    assert ids[0].tolist() == [10, 5, 6] and dists[0].tolist() == [1.0, 36.0, 56.25]
+    assert stats[0, :3].tolist() == [1 + 5, 5, 7]
 
 
 def golden_cases():
@@ -169,6 +178,27 @@ def test_ring_graph_hand_computed(orc):
     # queue holds no unexpanded entry.  0->9,1; 9->8; 8->7; 7->6; 6->5; 5->4(rejected): 6 expansions
     assert stats[0, 1] == 6 and stats[0, 0] == 1 + 6
     assert stats[0, 2] == 8  # 0,9,1,8,7,6,5,4
+
+
+def test_rounds_policy_hand_computed_counters(orc):
+    """Every counter of a traversal worked out by hand (util.rounds_hand_case): the threshold that is not tightened
+    when an append fills the beam exactly, the threshold frozen inside a round, the strict comparison, the start id
+    that is not a hop -- each of them changes `hops` if it is restated wrongly."""
+    base, nbrs, starts, q, L, k, want = rounds_hand_case()
+    prob = orc.Problem(base, nbrs, starts)
+    for order in (0, 1, 2, 3):
+        ids, dists, stats, _ = orc.search_B(prob, q, k, L, start_order=order, nbr_order=order)
+        assert ids[0].tolist() == want["ids"] and dists[0].tolist() == want["dists"]
+        assert stats[0].tolist() == [want["hops"], want["expansions"], want["dist_evals"], want["rounds"]]
+    dist = {i: float(x) ** 2 for i, x in enumerate(base[:, 2])}
+    sim = pysim.policy_rounds(nbrs.tolist(), starts.tolist(), dist, L, k)
+    assert sim == (want["ids"], want["hops"], want["expansions"], want["dist_evals"])
+    # the same points under best-first: 0 -> 1, 2; 2 -> 5 (0 leaves the queue); 5 -> 6, 7 (1 and 2 leave);
+    # 6 -> 10 (7 leaves, unexpanded); 10 -> nothing new.  Five expansions, seven distances, and a different
+    # answer: 4 is never reached, because 1, the only way to it, was dropped unexpanded.
+    ids, dists, stats, _ = orc.search_A(prob, q, k, L, order=0)
+    assert ids[0].tolist() == [10, 5, 6] and dists[0].tolist() == [1.0, 36.0, 56.25]
+    assert stats[0, :3].tolist() == [1 + 5, 5, 7]
 
 
 @pytest.mark.parametrize("policy", ["A", "B"])

@@ -63,3 +63,35 @@ def near_tie_equal(ids_a, d_a, ids_b, d_b, rel=1e-6):
                 if abs(other_d[k - 1] - mine_d) > rel * max(abs(mine_d), 1e-30) * 4:
                     return False
     return len(sa ^ sb) <= 2 * k
+
+
+def rounds_hand_case():
+    """A traversal of the expand-all-rounds policy (src/search_gpu.cu:412-483, 525-576) worked out by hand.
+
+    Eleven points on a line (distance to the query at the origin = x squared, exact in fp32 in any summation order),
+    L = 3, one start id.  Every rule that sets this policy apart from a best-first search decides a counter:
+
+      round 1  expands 0 (100): 1 (81) and 2 (64) pass the initial threshold; beam {0, 1, 2} is exactly full by
+               APPENDING, so the threshold stays at the sentinel (:477-483).
+      round 2  expands 1 and 2: 3 (400), 4 (49), 5 (36).  3 is farther than everything in the beam and still
+               counts as a candidate because the threshold was not tightened.  Overflow: beam {5, 4, 2}, threshold 64.
+      round 3  expands 5 then 4: 6 (56.25) passes; 7 (60.0625) passes although it no longer fits beside 6, because
+               the threshold is frozen for the round (:412-439); 7 is listed by 4 as well and is measured once;
+               8 (72.25) fails; 9 (64) fails: the comparison is strict.  Beam {5, 4, 6}, threshold 56.25.
+      round 4  expands 6: 10 (1) passes.  Beam {10, 5, 4}, threshold 49.
+      round 5  expands 10: its only neighbour, 0, is visited; no candidate, the search ends.
+
+    hops = candidates = 2 + 3 + 2 + 1 = 8 (start ids are not counted), expansions = 1 + 2 + 2 + 1 + 1 = 7,
+    distance evaluations = 1 + 2 + 3 + 4 + 1 = 11, rounds = 5.  With the threshold tightened on the exact fit, or
+    moved inside a round, hops is 7; with a non-strict comparison, or the start counted, 9.
+    """
+    xs = [10, 9, 8, 20, 7, 6, 7.5, 7.75, 8.5, 8, 1]
+    base = np.zeros((len(xs), 4), np.float32)
+    base[:, 2] = xs
+    rows = {0: [1, 2], 1: [3, 4], 2: [5], 4: [7, 8, 9], 5: [6, 7], 6: [10], 10: [0]}
+    nbrs = np.full((len(xs), 3), -1, np.int32)
+    for i, r in rows.items():
+        nbrs[i, :len(r)] = r
+    q = np.zeros((1, 4), np.float32)
+    expect = dict(ids=[10, 5, 4], dists=[1.0, 36.0, 49.0], hops=8, expansions=7, dist_evals=11, rounds=5)
+    return base, nbrs, np.array([0], np.int32), q, 3, 3, expect
