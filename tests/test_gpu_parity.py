@@ -115,12 +115,19 @@ def test_hand_computed_traversals_through_the_c_abi():
         assert idx.query_counters(1)[0].tolist() == [want["hops"], want["expansions"], want["dist_evals"],
                                                       want["rounds"]]
         assert (st.hops, st.expansions, st.dist_evals) == (want["hops"], want["expansions"], want["dist_evals"])
+    idx.set_deleted(np.array([1 << 5], np.uint32))  # node 5 tombstoned: same traversal, 5 left out of the output
+    idx.prepare(1, L, policy=0)
+    ids, dists, st = idx.search(q, k, L, policy=0, have_delete=True)
+    assert ids[0].tolist() == [10, 4, -1] and dists[0].tolist() == [1.0, 49.0, float(np.finfo(np.float32).max)]
+    assert idx.query_counters(1)[0].tolist() == [want["hops"], want["expansions"], want["dist_evals"], want["rounds"]]
     for in_lds, packed, table in ((False, False, 0), (False, True, 0), (True, False, 0), (False, False, -1),
                                   (False, False, 8)):
         idx.prepare(1, L, policy=1, best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=table)
         ids, dists, st = idx.search(q, k, L, policy=1)
         assert ids[0].tolist() == [10, 5, 6] and dists[0].tolist() == [1.0, 36.0, 56.25]
         assert idx.query_counters(1)[0, :3].tolist() == [1 + 5, 5, 7]
+        ids, dists, st = idx.search(q, k, L, policy=1, have_delete=True)
+        assert ids[0].tolist() == [10, 6, -1] and dists[0, :2].tolist() == [1.0, 56.25]
     idx.close()
 
 

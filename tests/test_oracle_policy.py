@@ -193,6 +193,12 @@ def test_rounds_policy_hand_computed_counters(orc):
     dist = {i: float(x) ** 2 for i, x in enumerate(base[:, 2])}
     sim = pysim.policy_rounds(nbrs.tolist(), starts.tolist(), dist, L, k)
     assert sim == (want["ids"], want["hops"], want["expansions"], want["dist_evals"])
+    # node 5 tombstoned (src/search_gpu.cu:695-725): the traversal and its counters are untouched, the output
+    # skips 5 and, the beam exhausted, ends in id -1 with the farthest distance
+    dead = orc.Problem(base, nbrs, starts, deleted=np.array([1 << 5], np.uint32))
+    ids, dists, stats, _ = orc.search_B(dead, q, k, L, start_order=0, nbr_order=0)
+    assert ids[0].tolist() == [10, 4, -1] and dists[0].tolist() == [1.0, 49.0, float(np.finfo(np.float32).max)]
+    assert stats[0].tolist() == [want["hops"], want["expansions"], want["dist_evals"], want["rounds"]]
     # the same points under best-first: 0 -> 1, 2; 2 -> 5 (0 leaves the queue); 5 -> 6, 7 (1 and 2 leave);
     # 6 -> 10 (7 leaves, unexpanded); 10 -> nothing new.  Five expansions, seven distances, and a different
     # answer: 4 is never reached, because 1, the only way to it, was dropped unexpanded.
