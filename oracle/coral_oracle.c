@@ -29,9 +29,11 @@
  *     that were written from it; plus brute-force invariants.
  *   - oracle_dist ORDER_GPU_SEQ / ORDER_GPU_WARP32 / ORDER_WAVE64: fp64 closed
  *     form within 1e-5 relative; special cases (identical vectors, unit vectors,
- *     one-hot vectors that expose index or sign mistakes).  The exact rounding of
- *     the two CUDA orders cannot be executed anywhere here: they are pinned by
- *     code reading only; the 1e-5 tolerance of the search contract covers it.
+ *     one-hot vectors that expose index or sign mistakes).  The two CUDA orders
+ *     cannot be executed anywhere here; their order of additions is pinned by
+ *     hand-computed inputs on which fp32 absorbs an addend (2^24 + 1), so that a
+ *     chain, a lane stride of 32 and a shuffle-down tree from offset 16 each give
+ *     a different, known value.
  *   - oracle_search_B: nothing executable exists for it (the CUDA kernel cannot
  *     be built or run here).  Pinned by code reading plus invariants: result ==
  *     top-k of top-L(visited) under (distance,id); every beam entry expanded at

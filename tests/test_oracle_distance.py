@@ -106,3 +106,43 @@ def test_normalize_matches_numpy_restatement(orc):
     assert not y[7].any()
     n = np.linalg.norm(y.astype(np.float64), axis=1)
     assert np.allclose(np.delete(n, 7), 1.0, atol=1e-6)
+
+
+def test_cuda_summation_orders_known_answers(orc):
+    """Inputs on which fp32 absorbs an addend (2^24 + 1 rounds back to 2^24), so that the ORDER of the additions
+    decides the result and each result can be worked out by hand: the one-thread chain of include/utils.cuh:254-275
+    and :307-323 (order 0) against the lane-strided partial sums and the shuffle-down tree, offsets 16 to 1, of
+    src/search_gpu.cu:14-23 (order 1).  A chain summed as a tree, a lane stride other than 32 or a tree walked from
+    offset 1 upwards gives the other value."""
+    big = float(2 ** 24)
+    ones = np.ones(64, np.float32)
+
+    def vec(**at):
+        b = np.zeros(64, np.float32)
+        for i, x in at.items():
+            b[int(i[1:])] = x
+        return b
+
+    # inner product with a vector of ones = the plain sum of b
+    # chain: (2^24 + 1) - 2^24 = 0;  lanes 0, 1, 2 -> tree: (2^24 - 2^24) + 1 = 1
+    b = vec(i0=big, i1=1.0, i2=-big)
+    assert orc.dist(ones, b, orc.IP, 0) == 0.0 and orc.dist(ones, b, orc.IP, 1) == 1.0
+    # chain: (2^24 - 2^24) + 1 = 1;  lane 0 holds coordinates 0 and 32: (2^24 + 1) - 2^24 = 0
+    b = vec(i0=big, i1=-big, i32=1.0)
+    assert orc.dist(ones, b, orc.IP, 0) == 1.0 and orc.dist(ones, b, orc.IP, 1) == 0.0
+    # the tree adds lane 16 to lane 0 before lane 1: (2^24 - 2^24) + 1 = 1; from offset 1 upwards it would be 0.
+    # chain: (2^24 + 1) - 2^24 = 0
+    b = vec(i0=big, i1=1.0, i16=-big)
+    assert orc.dist(ones, b, orc.IP, 1) == 1.0 and orc.dist(ones, b, orc.IP, 0) == 0.0
+    # squared L2 from the origin: 4096^2 + 1 + 1.  chain: both ones absorbed; tree: lanes 1 and 3 meet first (2),
+    # then 2^24 + 2 is exact.  The CPU routine (include/efanna2e/distance.h:39-89) ends in
+    # (m0 + m1) + (m2 + m3) = (2^24 + 1) + (0 + 1): both absorbed
+    zero = np.zeros(64, np.float32)
+    b = vec(i0=4096.0, i1=1.0, i3=1.0)
+    assert orc.dist(zero, b, orc.L2, 0) == big and orc.dist(zero, b, orc.L2, 1) == big + 2.0
+    assert orc.dist(zero, b, orc.L2, 2) == big
+    # ones in lanes 4 and 5 never meet each other in the shuffle-down tree: offset 4 brings lane 4 to lane 0
+    # (absorbed) and lane 5 to lane 1, offset 1 adds lane 1 (absorbed).  A tree that pairs neighbours first
+    # would give 2^24 + 2.  CPU: m2 = [2^24 + 1 -> 2^24, 1, 0, 0] -> 2^24 + 1 -> 2^24
+    b = vec(i0=4096.0, i4=1.0, i5=1.0)
+    assert orc.dist(zero, b, orc.L2, 1) == big and orc.dist(zero, b, orc.L2, 2) == big
