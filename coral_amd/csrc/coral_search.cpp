@@ -37,7 +37,7 @@ int fail(int code, const char* fmt, ...) {
 namespace {
 using coral::fail;
 
-constexpr int kMaxL = 2048;
+constexpr int kMaxL = CORAL_MAX_BEAM;
 constexpr int kMaxLdsBytes = 160 * 1024;
 
 // bits of a mixed id that a cell of the wavefront kernel's table stores: what the bucket index (a quarter of the

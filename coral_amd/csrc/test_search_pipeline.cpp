@@ -209,7 +209,14 @@ int main(int argc, char** argv) {
             const float avg_hops = tr.avg_hops((int)q_pts);
             std::cout << L << "\t\t" << qps << "\t\t" << time << "\t\t" << recall << "\t\t" << avg_hops << std::endl;
             evaluation_out << L << "," << qps << "," << time << "," << recall << "," << avg_hops << std::endl;
-            if (max_recall > 0.5 && recall < max_recall) L_vec.push_back(128 + L_vec.back());
+            if (max_recall > 0.5 && recall < max_recall) {
+                if (128 + L_vec.back() > CORAL_MAX_BEAM) {
+                    std::cout << "Beam capacity limit " << CORAL_MAX_BEAM
+                              << " reached, judged as unable to meet the recall requirement, termination" << std::endl;
+                    break;
+                }
+                L_vec.push_back(128 + L_vec.back());
+            }
             if (i > 50) {
                 std::cout << "Queue is too long, judged as unable to meet the recall requirement, termination"
                           << std::endl;

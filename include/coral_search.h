@@ -140,8 +140,11 @@ CORAL_API int coral_index_get_deleted(coral_index* idx, uint32_t* host_mask);
 CORAL_API int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* R,
                      int32_t* n_start, int32_t* metric);
 
+/* Largest beam capacity L: the beam lives in LDS (the reference keeps it in global memory and sets no limit). */
+#define CORAL_MAX_BEAM 2048
+
 /* GPUFuncs::search_prepare(Q, L) (src/search.cu:400-408): fixes the beam
- * capacity and (re)allocates per-workgroup scratch. */
+ * capacity (1..CORAL_MAX_BEAM) and (re)allocates per-workgroup scratch. */
 CORAL_API int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tuning* tuning);
 
 /* GPUFuncs::search_gpu (src/search_gpu.cu:835-886): device pointers in and out,

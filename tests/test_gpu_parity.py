@@ -437,6 +437,21 @@ def test_cli_end_to_end(orc, tmp_path):
     row = [l for l in r.stdout.splitlines() if l.startswith("32\t")][0].split()
     assert abs(float(row[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
     assert abs(float(row[4]) - os_[:, 0].sum() / Q) < 1e-2
+    # no --L but a recall to reach: L starts at 128 and grows by 128 until the recall is met
+    # (tests/test_search_pipeline.cpp:278-313) ...
+    def table_rows(out):
+        return [l.split() for l in out.splitlines() if l[:1].isdigit() and len(l.split()) == 5]
+    grow = args[:-7] + ["--config_file", str(work / "config.json")]
+    r = subprocess.run(grow + ["--max_recall", "0.9"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    rows = table_rows(r.stdout)
+    assert [int(f[0]) for f in rows] == [128 * (i + 1) for i in range(len(rows))]
+    assert float(rows[-1][3]) >= 0.9 and all(float(f[3]) < 0.9 for f in rows[:-1])
+    # ... or until the beam capacity the library supports: a recall that cannot be met ends the run in good order
+    r = subprocess.run(grow + ["--max_recall", "1.01"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert [int(f[0]) for f in table_rows(r.stdout)] == list(range(128, 2048 + 1, 128))
+    assert "Beam capacity limit 2048 reached" in r.stdout
 
 
 def test_randomised_shapes(orc):
