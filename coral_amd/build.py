@@ -40,9 +40,10 @@ def _run(cmd):
         raise RuntimeError("build step failed: " + " ".join(cmd))
 
 
-def build(verbose=True):
+def build(verbose=True, jobs=None):
+    from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIBDIR, exist_ok=True)
-    objs = []
+    objs, cmds = [], []
     for src in LIB_SOURCES:
         path = os.path.join(CSRC, src)
         if not os.path.exists(path):
@@ -50,8 +51,11 @@ def build(verbose=True):
         obj = os.path.join(LIBDIR, src + ".o")
         cmd = [HIPCC] + COMMON + ["-fopenmp", "-fvisibility=hidden", "-DCORAL_BUILD"]
         cmd += DEVICE if src.endswith(".hip") else HOST
-        _run(cmd + ["-c", path, "-o", obj])
+        cmds.append(cmd + ["-c", path, "-o", obj])
         objs.append(obj)
+    # the translation units are independent: compile them side by side
+    with ThreadPoolExecutor(jobs or min(8, os.cpu_count() or 1)) as ex:
+        list(ex.map(_run, cmds))
     _run([HIPCC, "-shared", "-fopenmp", "-o", LIB] + objs)
     for src in CLI_SOURCES:
         path = os.path.join(CSRC, src)

@@ -14,6 +14,7 @@ LIB_PATH = os.environ.get("CORAL_SEARCH_LIB") or os.path.join(HERE, "lib", "libc
 
 L2, IP = 0, 1
 POLICY_ROUNDS, POLICY_BEST_FIRST = 0, 1
+MAX_LDS_BEAM, MAX_BEAM = 2048, 65536  # CORAL_MAX_LDS_BEAM, CORAL_MAX_BEAM
 
 OK, ERR_ARG, ERR_GRAPH, ERR_DEVICE, ERR_MEMORY, ERR_IO, ERR_STATE = range(7)
 
@@ -41,7 +42,7 @@ class Stats(C.Structure):
 class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
                 ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("best_first_packed", C.c_int32),
-                ("best_first_table_log2", C.c_int32), ("reserved", C.c_int32 * 1)]
+                ("best_first_table_log2", C.c_int32), ("beam_in_hbm", C.c_int32)]
 
 
 class BuildParams(C.Structure):
@@ -197,9 +198,9 @@ class Index:
         return m
 
     def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False,
-                best_first_packed=False, best_first_table_log2=0):
+                best_first_packed=False, best_first_table_log2=0, beam_in_hbm=False):
         t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)),
-                   int(bool(best_first_packed)), best_first_table_log2)
+                   int(bool(best_first_packed)), best_first_table_log2, int(bool(beam_in_hbm)))
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

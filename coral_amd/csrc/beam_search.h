@@ -34,6 +34,14 @@ struct SearchArgs {
     int32_t dmax;              // largest displacement a cell can encode (-1: table unused)
     int32_t ocap;              // LDS list of ids sent to the global bitmap (multiple of 4)
     int32_t tcap, ccap;        // LDS todo / candidate capacities (multiples of 4, ccap >= tcap)
+    // Beams too long for LDS (launches of the kernel's BIG form): the two beam buffers and the list of entries to
+    // expand live in global memory, beam_stride 64-bit words per workgroup ([2][Lp] keys, then Lp ids).
+    uint64_t* beam_scratch;
+    size_t beam_stride;
+    // BIG form only: the visited set is a plain bitmap of the n ids in LDS (table_words 32-bit words) instead of
+    // the table of 16-bit cells; no id ever goes to the bitmap in global memory then
+    int32_t direct_bitmap;
+    int32_t table_words;       // 32-bit words of LDS the visited structure takes (cells / 2, or ceil(n / 32) rounded up to 4)
 };
 
 // What the wavefront-per-query best-first kernel (best_first.hip) needs beyond SearchArgs.
@@ -74,10 +82,15 @@ hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStr
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice
 hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream);
 
-size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap, int ocap);
-hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu);
-hipError_t launch_search(const SearchArgs& a, int workgroups, int threads, size_t lds_bytes,
+// LDS bytes of one workgroup.  big: the beams and the expand list are in global memory, LDS holds the candidate
+// buffer, the visited structure (table_words 32-bit words), the todo list, the overflow list and the query.
+size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big);
+// 64-bit words of global scratch one workgroup of a BIG launch needs for a beam of capacity L
+size_t search_beam_stride(int L);
+hipError_t search_kernel_prepare(int dim, bool big, size_t lds_bytes, int threads, int* max_wg_per_cu);
+hipError_t launch_search(const SearchArgs& a, bool big, int workgroups, int threads, size_t lds_bytes,
                          hipStream_t stream);
+
 hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,
                          hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t stream);

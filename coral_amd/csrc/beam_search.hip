@@ -15,7 +15,12 @@
 //     flight per wave, and reduced across lanes (the reference lets one thread
 //     walk a whole row, include/utils.cuh:254-275);
 //   * candidates are bitonic-sorted and merged into the beam by rank; the
-//     reference replaces the current worst entry one candidate at a time (:530-570).
+//     reference replaces the current worst entry one candidate at a time (:530-570);
+//   * beams too long for LDS (the reference sets no limit on L, src/search.cu:400-408) run the
+//     kernel's BIG form: the two beam buffers move to a per-workgroup block of global memory
+//     (read and written in whole coalesced passes by the merge, so they live in L2), and the LDS
+//     they leave holds the visited set as a plain bitmap of all n ids where n allows
+//     (a million nodes = 125 KB): one LDS atomic per test, nothing ever spills.
 //
 // Distance summation order (mirrored bit for bit by the test oracle): lane l of a
 // group of G lanes accumulates float4 chunks l, l+G, ... with four fused
@@ -74,6 +79,7 @@ struct VisitedSet {
     uint32_t* bitmap;  // global
     uint32_t smask, bmask, rmask;
     int rb, xs, dmax, ocap;
+    bool direct;       // words is a bitmap of all ids (BIG launches over few enough nodes)
 
     __device__ __forceinline__ uint32_t mix(uint32_t id) const {
         uint32_t h = (id * 0x9E3779B1u) & bmask;
@@ -84,7 +90,12 @@ struct VisitedSet {
     }
 
     // 1 if id was not yet in the set (and now is), 0 if it was
+    template <bool BIG>
     __device__ __forceinline__ int test_and_set(uint32_t id, bool frozen) {
+        if (BIG && direct) {
+            const uint32_t b = 1u << (id & 31);
+            return (atomicOr(&words[id >> 5], b) & b) == 0u;
+        }
         const uint32_t h = mix(id);
         const uint32_t home = h >> rb, rem = h & rmask;
         const uint16_t* cells = reinterpret_cast<const uint16_t*>(words);
@@ -123,7 +134,7 @@ struct WgState {
     uint64_t live;    // key of the worst entry of a full beam, else kKeyMax
 };
 
-template <int G, int CPL>
+template <int G, int CPL, bool BIG>
 __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, NT = blockDim.x;
@@ -133,16 +144,28 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     const int slots = 1 << a.slots_log2;
     const int TCAP = a.tcap, CCAP = a.ccap;
 
-    uint64_t* beam0 = (uint64_t*)smem;
-    uint64_t* beam1 = beam0 + Lp;
-    uint64_t* cand = beam1 + Lp;
-    uint32_t* table = (uint32_t*)(cand + CCAP);  // slots 16-bit cells
-    uint32_t* todo = table + (slots >> 1);
-    uint32_t* elist = todo + TCAP;
-    uint32_t* olist = elist + Lp;
+    uint64_t *beam0, *beam1, *cand;
+    uint32_t *table, *todo, *elist, *olist;
+    if constexpr (BIG) {
+        uint64_t* g = a.beam_scratch + (size_t)blockIdx.x * a.beam_stride;
+        beam0 = g, beam1 = g + Lp, elist = (uint32_t*)(g + 2 * (size_t)Lp);
+        cand = (uint64_t*)smem;
+        table = (uint32_t*)(cand + CCAP);  // 16-bit cells, or the bitmap of all ids
+        todo = table + a.table_words;
+        olist = todo + TCAP;
+    } else {
+        beam0 = (uint64_t*)smem;
+        beam1 = beam0 + Lp;
+        cand = beam1 + Lp;
+        table = (uint32_t*)(cand + CCAP);  // slots 16-bit cells
+        todo = table + a.table_words;
+        elist = todo + TCAP;
+        olist = elist + Lp;
+    }
     float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_cursor, s_outpos, s_nover;
+    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_cursor, s_nover;
+    __shared__ int s_wcnt[16];
 
     VisitedSet vs;
     vs.words = table, vs.olist = olist, vs.ocount = &s_nover;
@@ -150,6 +173,8 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     vs.smask = (uint32_t)slots - 1u, vs.bmask = a.id_bits >= 32 ? 0xffffffffu : (1u << a.id_bits) - 1u;
     vs.rb = a.rem_bits, vs.rmask = (1u << a.rem_bits) - 1u;
     vs.xs = a.id_bits > 1 ? a.id_bits / 2 : 1, vs.dmax = a.dmax, vs.ocap = a.ocap;
+    vs.direct = BIG && a.direct_bitmap != 0;
+    (void)slots;
 
     constexpr int GPW = 64 / G;                    // row groups per wave
     constexpr int U = (CPL >= 8) ? 1 : (8 / CPL);  // rows in flight per group
@@ -164,7 +189,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         if (qid >= a.Q) break;
         PHASE_DECL;
 
-        for (int i = tid; i < (slots >> 1); i += NT) table[i] = 0u;
+        for (int i = tid; i < a.table_words; i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
         if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0, s_cursor = 0;
         __syncthreads();
@@ -361,7 +386,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         const int M = a.M;
         for (int i = tid; i < M; i += NT) {
             const uint32_t id = (uint32_t)a.start_ids[i];
-            vs.test_and_set(id, false);
+            vs.template test_and_set<BIG>(id, false);
             todo[i] = id;
         }
         __syncthreads();
@@ -450,7 +475,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                         v = a.nbrs[(size_t)elist[e0 + e] * R + (f - e * R)];
                     }
                     bool isnew = false;
-                    if (v >= 0) isnew = vs.test_and_set((uint32_t)v, spill) != 0;
+                    if (v >= 0) isnew = vs.template test_and_set<BIG>((uint32_t)v, spill) != 0;
                     const uint64_t m = __ballot(isnew);
                     if (m) {
                         int pos = 0;
@@ -490,9 +515,10 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             const uint64_t* beam = st.cur ? beam1 : beam0;
             int32_t* ids_out = a.ids_out + (size_t)qid * a.k;
             float* dists_out = a.dists_out ? a.dists_out + (size_t)qid * a.k : nullptr;
-            if (tid == 0) s_outpos = 0;
-            __syncthreads();
-            for (int i0 = 0; i0 < st.nb; i0 += NT) {
+            // ordered compaction: every wave posts how many live entries it holds, and each finds its place
+            // from the counts of the waves before it; outpos is the same in every thread
+            int outpos = 0;
+            for (int i0 = 0; i0 < st.nb && outpos < a.k; i0 += NT) {
                 const int i = i0 + tid;
                 uint64_t key = 0;
                 bool livee = false;
@@ -504,27 +530,27 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                         livee = ((a.deleted[id >> 5] >> (id & 31)) & 1u) == 0;
                     }
                 }
-                // ordered compaction: waves take their turn through s_outpos
                 const uint64_t m = __ballot(livee);
+                if (lane == 0) s_wcnt[wave] = __popcll(m);
+                __syncthreads();
+                int before = 0, total = 0;
                 for (int w = 0; w < NW; ++w) {
-                    if (w == wave) {
-                        const int basepos = s_outpos;
-                        const int pos = basepos + prefix_popc(m);
-                        if (livee && pos < a.k) {
-                            ids_out[pos] = key_id(key);
-                            if (dists_out) {
-                                const float s = key_s(key);
-                                dists_out[pos] = a.metric == 0 ? s : 0.0f - s;
-                            }
-                        }
-                        if (lane == 0) s_outpos = basepos + __popcll(m);
-                    }
-                    __syncthreads();
+                    const int c = s_wcnt[w];
+                    before += w < wave ? c : 0;
+                    total += c;
                 }
-                if (s_outpos >= a.k) break;
+                const int pos = outpos + before + prefix_popc(m);
+                if (livee && pos < a.k) {
+                    ids_out[pos] = key_id(key);
+                    if (dists_out) {
+                        const float s = key_s(key);
+                        dists_out[pos] = a.metric == 0 ? s : 0.0f - s;
+                    }
+                }
+                outpos += total;
+                __syncthreads();  // the counts are read before the next chunk posts its own
             }
-            __syncthreads();
-            for (int i = s_outpos + tid; i < a.k; i += NT) {
+            for (int i = outpos + tid; i < a.k; i += NT) {
                 ids_out[i] = -1;
                 // unfilled slots: the farthest sentinel (rounds: +-FLT_MAX as the CUDA kernel pads its
                 // beam, src/search_gpu.cu:408; best-first: +-infinity, src/search_in_cpu.cpp:33-35)
@@ -586,25 +612,35 @@ __global__ void fill_u32_kernel(uint32_t* p, size_t n, uint32_t v) {
 
 typedef void (*kernel_fn)(const SearchArgs);
 
-static kernel_fn pick_kernel(int dim) {
-    const int chunks = dim / 4;
-    if (chunks <= 16) return beam_search_kernel<16, 1>;
-    if (chunks <= 32) return beam_search_kernel<32, 1>;
-    if (chunks <= 64) return beam_search_kernel<64, 1>;
-    if (chunks <= 128) return beam_search_kernel<64, 2>;
-    if (chunks <= 256) return beam_search_kernel<64, 4>;
-    if (chunks <= 512) return beam_search_kernel<64, 8>;
+template <bool BIG>
+static kernel_fn pick_kernel_form(int chunks) {
+    if (chunks <= 16) return beam_search_kernel<16, 1, BIG>;
+    if (chunks <= 32) return beam_search_kernel<32, 1, BIG>;
+    if (chunks <= 64) return beam_search_kernel<64, 1, BIG>;
+    if (chunks <= 128) return beam_search_kernel<64, 2, BIG>;
+    if (chunks <= 256) return beam_search_kernel<64, 4, BIG>;
+    if (chunks <= 512) return beam_search_kernel<64, 8, BIG>;
     return nullptr;
 }
 
-size_t search_lds_bytes(int L, int dim, int slots_log2, int tcap, int ccap, int ocap) {
-    const size_t Lp = (size_t)((L + 3) & ~3);
-    return Lp * 8 * 2 + (size_t)ccap * 8 + ((size_t)2 << slots_log2) + (size_t)tcap * 4 + Lp * 4 +
-           (size_t)ocap * 4 + (size_t)((dim + 3) & ~3) * 4;
+static kernel_fn pick_kernel(int dim, bool big) {
+    return big ? pick_kernel_form<true>(dim / 4) : pick_kernel_form<false>(dim / 4);
 }
 
-hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* max_wg_per_cu) {
-    kernel_fn fn = pick_kernel(dim);
+size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big) {
+    const size_t Lp = (size_t)((L + 3) & ~3);
+    const size_t beams = big ? 0 : Lp * 8 * 2 + Lp * 4;  // two key buffers and the expand list
+    return beams + (size_t)ccap * 8 + (size_t)table_words * 4 + (size_t)tcap * 4 + (size_t)ocap * 4 +
+           (size_t)((dim + 3) & ~3) * 4;
+}
+
+size_t search_beam_stride(int L) {
+    const size_t Lp = (size_t)((L + 3) & ~3);
+    return (2 * Lp + Lp / 2 + 15) & ~(size_t)15;  // [2][Lp] keys + Lp 32-bit ids, a multiple of 128 bytes
+}
+
+hipError_t search_kernel_prepare(int dim, bool big, size_t lds_bytes, int threads, int* max_wg_per_cu) {
+    kernel_fn fn = pick_kernel(dim, big);
     if (!fn) return hipErrorInvalidValue;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -617,9 +653,9 @@ hipError_t search_kernel_prepare(int dim, size_t lds_bytes, int threads, int* ma
     return hipSuccess;
 }
 
-hipError_t launch_search(const SearchArgs& a, int workgroups, int threads, size_t lds_bytes,
+hipError_t launch_search(const SearchArgs& a, bool big, int workgroups, int threads, size_t lds_bytes,
                          hipStream_t stream) {
-    kernel_fn fn = pick_kernel(a.dim);
+    kernel_fn fn = pick_kernel(a.dim, big);
     if (!fn) return hipErrorInvalidValue;
     hipLaunchKernelGGL(fn, dim3(workgroups), dim3(threads), lds_bytes, stream, a);
     return hipGetLastError();

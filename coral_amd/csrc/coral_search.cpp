@@ -37,7 +37,7 @@ int fail(int code, const char* fmt, ...) {
 namespace {
 using coral::fail;
 
-constexpr int kMaxL = CORAL_MAX_BEAM;
+constexpr int kMaxL = CORAL_MAX_BEAM;  // beams beyond CORAL_MAX_LDS_BEAM live in global memory
 constexpr int kMaxLdsBytes = 160 * 1024;
 
 // bits of a mixed id that a cell of the wavefront kernel's table stores: what the bucket index (a quarter of the
@@ -180,6 +180,7 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_start);
     (void)hipFree(idx->d_deleted);
     (void)hipFree(idx->d_spill);
+    (void)hipFree(idx->d_beam);
     (void)hipFree(idx->d_counters);
     (void)hipFree(idx->d_scalars);
     (void)hipFree(idx->d_hit);
@@ -248,55 +249,75 @@ int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* 
     return CORAL_OK;
 }
 
-int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tuning* tuning) {
-    if (!idx) return fail(CORAL_ERR_ARG, "null index");
-    if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
+// Launch geometry of the workgroup-per-query kernel for a beam of capacity L: arithmetic, the kernel's LDS
+// attribute and an occupancy query; nothing is allocated.  bump_log2 raises the library's own choice of table size.
+static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral_tuning& t, int bump_log2,
+                       coral_search_plan* out) {
     if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
     if (L <= 0 || L > kMaxL) return fail(CORAL_ERR_ARG, "L must be in 1..%d (got %d)", kMaxL, L);
     if (idx->M <= 0) return fail(CORAL_ERR_STATE, "the graph has no start ids yet (rows under construction)");
     if (idx->M > L)
         return fail(CORAL_ERR_ARG, "%d start ids do not fit a beam of capacity %d", idx->M, L);
-    coral_tuning t;
-    std::memset(&t, 0, sizeof t);
-    if (tuning) t = *tuning;
     if (t.policy != CORAL_POLICY_ROUNDS && t.policy != CORAL_POLICY_BEST_FIRST)
         return fail(CORAL_ERR_ARG, "unknown policy %d", t.policy);
     const bool best_first = t.policy == CORAL_POLICY_BEST_FIRST;
-    HIP_TRY(hipSetDevice(idx->device));
-    HIP_TRY(hipStreamSynchronize(idx->stream));
-
-    // todo / candidate buffers: sized below, once the visited table is known
+    coral_search_plan p;
+    p.L = L;
+    p.big = L > CORAL_MAX_LDS_BEAM || t.beam_in_hbm != 0;
+    // todo / candidate buffers: sized below, once the visited structure is known
     int min_cap = 256;
     while (min_cap < idx->M || min_cap < idx->R * 4) min_cap <<= 1;
     int tcap = min_cap;
-    const int ocap = 256;
+    int ocap = 256;
     int id_bits = 1;
     while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
     int slots_log2 = t.visited_slots_log2;
-    if (slots_log2 == 0) {
+    auto table_lds = [&](int lg, int cap) {
+        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, ocap, p.big) + 64;
+    };
+    if (p.big) {
+        // The beams are out of LDS.  What they leave takes the visited set as a bitmap of all n ids where that fits
+        // (a million nodes = 125 KB), else the largest table of cells; one workgroup of 1024 threads per CU.
+        if (!best_first) tcap = std::max(tcap, 1024);
+        const int bitmap_words = (int)(((idx->n + 31) / 32 + 3) & ~(int64_t)3);
+        if (slots_log2 == 0 && idx->n <= ((int64_t)1 << 21) &&
+            coral::search_lds_bytes(L, idx->dim, bitmap_words, tcap, tcap, 4, true) + 64 <= (size_t)kMaxLdsBytes) {
+            p.direct = 1, p.table_words = bitmap_words, ocap = 4;
+        } else if (slots_log2 == 0) {
+            slots_log2 = 16;
+            while (slots_log2 > 12 && table_lds(slots_log2, tcap) > (size_t)kMaxLdsBytes) --slots_log2;
+        }
+    } else if (slots_log2 == 0) {
         // a degree-32 graph over a million nodes sees about 75 first visits per beam
         // entry; 112 cells per entry keep the load factor near 0.65
         // (best-first: about 31 first visits per entry, 48 cells)
         slots_log2 = 12;
         while ((1 << slots_log2) < (best_first ? 48 : 112) * L && slots_log2 < 16) ++slots_log2;
-        if (idx->bump_L == L) slots_log2 = std::min(16, slots_log2 + idx->bump_log2);  // see coral_search_gpu
-        while (slots_log2 > 12 &&
-               coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap) + 64 > (size_t)kMaxLdsBytes)
-            --slots_log2;
+        slots_log2 = std::min(16, slots_log2 + bump_log2);  // see coral_search_gpu
+        while (slots_log2 > 12 && table_lds(slots_log2, tcap) > (size_t)kMaxLdsBytes) --slots_log2;
     }
-    if (slots_log2 < 10 || slots_log2 > 16)
-        return fail(CORAL_ERR_ARG, "visited_slots_log2 must be in 10..16");
-    const int slots = 1 << slots_log2;
-    const int rem_bits = std::max(0, id_bits - slots_log2);
-    // a cell is 1 + ((d << rem_bits) | remainder) in 16 bits
-    int dmax = rem_bits >= 16 ? -1 : std::min(63, (65535 >> rem_bits) - 1);
-    const int vis_limit = dmax < 0 ? 0 : slots - slots / 4;
+    if (!p.direct) {
+        if (slots_log2 < 10 || slots_log2 > 16)
+            return fail(CORAL_ERR_ARG, "visited_slots_log2 must be in 10..16");
+        const int slots = 1 << slots_log2;
+        p.slots_log2 = slots_log2, p.table_words = slots >> 1;
+        p.rem_bits = std::max(0, id_bits - slots_log2);
+        // a cell is 1 + ((d << rem_bits) | remainder) in 16 bits
+        p.dmax = p.rem_bits >= 16 ? -1 : std::min(63, (65535 >> p.rem_bits) - 1);
+        p.vis_limit = p.dmax < 0 ? 0 : slots - slots / 4;
+        p.spill_words = ((size_t)idx->n + 31) / 32;
+    } else {
+        p.dmax = -1, p.vis_limit = 0x7fffffff;
+    }
     // Larger chunks mean fewer latency-bound steps per round: take the largest todo /
     // candidate capacity that does not lower the number of workgroups a CU can hold.
-    auto lds_for = [&](int cap) { return coral::search_lds_bytes(L, idx->dim, slots_log2, cap, cap, ocap) + 64; };
+    auto lds_for = [&](int cap) {
+        return coral::search_lds_bytes(L, idx->dim, p.table_words, cap, cap, ocap, p.big) + 64;
+    };
     if (lds_for(min_cap) > (size_t)kMaxLdsBytes)
-        return fail(CORAL_ERR_ARG, "L=%d with a %d-cell visited table needs %zu bytes of LDS", L, slots,
+        return fail(CORAL_ERR_ARG, "L=%d with %d words of visited state needs %zu bytes of LDS", L, p.table_words,
                     lds_for(min_cap));
+    while (tcap > min_cap && lds_for(tcap) > (size_t)kMaxLdsBytes) tcap >>= 1;
     const int wg_fit = (int)((size_t)kMaxLdsBytes / lds_for(min_cap));
     // (capacities are powers of two: the candidate buffer is bitonic-sorted in place)
     for (int cap : {1024, 512}) {
@@ -307,29 +328,58 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         }
     }
     int threads = t.threads;
-    if (threads == 0) threads = best_first ? 256 : (lds_for(tcap) > (size_t)kMaxLdsBytes / 2 ? 1024 : 512);
+    if (threads == 0)
+        threads = p.big ? 1024 : best_first ? 256 : (lds_for(tcap) > (size_t)kMaxLdsBytes / 2 ? 1024 : 512);
     if (threads != 128 && threads != 256 && threads != 512 && threads != 1024)
         return fail(CORAL_ERR_ARG, "threads must be 128, 256, 512 or 1024");
-    const size_t lds = coral::search_lds_bytes(L, idx->dim, slots_log2, tcap, tcap, ocap);
+    p.lds_bytes = coral::search_lds_bytes(L, idx->dim, p.table_words, tcap, tcap, ocap, p.big);
     int wg_per_cu = 0;
-    HIP_TRY(coral::search_kernel_prepare(idx->dim, lds, threads, &wg_per_cu));
+    HIP_TRY(coral::search_kernel_prepare(idx->dim, p.big, p.lds_bytes, threads, &wg_per_cu));
     if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
     int workgroups = t.workgroups > 0 ? t.workgroups : wg_per_cu * idx->num_cu;
-    workgroups = std::min(workgroups, (int)Q);
+    p.workgroups = std::min(workgroups, (int)Q);
+    p.tcap = tcap, p.ccap = tcap, p.threads = threads, p.id_bits = id_bits, p.ocap = ocap;
+    p.beam_stride = p.big ? coral::search_beam_stride(L) : 0;
+    *out = p;
+    return CORAL_OK;
+}
 
-    int table_log2 = 0;  // of the wavefront-per-query best-first kernel
-    if (best_first && !t.best_first_in_lds)
+int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tuning* tuning) {
+    if (!idx) return fail(CORAL_ERR_ARG, "null index");
+    if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
+    coral_tuning t;
+    std::memset(&t, 0, sizeof t);
+    if (tuning) t = *tuning;
+    HIP_TRY(hipSetDevice(idx->device));
+    coral_search_plan plan;
+    if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, &plan)) return rc;
+    HIP_TRY(hipStreamSynchronize(idx->stream));
+    const bool best_first = t.policy == CORAL_POLICY_BEST_FIRST;
+    const int id_bits = plan.id_bits;
+    const int workgroups = plan.workgroups;
+
+    // the wavefront-per-query best-first kernel keeps its beam in LDS: four wavefronts of a workgroup must fit
+    const bool wave_form = best_first && !t.best_first_in_lds && !plan.big &&
+                           coral::best_first_wave_lds_bytes(L, 0, 0) * 4 <= (size_t)kMaxLdsBytes;
+    int table_log2 = 0;
+    if (wave_form)
         if (int rc = choose_bf_table(L, id_bits, t.best_first_table_log2, &table_log2)) return rc;
     // from here on buffers are replaced: a failure part-way leaves the index unprepared, not half-prepared
     idx->prepared = false;
-    const size_t spill_words = ((size_t)idx->n + 31) / 32;
-    const size_t need_words = spill_words * (size_t)workgroups;
+    const size_t need_words = plan.spill_words * (size_t)workgroups;
     if (need_words > idx->spill_alloc_words) {
         (void)hipFree(idx->d_spill);
         idx->d_spill = nullptr, idx->spill_alloc_words = 0;
         HIP_TRY(hipMalloc(&idx->d_spill, need_words * sizeof(uint32_t)));
         idx->spill_alloc_words = need_words;
         HIP_TRY(coral::launch_fill_u32(idx->d_spill, need_words, 0u, idx->stream));
+    }
+    const size_t need_beam = plan.beam_stride * (size_t)workgroups;
+    if (need_beam > idx->beam_alloc_words) {
+        (void)hipFree(idx->d_beam);
+        idx->d_beam = nullptr, idx->beam_alloc_words = 0;
+        HIP_TRY(hipMalloc(&idx->d_beam, need_beam * sizeof(uint64_t)));
+        idx->beam_alloc_words = need_beam;
     }
     const size_t need_counters = (size_t)Q * 4;
     if (need_counters > idx->counters_alloc) {
@@ -343,7 +393,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // Best-first: one wavefront per query with the visited state in HBM (best_first.hip), when the memory for it
     // is there: n bytes per wavefront (n / 6 in the packed form), up to a third of what is free and 64 GiB.
     idx->bf_ready = false;
-    if (best_first && !t.best_first_in_lds) {
+    if (wave_form) {
         int bf_wg_per_cu = 0;
         const int chunks = idx->dim / 4;
         idx->bf_table_log2 = table_log2;
@@ -399,14 +449,30 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         }
     }
     HIP_TRY(hipStreamSynchronize(idx->stream));
-    idx->Q = Q, idx->L = L, idx->slots_log2 = slots_log2, idx->vis_limit = vis_limit;
-    idx->tcap = tcap, idx->ccap = tcap, idx->threads = threads, idx->workgroups = workgroups;
-    idx->id_bits = id_bits, idx->rem_bits = rem_bits, idx->dmax = dmax, idx->ocap = ocap;
+    idx->Q = Q, idx->L = L, idx->plan = plan;
     idx->prepared_policy = t.policy;
     idx->tuning = t;
-    idx->lds_bytes = lds, idx->spill_words = spill_words;
     idx->prepared = true;
     return CORAL_OK;
+}
+
+// the kernel's argument block for one call under a plan; scratch pointers are the caller's
+static coral::SearchArgs search_args(const coral_index* idx, const coral_search_plan& p, const float* d_queries,
+                                     int32_t* d_ids, float* d_dists, int32_t Q, int32_t k, int32_t policy,
+                                     int32_t have_delete) {
+    coral::SearchArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.vec = idx->d_vec, a.nbrs = idx->d_nbrs, a.start_ids = idx->d_start;
+    a.deleted = have_delete ? idx->d_deleted : nullptr;
+    a.queries = d_queries, a.ids_out = d_ids, a.dists_out = d_dists;
+    a.spill_words = p.spill_words, a.n = idx->n;
+    a.dim = idx->dim, a.R = idx->R, a.M = idx->M, a.Q = Q, a.k = k, a.L = p.L;
+    a.metric = idx->metric, a.policy = policy;
+    a.slots_log2 = p.slots_log2, a.vis_limit = p.vis_limit;
+    a.tcap = p.tcap, a.ccap = p.ccap;
+    a.id_bits = p.id_bits, a.rem_bits = p.rem_bits, a.dmax = p.dmax, a.ocap = p.ocap;
+    a.beam_stride = p.beam_stride, a.direct_bitmap = p.direct, a.table_words = p.table_words;
+    return a;
 }
 
 int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, float* d_dists,
@@ -424,19 +490,10 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     HIP_TRY(hipSetDevice(idx->device));
     hipStream_t stream = stream_ ? (hipStream_t)stream_ : idx->stream;
 
-    coral::SearchArgs a;
-    std::memset(&a, 0, sizeof a);
-    a.vec = idx->d_vec, a.nbrs = idx->d_nbrs, a.start_ids = idx->d_start;
-    a.deleted = have_delete ? idx->d_deleted : nullptr;
-    a.queries = d_queries, a.ids_out = d_ids, a.dists_out = d_dists;
-    a.counters = idx->d_counters, a.spill = idx->d_spill;
+    const coral_search_plan& plan = idx->plan;
+    coral::SearchArgs a = search_args(idx, plan, d_queries, d_ids, d_dists, Q, k, policy, have_delete);
+    a.counters = idx->d_counters, a.spill = idx->d_spill, a.beam_scratch = idx->d_beam;
     a.next_qid = idx->d_scalars, a.spill_count = idx->d_scalars + 1;
-    a.spill_words = idx->spill_words, a.n = idx->n;
-    a.dim = idx->dim, a.R = idx->R, a.M = idx->M, a.Q = Q, a.k = k, a.L = idx->L;
-    a.metric = idx->metric, a.policy = policy;
-    a.slots_log2 = idx->slots_log2, a.vis_limit = idx->vis_limit;
-    a.tcap = idx->tcap, a.ccap = idx->ccap;
-    a.id_bits = idx->id_bits, a.rem_bits = idx->rem_bits, a.dmax = idx->dmax, a.ocap = idx->ocap;
 
     const bool wave_kernel = policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready;
     if (wave_kernel && idx->rows_unique < 0) {
@@ -466,14 +523,14 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         b.packed = idx->bf_packed;
         b.bloom_log2 = idx->bf_bloom_log2;
         b.table_log2 = idx->bf_table_log2;
-        b.id_bits = idx->id_bits, b.rem_bits = idx->bf_table_rem_bits;
+        b.id_bits = plan.id_bits, b.rem_bits = idx->bf_table_rem_bits;
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;
         HIP_TRY(coral::launch_best_first(a, b, stream));
     } else {
-        const int wgs = std::min(idx->workgroups, (int)Q);
-        HIP_TRY(coral::launch_search(a, wgs, idx->threads, idx->lds_bytes, stream));
+        const int wgs = std::min(plan.workgroups, (int)Q);
+        HIP_TRY(coral::launch_search(a, plan.big, wgs, plan.threads, plan.lds_bytes, stream));
     }
     HIP_TRY(hipEventRecord(evk, stream));
     HIP_TRY(hipMemcpyAsync(idx->h_counters, idx->d_counters, (size_t)Q * 4 * sizeof(int32_t),
@@ -501,13 +558,13 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     // The table size the library picks assumes about 75 first visits per beam entry.  Data on which a query visits
     // more sends queries to the global bitmap (same results, slower): when more than a twentieth of a batch went
     // there, the next launches get a table twice the size.
-    const bool lds_table = !(policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready);
-    if (lds_table && idx->tuning.visited_slots_log2 == 0 && (int64_t)scal[1] * 20 > Q && idx->slots_log2 < 16) {
-        const int had = idx->slots_log2;
+    const bool lds_table = !(policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready) && !plan.big;
+    if (lds_table && idx->tuning.visited_slots_log2 == 0 && (int64_t)scal[1] * 20 > Q && plan.slots_log2 < 16) {
+        const int had = plan.slots_log2;
         idx->bump_log2 = idx->bump_L == idx->L ? idx->bump_log2 + 1 : 1;
         idx->bump_L = idx->L;
         coral_tuning t = idx->tuning;
-        if (coral_search_prepare(idx, idx->Q, idx->L, &t) != CORAL_OK || idx->slots_log2 == had) {
+        if (coral_search_prepare(idx, idx->Q, idx->L, &t) != CORAL_OK || idx->plan.slots_log2 == had) {
             idx->bump_log2 -= 1;  // no room in LDS for more: stay
             if (!idx->prepared) return fail(CORAL_ERR_DEVICE, "could not restore the search scratch");
         }

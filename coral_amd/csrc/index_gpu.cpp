@@ -45,11 +45,18 @@ bool json_number(const std::string& text, const char* key, double* out) {
 
 ProConfig& GetProConfig() { return g_config; }
 
-IndexGPU::IndexGPU(const size_t dimension, const size_t n, Metric m, void* initializer)
-    : dimension_(dimension), nd_(n), metric_enum_(m) {
-    (void)initializer;
+// src/index.cpp:9-29 without the host-side Distance object and its message
+Index::Index(const size_t dimension, const size_t n, Metric metric) : dimension_(dimension), nd_(n), metric_(metric) {}
+Index::~Index() {}
+
+IndexGPU::IndexGPU(const size_t dimension, const size_t n, Metric m, Index* initializer)
+    : Index(dimension, n, m), initializer_(initializer), row_width_((dimension + 3) / 4 * 4) {
     if (m == COSINE) need_normalize = true;
 }
+
+// empty in the reference as well (src/index_gpu.cpp:652-654)
+void IndexGPU::Build(size_t, const float*, const Parameters&) {}
+void IndexGPU::Search(const float*, const float*, size_t, const Parameters&, unsigned*, float*) {}
 
 IndexGPU::~IndexGPU() { RunFree(); }
 
@@ -58,6 +65,7 @@ void IndexGPU::RunFree() {
     index_ = nullptr;
     std::free(h_base_);
     h_base_ = nullptr;
+    data_bp_ = nullptr;
 }
 
 void IndexGPU::load_config(const std::string& config_file) {
@@ -98,7 +106,7 @@ void IndexGPU::LoadSearchNeededData(const char* base_file, const char* sampled_q
     // rows are padded with zeros to a multiple of 4 floats (include/efanna2e/util.h:194-208);
     // unlike the reference the padded width is then used consistently
     const int32_t stride = (dim + 3) / 4 * 4;
-    if ((size_t)stride != ((dimension_ + 3) / 4 * 4))
+    if ((size_t)stride != row_width_)
         throw std::runtime_error("base dimension does not match the index dimension");
     std::free(h_base_);
     h_base_ = nullptr;
@@ -106,9 +114,9 @@ void IndexGPU::LoadSearchNeededData(const char* base_file, const char* sampled_q
         throw std::runtime_error("out of host memory for the base vectors");
     if (coral_fbin_read(base_file, h_base_, n, dim, stride)) raise("load_data");
     if (m == DIST_METRIC::IP_) coral_normalize_l2(h_base_, n, stride);
-    dimension_ = (size_t)stride;
     nd_ = (size_t)n;
-    metric_ = m;
+    data_bp_ = h_base_;
+    dist_metric_ = m;
 }
 
 void IndexGPU::RunPrepare(Parameters& parameters, Mode mode, size_t n_bp, float* bp_data) {
@@ -120,14 +128,15 @@ void IndexGPU::RunPrepare(Parameters& parameters, Mode mode, size_t n_bp, float*
     graph_dir_ = parameters.Get<std::string>("graph_file");
     k_ = parameters.Get<int>("k");
     max_degree_ = parameters.Get<int>("max_degree");
-    metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
-    if (n_bp > 0) {  // caller-owned vectors (src/index_gpu.cpp:246-251); copied, rows dimension_ wide
+    dist_metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
+    if (n_bp > 0) {  // caller-owned vectors (src/index_gpu.cpp:246-251); copied, rows GetRowWidth() wide
         std::free(h_base_);
         h_base_ = nullptr;
-        if (posix_memalign((void**)&h_base_, 32, n_bp * dimension_ * sizeof(float)) != 0)
+        if (posix_memalign((void**)&h_base_, 32, n_bp * row_width_ * sizeof(float)) != 0)
             throw std::runtime_error("out of host memory for the base vectors");
-        std::memcpy(h_base_, bp_data, n_bp * dimension_ * sizeof(float));
+        std::memcpy(h_base_, bp_data, n_bp * row_width_ * sizeof(float));
         nd_ = n_bp;
+        data_bp_ = h_base_;
     }
     if (!h_base_) throw std::runtime_error("RunPrepare before LoadSearchNeededData");
     nbrs_.assign(nd_ * (size_t)max_degree_, -1);
@@ -141,9 +150,9 @@ void IndexGPU::RunPrepare(Parameters& parameters, Mode mode, size_t n_bp, float*
     if (start_ids_.empty()) throw std::runtime_error("graph.search_start_ids is missing or empty in " + graph_dir_);
     coral_index_desc d;
     std::memset(&d, 0, sizeof d);
-    d.base = h_base_, d.nbrs = nbrs_.data(), d.n = (int64_t)nd_, d.dim = (int32_t)dimension_;
+    d.base = h_base_, d.nbrs = nbrs_.data(), d.n = (int64_t)nd_, d.dim = (int32_t)row_width_;
     d.R = max_degree_, d.start_ids = start_ids_.data(), d.n_start = (int32_t)start_ids_.size();
-    d.metric = metric_ == DIST_METRIC::L2_ ? CORAL_L2 : CORAL_IP, d.device = 0;
+    d.metric = dist_metric_ == DIST_METRIC::L2_ ? CORAL_L2 : CORAL_IP, d.device = 0;
     if (index_) coral_index_destroy(index_);
     index_ = nullptr;
     if (coral_index_create(&d, &index_)) raise("create index");
@@ -156,21 +165,22 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     if (CE < 0 || CE > 2) throw std::runtime_error("BuildGPU: CE must be 0 (none), 1 (after the build) or 2 (only)");
     max_degree_ = parameters.Get<int>("max_degree");
     k_ = parameters.Get<int>("k");
-    metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
+    dist_metric_ = parameters.Get<std::string>("dist") == "l2" ? DIST_METRIC::L2_ : DIST_METRIC::IP_;
     graph_dir_ = parameters.Get<std::string>("graph_file");
     if (!bp_data || n_bp == 0) throw std::runtime_error("BuildGPU: empty input");
     if (bp_data != h_base_) {  // keep a copy, like RunPrepare does with caller-owned vectors
         std::free(h_base_);
         h_base_ = nullptr;
-        if (posix_memalign((void**)&h_base_, 32, n_bp * dimension_ * sizeof(float)) != 0)
+        if (posix_memalign((void**)&h_base_, 32, n_bp * row_width_ * sizeof(float)) != 0)
             throw std::runtime_error("out of host memory for the base vectors");
-        std::memcpy(h_base_, bp_data, n_bp * dimension_ * sizeof(float));
+        std::memcpy(h_base_, bp_data, n_bp * row_width_ * sizeof(float));
+        data_bp_ = h_base_;
     }
     nd_ = n_bp;
     coral_index_desc d;
     std::memset(&d, 0, sizeof d);
-    d.base = h_base_, d.n = (int64_t)nd_, d.dim = (int32_t)dimension_;
-    d.metric = metric_ == DIST_METRIC::L2_ ? CORAL_L2 : CORAL_IP, d.device = 0;
+    d.base = h_base_, d.n = (int64_t)nd_, d.dim = (int32_t)row_width_;
+    d.metric = dist_metric_ == DIST_METRIC::L2_ ? CORAL_L2 : CORAL_IP, d.device = 0;
     if (index_) coral_index_destroy(index_);
     index_ = nullptr;
     if (coral_index_create(&d, &index_)) raise("create index");
@@ -269,7 +279,7 @@ Test_Result IndexGPU::Search_and_Verify(const float* queries, const int* gts, in
     const int L = beam_capacity > 0 ? beam_capacity : PC.test_beam_capacity;
     float* d_q = nullptr;
     int32_t *d_ids = nullptr, *d_gt = nullptr;
-    const size_t qb = (size_t)num * dimension_ * sizeof(float), ib = (size_t)num * k_ * sizeof(int32_t);
+    const size_t qb = (size_t)num * row_width_ * sizeof(float), ib = (size_t)num * k_ * sizeof(int32_t);
     auto release = [&]() {
         (void)hipFree(d_q);
         (void)hipFree(d_ids);

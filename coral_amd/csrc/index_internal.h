@@ -17,6 +17,19 @@
     } while (0)
 
 
+// Launch geometry of the workgroup-per-query search kernel for one beam capacity: what coral_search_prepare works
+// out and a search call hands to the kernel.
+struct coral_search_plan {
+    int L = 0;
+    bool big = false;         // beams in global memory (the kernel's BIG form)
+    int direct = 0;           // BIG only: the visited set is a bitmap of all ids in LDS
+    int slots_log2 = 0, table_words = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
+    int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0;
+    size_t lds_bytes = 0;
+    size_t spill_words = 0;   // words of one workgroup's overflow bitmap in global memory (0: never used)
+    size_t beam_stride = 0;   // 64-bit words of one workgroup's beam block in global memory (0 unless big)
+};
+
 struct coral_index {
     int device = 0;
     int64_t n = 0;
@@ -30,13 +43,12 @@ struct coral_index {
 
     // state of search_prepare
     bool prepared = false;
-    int Q = 0, L = 0;
-    int slots_log2 = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
-    int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0, prepared_policy = 0;
-    size_t lds_bytes = 0;
-    size_t spill_words = 0;
+    int Q = 0, L = 0, prepared_policy = 0;
+    coral_search_plan plan;
     uint32_t* d_spill = nullptr;
     size_t spill_alloc_words = 0;
+    uint64_t* d_beam = nullptr;  // beam blocks of a BIG launch, plan.workgroups x plan.beam_stride words
+    size_t beam_alloc_words = 0;
     int32_t* d_counters = nullptr;
     size_t counters_alloc = 0;
     int* d_scalars = nullptr;  // [0] next_qid, [1] spill_count

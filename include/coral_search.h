@@ -109,7 +109,8 @@ typedef struct {
                                    what outgrows it in HBM: log2 of the cells per query, 8..14; 0 = chosen from L
                                    where 8192 cells hold most of a query's visits (L <= 409 at up to 2^25 nodes),
                                    none otherwise; -1 = none */
-    int32_t reserved[1];
+    int32_t beam_in_hbm;        /* 1 = keep the beam in global memory whatever L is (the form beams longer than
+                                   CORAL_MAX_LDS_BEAM always take) */
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);
@@ -140,8 +141,12 @@ CORAL_API int coral_index_get_deleted(coral_index* idx, uint32_t* host_mask);
 CORAL_API int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* R,
                      int32_t* n_start, int32_t* metric);
 
-/* Largest beam capacity L: the beam lives in LDS (the reference keeps it in global memory and sets no limit). */
-#define CORAL_MAX_BEAM 2048
+/* Beam capacity L.  Up to CORAL_MAX_LDS_BEAM the beam lives in LDS; longer beams are kept per workgroup in global
+ * memory, as the reference keeps every beam (src/search.cu:400-402, include/gpufuncs.cuh:557-564), up to
+ * CORAL_MAX_BEAM.  The reference sets no limit; its driver grows L by 128 for at most 51 steps
+ * (tests/test_search_pipeline.cpp:278-313) and its config.json defaults to 1024. */
+#define CORAL_MAX_LDS_BEAM 2048
+#define CORAL_MAX_BEAM 65536
 
 /* GPUFuncs::search_prepare(Q, L) (src/search.cu:400-408): fixes the beam
  * capacity (1..CORAL_MAX_BEAM) and (re)allocates per-workgroup scratch. */

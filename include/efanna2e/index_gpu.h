@@ -13,7 +13,8 @@
 //     CPU or disk tier above 10.01M / 100M nodes (src/index_gpu.cpp:256-257).
 //     SetPolicy() chooses the traversal instead: ROUNDS (the reference's GPU
 //     kernel) by default, BEST_FIRST (its CPU path) on request;
-//   * build, insert and delete are not part of this library;
+//   * BuildGPU (all three --CE modes) and Delete in its tombstone-only mode are provided;
+//     Insert and the repair of rows after a deletion are not part of this library;
 //   * failures throw std::runtime_error with the library's message where the
 //     reference prints and exits (include/utils.cuh:50-58).
 #pragma once
@@ -23,13 +24,13 @@
 #include <vector>
 
 #include "../coral_search.h"
+#include "index.h"
 #include "parameters.h"
 
 enum DIST_METRIC { L2_, IP_, COS_ };  // include/uni.h:93
 
 namespace efanna2e {
 
-enum Metric { L2 = 0, INNER_PRODUCT = 1, FAST_L2 = 2, PQ = 3, COSINE = 4 };  // efanna2e/distance.h:15
 enum Mode { CONS, SEARCH, UPD, CE };                                          // include/uni.h:147
 enum GraphType { GPU, CPU, DISK };                                            // include/uni.h:149
 
@@ -78,13 +79,22 @@ class CORAL_API Test_Result {
     size_t expansions = 0, dist_evals = 0, rounds = 0, spills = 0;
 };
 
-class CORAL_API IndexGPU {
+class CORAL_API IndexGPU : public Index {
    public:
-    // `initializer` is kept for signature compatibility and must be nullptr
-    explicit IndexGPU(const size_t dimension, const size_t n, Metric m, void* initializer);
-    ~IndexGPU();
+    // include/index_gpu.h:46; `initializer` is stored and never used, as in the reference
+    // (src/index_gpu.cpp:26-27)
+    explicit IndexGPU(const size_t dimension, const size_t n, Metric m, Index* initializer);
+    virtual ~IndexGPU();
     IndexGPU(const IndexGPU&) = delete;
     IndexGPU& operator=(const IndexGPU&) = delete;
+    // the base class's interface; all four are empty in the reference too (include/index_gpu.h:48-49,
+    // src/index_gpu.cpp:652-654)
+    virtual void Save(const char*) override {}
+    virtual void Load(const char*) override {}
+    virtual void Build(size_t n, const float* data, const Parameters& parameters) override;
+    virtual void Search(const float* query, const float* x, size_t k, const Parameters& parameters,
+                        unsigned* indices, float* res_dists) override;
+    Index* initializer_;
 
     // src/index_gpu.cpp:625-650: reads base_file (.fbin), L2-normalises it for IP_
     void LoadSearchNeededData(const char* base_file, const char* sampled_query_file,
@@ -104,9 +114,10 @@ class CORAL_API IndexGPU {
     void LoadRoarGraph(std::string filename);
     // src/index_gpu.cpp:308-383: builds the graph over the n_bp base vectors from the n_sq auxiliary ("sampled")
     // queries and writes the index directory parameters["graph_file"] (graph.part*.idx/.data, graph.search_start_ids,
-    // graph.batch_id).  Reads config_file, CE (0 or 1; 2, "only CE", is not provided), max_degree, k (the cluster
+    // graph.batch_id).  Reads config_file, CE (0, 1, or 2 = the enhancement alone on the rows, distances and
+    // hits.bin that a CE = 0 build left in graph_file, src/index_gpu.cpp:332-333, 367-373), max_degree, k (the cluster
     // size), dist, graph_file, train_gt_file (optional: the clusters, as a ground-truth file of the sampled queries with k
-    // ids per row; sq_data is then unused).  Both arrays hold rows of GetDimension() floats.  The built index stays loaded, so
+    // ids per row; sq_data is then unused).  Both arrays hold rows of GetRowWidth() floats.  The built index stays loaded, so
     // Search works right after.  The timings and counts of the run are in last_build.
     void BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data, Parameters& parameters);
     coral_build_stats last_build{};
@@ -130,18 +141,17 @@ class CORAL_API IndexGPU {
     Test_Result SearchWithDists(const float* queries, int num, int beam_capacity, int* ids_res,
                                 float* dists_res);
 
-    Metric GetMetric() const { return metric_enum_; }
-    size_t GetDimension() const { return dimension_; }
-    size_t GetSizeOfDataset() const { return nd_; }
-    const float* GetBasePointSet() const { return h_base_; }
+    Metric GetMetric() const { return metric_; }
+    // floats per vector row as the library holds them: the dimension padded to a multiple of 4 with zeros, which
+    // is what the reference's loaders hand to the constructor in the first place (include/efanna2e/util.h:194-208)
+    size_t GetRowWidth() const { return row_width_; }
     const std::vector<int>& GetStartIds() const { return start_ids_; }
     bool need_normalize = false;
 
    private:
     Test_Result run(const float* queries, int num, int L, int* ids_res, float* dists_res);
-    size_t dimension_, nd_;
-    Metric metric_enum_;
-    DIST_METRIC metric_ = DIST_METRIC::L2_;
+    size_t row_width_;
+    DIST_METRIC dist_metric_ = DIST_METRIC::L2_;
     Parameters parameters_;
     int k_ = 0, max_degree_ = 32;
     int policy_ = -1;  // -1: by size, see GetPolicy

@@ -4,8 +4,9 @@ tiny inputs.  Distances are supplied by the caller so that only the traversal
 logic is under test."""
 
 
-def policy_rounds(nbrs, starts, dist, L, k, deleted=frozenset()):
-    """dist: dict id -> signed distance (smaller is closer).  Returns (ids, hops, expansions, evals)."""
+def policy_rounds(nbrs, starts, dist, L, k, deleted=frozenset(), trace=None):
+    """dist: dict id -> signed distance (smaller is closer).  Returns (ids, hops, expansions, evals).
+    trace (a list) receives, per round, (ids expanded in the round, ids in the beam after its merge)."""
     visited = set(starts)
     beam = {s: False for s in starts}  # id -> expanded
     evals = len(starts)
@@ -13,7 +14,8 @@ def policy_rounds(nbrs, starts, dist, L, k, deleted=frozenset()):
     hops = expansions = 0
     while True:
         cand = []
-        for v in [v for v, ex in beam.items() if not ex]:
+        todo = [v for v, ex in beam.items() if not ex]
+        for v in todo:
             beam[v] = True
             expansions += 1
             for w in nbrs[v]:
@@ -35,12 +37,15 @@ def policy_rounds(nbrs, starts, dist, L, k, deleted=frozenset()):
             keep = sorted(beam, key=lambda v: (dist[v], v))[:L]
             beam = {v: beam[v] for v in keep}
             thr = dist[keep[-1]]
+        if trace is not None:
+            trace.append((frozenset(todo), frozenset(beam)))
     order = sorted(beam, key=lambda v: (dist[v], v))
     live = [v for v in order if v not in deleted][:k]
     return live + [-1] * (k - len(live)), hops, expansions, evals
 
 
-def policy_best_first(nbrs, starts, dist, L, k, deleted=frozenset()):
+def policy_best_first(nbrs, starts, dist, L, k, deleted=frozenset(), trace=None):
+    """trace (a list) receives, per step, (the id expanded, ids in the beam after the step's inserts)."""
     visited = set()
     beam = {}
     evals = 0
@@ -76,6 +81,8 @@ def policy_best_first(nbrs, starts, dist, L, k, deleted=frozenset()):
             evals += 1
             insert(w)
             visited.add(w)
+        if trace is not None:
+            trace.append((frozenset([v]), frozenset(beam)))
     order = sorted(beam, key=lambda v: (dist[v], v))
     live = [v for v in order if v not in deleted][:k]
     return live + [-1] * (k - len(live)), hops, expansions, evals

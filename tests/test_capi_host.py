@@ -39,8 +39,94 @@ def test_cxx_class_symbols_are_exported():
                 "efanna2e::IndexGPU::RunPrepare(efanna2e::Parameters&, efanna2e::Mode, unsigned long, float*)",
                 "efanna2e::IndexGPU::LoadSearchNeededData(char const*, char const*, DIST_METRIC)",
                 "efanna2e::IndexGPU::LoadRoarGraph(", "efanna2e::IndexGPU::load_config(",
-                "efanna2e::IndexGPU::RunFree()", "efanna2e::GetProConfig()"):
+                "efanna2e::IndexGPU::RunFree()", "efanna2e::GetProConfig()",
+                # the reference's class hierarchy (include/efanna2e/index.h:20-40, include/index_gpu.h:42-46)
+                "efanna2e::IndexGPU::IndexGPU(unsigned long, unsigned long, efanna2e::Metric, efanna2e::Index*)",
+                "efanna2e::Index::Index(unsigned long, unsigned long, efanna2e::Metric)",
+                "vtable for efanna2e::Index", "vtable for efanna2e::IndexGPU", "typeinfo for efanna2e::Index",
+                "efanna2e::IndexGPU::BuildGPU(unsigned long, float*, unsigned long, float*, efanna2e::Parameters&)",
+                "efanna2e::IndexGPU::Delete(std::vector<int, std::allocator<int> >)"):
         assert sym in out, sym
+
+
+CALLER = r"""
+// A caller in the shape of the reference's search driver (tests/test_search_pipeline.cpp:241-292) and of code that
+// holds the index through its base class (include/efanna2e/index.h:20-64).
+#include <cstring>
+#include <iostream>
+#include <string>
+#include <vector>
+#include "efanna2e/index.h"
+#include "efanna2e/index_gpu.h"
+#include "efanna2e/parameters.h"
+
+using namespace efanna2e;  // as the reference's driver does (tests/test_search_pipeline.cpp:23)
+
+static float run(efanna2e::Index* base_ptr, const std::vector<float>& queries, int q_pts, int k,
+                 std::vector<int> L_vec, const std::string& index_type) {
+    efanna2e::IndexGPU& index = *static_cast<efanna2e::IndexGPU*>(base_ptr);
+    int* res = new int[(size_t)q_pts * k];
+    std::memset(res, 0, sizeof(int) * (size_t)q_pts * k);
+    float last = 0.f;
+    for (size_t i = 0; i < L_vec.size(); ++i) {
+        int L = L_vec[i];
+        auto tr = index_type == "" ? index.Search(queries.data(), q_pts, L, res)
+                                   : index.Search(queries.data(), q_pts, L, res, 1);
+        const float qps = (float)q_pts / tr.get_time(), time = tr.get_time();
+        const float avg_hops = tr.avg_hops(q_pts);
+        std::cout << L << "		" << qps << "		" << time << "		" << avg_hops << std::endl;
+        last = qps;
+    }
+    delete[] res;
+    return last;
+}
+
+int main(int argc, char** argv) {
+    efanna2e::Metric dist_metric = efanna2e::INNER_PRODUCT;
+    DIST_METRIC metric = DIST_METRIC::IP_;
+    size_t q_dim = 200, base_num = 0, sq_num = 0;
+    efanna2e::Parameters parameters;
+    parameters.Set<std::string>("config_file", "default");
+    parameters.Set<std::string>("graph_file", "../indexes/x_ip_32_1.0_1/");
+    parameters.Set<int>("k", 100);
+    parameters.Set<int>("max_degree", 32);
+    parameters.Set<std::string>("dist", "ip");
+    efanna2e::IndexGPU index(q_dim, base_num + sq_num, dist_metric, nullptr);
+    efanna2e::Index* as_base = &index;                       // IndexGPU is an Index
+    efanna2e::IndexGPU second(q_dim, 0, efanna2e::L2, as_base);  // ... and takes one as its initializer
+    if (argc > 100) {  // never run: this file is compiled and linked, not executed
+        index.LoadSearchNeededData(argv[1], argv[2], metric);
+        index.RunPrepare(parameters, Mode::SEARCH);
+        index.LoadRoarGraph(std::string("../data/") + argv[3] + "/indexes/roar.index");
+        std::vector<float> q(q_dim);
+        run(as_base, q, 1, 100, {256, 512}, "");
+        Test_Result tr = index.Search_and_Verify(q.data(), nullptr, 1, 256);
+        tr.calc_recall(100);
+        as_base->Save("x");
+        as_base->Load("x");
+        as_base->Build(0, nullptr, parameters);
+        as_base->Search(nullptr, nullptr, 0, parameters, nullptr, nullptr);
+        index.RunFree();
+    }
+    return (int)(as_base->GetDimension() - q_dim) + (second.initializer_ == as_base ? 0 : 1) +
+           (as_base->HasBuilt() ? 1 : 0) + (int)as_base->GetSizeOfDataset();
+}
+"""
+
+
+def test_a_caller_written_against_the_reference_class_compiles_and_links(tmp_path):
+    """The fragment of the reference's driver that constructs, loads, prepares and searches the index, and a use of
+    the index through its abstract base, compile against include/efanna2e/*.h and link against the library (the
+    program constructs two indexes, touches no device and exits 0)."""
+    src = tmp_path / "caller.cpp"
+    src.write_text(CALLER)
+    exe = tmp_path / "caller"
+    libdir = os.path.dirname(capi.LIB_PATH)
+    r = subprocess.run(["g++", "-std=c++17", "-Wall", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                        "-L" + libdir, "-lcoral_search", "-Wl,-rpath," + libdir], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
 
 
 def test_index_create_validates_before_any_device_call():

@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 
 from coral_amd import capi, formats, synth
-from util import make_queries, near_tie_equal, ragged, rounds_hand_case
+from util import explain_divergence, make_queries, near_tie_equal, ragged, rounds_hand_case
 
 pytestmark = pytest.mark.gpu
 
@@ -102,6 +102,77 @@ def test_exact_against_same_order_oracle(orc, case):
     idx.close()
 
 
+BIG_CASES = [
+    # n, dim, R, metric, policy, L, k, M, ragged, slots_log2 (0: the library's choice, a bitmap of all ids in LDS at
+    # these sizes; else the table of cells that size with the overflow bitmap in global memory), workgroups, tombstones
+    (20000, 200, 32, "l2", 0, 4096, 100, 16, None, 0, 0, False),
+    (20000, 200, 32, "l2", 0, 6656, 100, 16, None, 0, 0, False),   # the reference driver's last step (128 * 52)
+    (20000, 200, 32, "l2", 1, 4096, 100, 16, None, 0, 0, False),
+    (20000, 200, 32, "l2", 1, 6656, 1000, 16, 9, 0, 0, True),
+    (30000, 128, 32, "l2", 0, 20000, 5000, 16, None, 0, 7, False),  # queries reuse a workgroup's beam block
+    (12000, 512, 24, "ip", 0, 3000, 100, 8, 5, 0, 5, True),
+    (12000, 64, 32, "l2", 0, 2500, 2500, 100, None, 12, 3, False),  # table of cells + overflow bitmap
+    (12000, 64, 32, "l2", 1, 2500, 17, 1, 3, 11, 3, True),
+    (3000, 200, 32, "l2", 0, 4000, 3500, 16, None, 0, 0, False),    # a beam longer than the graph
+    (3000, 200, 16, "ip", 1, 65536, 3000, 4, 21, 0, 0, False),      # the longest beam the library takes
+    (20000, 200, 32, "l2", 0, 256, 100, 16, None, 0, 0, False),     # short beams kept in global memory on request
+    (20000, 200, 32, "l2", 1, 64, 10, 16, None, 10, 2, False),
+]
+
+
+@pytest.mark.parametrize("case", BIG_CASES, ids=lambda c: "n%d_d%d_R%d_%s_p%d_L%d_k%d_M%d_rg%s_s%d_w%d_del%d" % c)
+def test_beams_in_global_memory_equal_the_oracle(orc, case):
+    """Beams beyond CORAL_MAX_LDS_BEAM (the reference sets no limit on L, src/search.cu:400-408; its driver grows L
+    to 128 * 52): the beam buffers live in global memory, the visited set is a bitmap of all ids in LDS or the table
+    of cells with its overflow bitmap.  Everything stays integer-exact against the oracle in the kernel's order."""
+    n, dim, R, metric, policy, L, k, M, rg, slots, wgs, dele = case
+    m = capi.IP if metric == "ip" else capi.L2
+    base, nbrs, starts = problem(n, dim, R, seed=dim + L % 1000, metric=metric, n_start=M, ragged_seed=rg,
+                                 isolate=5 if rg else 0)
+    Q = 40 if L >= 20000 else 120
+    q = make_queries(Q, dim, 700 + dim, metric)
+    mask = synth.tombstone_mask(n, 31 + L, modulo=3) if dele else None
+    print("case", case, flush=True)
+    prob = orc.Problem(base, nbrs, starts, mask)
+    if policy == 0:
+        oi, od, os_, _ = orc.search_B(prob, q, k, L, metric=m, start_order=WAVE64, nbr_order=WAVE64)
+    else:
+        oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=m, order=WAVE64)
+    idx = capi.Index(base, nbrs, starts, m)
+    if dele:
+        idx.set_deleted(mask)
+    idx.prepare(Q, L, visited_slots_log2=slots, workgroups=wgs, policy=policy, beam_in_hbm=True)
+    ids, dists, st = idx.search(q, k, L, policy=policy, have_delete=dele)
+    cnt = idx.query_counters(Q)
+    assert np.array_equal(ids, oi)
+    assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist()
+    assert np.array_equal(cnt, os_)
+    if slots:
+        assert st.spills > 0
+    # the same call again on the workgroups' used beam blocks and bitmaps
+    ids2, dists2, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
+    assert np.array_equal(ids2, oi) and dists2.tobytes() == od.tobytes()
+    if L <= capi.MAX_LDS_BEAM:  # and the form with the beam in LDS agrees
+        idx.prepare(Q, L, policy=policy, best_first_in_lds=True)
+        ids3, dists3, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
+        assert np.array_equal(ids3, oi) and dists3.tobytes() == od.tobytes()
+    idx.close()
+
+
+def test_beam_capacity_limits():
+    base, nbrs, starts, q, L, k, want = rounds_hand_case()
+    idx = capi.Index(base, nbrs, starts, capi.L2)
+    for bad in (0, -3, capi.MAX_BEAM + 1):
+        with pytest.raises(capi.CoralError) as e:
+            idx.prepare(1, bad)
+        assert e.value.code == capi.ERR_ARG
+    ids, dists, _ = idx.search(q, k, capi.MAX_BEAM)  # eleven nodes under the longest beam: all of them, in order
+    assert ids[0].tolist() == want["ids"]
+    ids, dists, _ = idx.search(q, 11, capi.MAX_BEAM)
+    assert sorted(ids[0].tolist()) == list(range(11)) and (np.diff(dists[0]) >= 0).all()
+    idx.close()
+
+
 def test_hand_computed_traversals_through_the_c_abi():
     """The traversal worked out by hand in util.rounds_hand_case, with no oracle in between: ids, distances and all
     four counters of the rounds policy (each rule of the policy decides one of them), and the best-first answer on
@@ -153,8 +224,11 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         dele, dup = rng.rand() < 0.35, rng.rand() < 0.3
         wgs = int(rng.choice([0, 0, 1, 2, 7]))
         tbl = int(rng.choice([0, 0, -1, 8, 9, 10, 12]))
+        big = rng.rand() < 0.25  # the beam in global memory, at up to eight times the length drawn above
+        if big:
+            L = min(n, L * int(rng.choice([1, 3, 8])))
         print("case", dict(c=c, n=n, dim=dim, R=R, metric=metric, policy=policy, L=L, k=k, M=M, Q=Q, slots=slots,
-                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl), flush=True)
+                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl, big=big), flush=True)
         m = capi.IP if metric == "ip" else capi.L2
         base = synth.gaussian_matrix(1000 + c, n, dim)
         if metric == "ip":
@@ -179,7 +253,8 @@ def test_randomised_search_problems_equal_the_oracle(orc):
             idx.set_deleted(mask)
         for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
             idx.prepare(Q, L, visited_slots_log2=slots, threads=threads, workgroups=wgs, policy=policy,
-                        best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=tbl)
+                        best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=tbl,
+                        beam_in_hbm=big)
             ids, dists, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
             assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
             assert np.array_equal(idx.query_counters(Q), os_)
@@ -241,6 +316,12 @@ def test_best_first_query_slots_are_reused(orc):
     idx.close()
 
 
+# queries (of 400) whose answers may differ from the reference-order oracle's by more than near-tie swaps, per case:
+# what was observed, not a tolerance chosen in advance; each such query is explained in the test
+NEAR_TIE_BUDGET = {("l2", 0, 200, 256, 100): 4, ("l2", 0, 128, 64, 10): 4, ("ip", 0, 512, 256, 100): 4,
+                   ("l2", 1, 200, 128, 100): 4}
+
+
 @pytest.mark.parametrize("metric,policy,dim,L,k", [("l2", 0, 200, 256, 100), ("l2", 0, 128, 64, 10),
                                                    ("ip", 0, 512, 256, 100), ("l2", 1, 200, 128, 100)])
 def test_tolerance_against_reference_order_oracle(orc, metric, policy, dim, L, k):
@@ -262,11 +343,19 @@ def test_tolerance_against_reference_order_oracle(orc, metric, policy, dim, L, k
     same = ids == oi
     rel = np.abs(dists - od) / np.maximum(np.abs(od), 1e-30)
     assert rel[same].max() <= 1e-5
-    # id lists: identical up to near-tie swaps for (almost) every query; a near-tie that
-    # decides membership of the beam's last slot can change what gets expanded next, which
-    # the 1e-6 rule does not cover; such queries must stay below 1 %
-    ok = sum(near_tie_equal(ids[i], dists[i], oi[i], od[i]) for i in range(Q))
-    assert ok >= 0.99 * Q, ok
+    # id lists: identical up to near-tie swaps.  A near-tie inside the traversal -- two nodes within 1e-6 of each
+    # other that the two summation orders rank in opposite ways, at the beam's last slot or as the next entry to
+    # expand -- sends the search on from a different node, and the lists that come out can then differ by more than a
+    # swap.  Such queries are counted, and each is replayed step by step in both orders to show that it parted at
+    # exactly such a pair and at nothing else.
+    bad = [i for i in range(Q) if not near_tie_equal(ids[i], dists[i], oi[i], od[i])]
+    print("queries beyond the near-tie rule: %d of %d %s" % (len(bad), Q, bad), flush=True)
+    assert len(bad) <= NEAR_TIE_BUDGET[(metric, policy, dim, L, k)]
+    for i in bad[:6]:
+        why = explain_divergence(orc, base, nbrs, starts, q[i], m, policy, L, k)
+        print("query %d parts at step %s: %s" % (i, why and why[0], why and why[1]), flush=True)
+        assert why is not None
+        assert all(gap < 1e-6 for _, _, gap in why[1]), why
     gt, _ = orc.bruteforce(base, q, k, m)
     r_gpu = orc.recall_hits(ids, gt, k) / (Q * k)
     r_ref = orc.recall_hits(oi, gt, k) / (Q * k)
@@ -365,7 +454,7 @@ def test_call_order_and_range_errors():
         idx.search(q, 2, 8, have_delete=True)
     assert e.value.code == capi.ERR_STATE
     with pytest.raises(capi.CoralError):
-        idx.prepare(10, 4096)
+        idx.prepare(10, capi.MAX_BEAM + 1)
     idx.close()
 
 
@@ -447,11 +536,16 @@ def test_cli_end_to_end(orc, tmp_path):
     rows = table_rows(r.stdout)
     assert [int(f[0]) for f in rows] == [128 * (i + 1) for i in range(len(rows))]
     assert float(rows[-1][3]) >= 0.9 and all(float(f[3]) < 0.9 for f in rows[:-1])
-    # ... or until the beam capacity the library supports: a recall that cannot be met ends the run in good order
-    r = subprocess.run(grow + ["--max_recall", "1.01"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
+    # ... or for the reference's 52 steps, up to L = 6656 (tests/test_search_pipeline.cpp:305-312): a recall that
+    # cannot be met ends the run in good order, with the reference's message
+    r = subprocess.run(grow + ["--max_recall", "1.01"], cwd=work / "cwd", capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
-    assert [int(f[0]) for f in table_rows(r.stdout)] == list(range(128, 2048 + 1, 128))
-    assert "Beam capacity limit 2048 reached" in r.stdout
+    assert [int(f[0]) for f in table_rows(r.stdout)] == list(range(128, 6656 + 1, 128))
+    assert "Queue is too long, judged as unable to meet the recall requirement, termination" in r.stdout
+    big = table_rows(r.stdout)[-1]  # L = 6656: the beam in global memory, through the driver
+    oi, _, os_, _ = orc.search_B(prob, q, k, 6656, start_order=WAVE64, nbr_order=WAVE64)
+    assert abs(float(big[3]) - orc.recall_hits(oi, gt, k) / (Q * k)) < 1e-6
+    assert abs(float(big[4]) - os_[:, 0].sum() / Q) < 1e-4 * float(big[4])  # (printed with six digits)
 
 
 def test_randomised_shapes(orc):

@@ -95,3 +95,49 @@ def rounds_hand_case():
     q = np.zeros((1, 4), np.float32)
     expect = dict(ids=[10, 5, 4], dists=[1.0, 36.0, 49.0], hops=8, expansions=7, dist_evals=11, rounds=5)
     return base, nbrs, np.array([0], np.int32), q, 3, 3, expect
+
+
+def explain_divergence(orc, base, nbrs, starts, q1, metric, policy, L, k, rel=1e-6):
+    """Why do the kernel's summation order and the reference's lead one query to different answers?
+
+    Both traversals are replayed step by step (tests/pysim.py) on the distances of every node in the kernel's order
+    (ORDER_WAVE64) and in the reference's (policy 0: the warp tree for start ids and the one-thread chain for
+    neighbours; policy 1: the AVX-512 order).  Up to the first step at which they part the two have done the same
+    work on the same beam, so what they do differently there -- another entry expanded, or another entry kept at the
+    beam's boundary -- is a pair of nodes that the two orders rank in opposite ways.  Returns (step, pairs): pairs =
+    [(x, y, relative gap of their exact distances)], each x chosen by one order where the other chose y.  The
+    contract allows such swaps only for near-ties, gap < 1e-6; None when the traversals never part."""
+    import pysim
+    n = base.shape[0]
+    sign = -1.0 if metric == orc.IP else 1.0
+
+    def all_dists(order):
+        ids, d = orc.bruteforce(base, q1[None, :], n, metric, order=order)
+        out = np.empty(n, np.float64)
+        out[ids[0]] = sign * d[0].astype(np.float64)
+        return out
+
+    d_gpu = all_dists(orc.ORDER_WAVE64)
+    if policy == 0:
+        d_ref = all_dists(orc.ORDER_GPU_SEQ)
+        d_ref[starts] = all_dists(orc.ORDER_GPU_WARP32)[starts]
+    else:
+        d_ref = all_dists(orc.ORDER_CPU_AVX512)
+    exact = all_dists(-1)
+    sim = pysim.policy_rounds if policy == 0 else pysim.policy_best_first
+    rows = [[int(v) for v in r] for r in nbrs]
+    ta, tb = [], []
+    sim(rows, [int(s) for s in starts], d_gpu, L, k, trace=ta)
+    sim(rows, [int(s) for s in starts], d_ref, L, k, trace=tb)
+    for step, (a, b) in enumerate(zip(ta, tb)):
+        if a == b:
+            continue
+        # the expanded ids differ, or the beams do; either way the ids on one side only
+        only_a = (a[0] - b[0]) or (a[1] - b[1])
+        only_b = (b[0] - a[0]) or (b[1] - a[1])
+        pairs = []
+        for x in sorted(only_a):
+            y = min(only_b, key=lambda v: abs(exact[v] - exact[x]))
+            pairs.append((x, int(y), abs(exact[x] - exact[y]) / max(abs(exact[x]), 1e-30)))
+        return step, pairs
+    return None
