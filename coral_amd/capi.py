@@ -89,6 +89,8 @@ SIGNATURES = {
     "coral_search_prepare": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(Tuning)]),
     "coral_search_gpu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                    C.c_int32, C.c_int32, C.c_void_p, C.POINTER(Stats)]),
+    "coral_search_gpu_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                           C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_search_query_counters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
     "coral_search": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(Stats)]),
@@ -221,6 +223,13 @@ class Index:
         _check(lib().coral_search_gpu(self._h, d_queries, d_ids, d_dists, Q, k, policy, int(have_delete),
                                       stream, C.byref(st)))
         return st
+
+    def search_device_noalloc(self, d_queries, d_ids, d_dists, Q, k, L, policy=POLICY_ROUNDS, have_delete=False,
+                              stream=None):
+        """coral_search_gpu_noalloc: device pointers (ints), fixed scratch inside the library, no allocation, no
+        wait: synchronise the stream before reading the results."""
+        _check(lib().coral_search_gpu_noalloc(self._h, d_queries, d_ids, d_dists, Q, k, L, policy, int(have_delete),
+                                              stream))
 
     def query_counters(self, Q):
         out = np.empty((Q, 4), dtype=np.int32)

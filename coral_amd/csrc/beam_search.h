@@ -91,6 +91,17 @@ hipError_t search_kernel_prepare(int dim, bool big, size_t lds_bytes, int thread
 hipError_t launch_search(const SearchArgs& a, bool big, int workgroups, int threads, size_t lds_bytes,
                          hipStream_t stream);
 
+// A fixed block of device memory inside the library's code object (no allocation call ever made for it): the
+// scratch of the entry point that must not allocate.  Layout: 256 bytes of scalars, kStaticMaxQ x 4 per-query
+// counters, kStaticSpillWords words of per-workgroup overflow bitmaps.  static_scratch_init(device) looks the
+// block's address up once per device (that device must be current) and static_scratch(device) returns it, or
+// nullptr before that.
+constexpr int kStaticMaxQ = 16384;
+constexpr size_t kStaticSpillWords = (size_t)8 << 20;  // 32 MiB
+constexpr int64_t kStaticMaxN = (int64_t)1 << 22;      // leaves at least 64 workgroups a bitmap each
+constexpr size_t kStaticScratchBytes = 256 + (size_t)kStaticMaxQ * 16 + kStaticSpillWords * 4;
+hipError_t static_scratch_init(int device);
+void* static_scratch(int device);
 hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,
                          hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t stream);

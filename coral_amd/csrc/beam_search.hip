@@ -661,6 +661,33 @@ hipError_t launch_search(const SearchArgs& a, bool big, int workgroups, int thre
     return hipGetLastError();
 }
 
+// ---- the block of device memory for callers that must not allocate
+//
+// `scratch` lives in the code object; in host code its name is only a handle for hipGetSymbolAddress, never an
+// address a kernel could use.  Every device that loads the library holds its own copy at its own address.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];
+}  // namespace
+
+hipError_t static_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    if (__atomic_load_n(&g_scratch_ptr[device], __ATOMIC_ACQUIRE)) return hipSuccess;
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    __atomic_store_n(&g_scratch_ptr[device], p, __ATOMIC_RELEASE);  // (two racing threads store the same address)
+    return hipSuccess;
+}
+
+void* static_scratch(int device) {
+    if (device < 0 || device >= kMaxDevices) return nullptr;
+    return __atomic_load_n(&g_scratch_ptr[device], __ATOMIC_ACQUIRE);
+}
+
 hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,
                          hipStream_t stream) {
     hipLaunchKernelGGL(ids_verify_kernel, dim3(Q < 1024 ? Q : 1024), dim3(64), 0, stream, res, gt, hit,

@@ -151,6 +151,7 @@ int coral_index_create(const coral_index_desc* d, coral_index** out) {
     HIP_TRY_C(hipGetDeviceProperties(&prop, d->device));
     idx->num_cu = prop.multiProcessorCount;
     HIP_TRY_C(hipStreamCreate(&idx->stream));
+    HIP_TRY_C(coral::static_scratch_init(d->device));  // address of the fixed scratch block on this device
     const size_t vec_bytes = (size_t)d->n * d->dim * sizeof(float);
     const size_t nbr_bytes = vectors_only ? 0 : (size_t)d->n * d->R * sizeof(int32_t);
     HIP_TRY_C(hipMalloc(&idx->d_vec, vec_bytes));
@@ -580,6 +581,48 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         }
         stats->spills = scal[1];
     }
+    return CORAL_OK;
+}
+
+int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* d_ids, float* d_dists, int32_t Q,
+                             int32_t k, int32_t L, int32_t policy, int32_t have_delete, void* stream_) {
+    if (!idx || !d_queries || !d_ids) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
+    if (Q <= 0 || Q > coral::kStaticMaxQ)
+        return fail(CORAL_ERR_ARG, "Q=%d is outside 1..%d, the queries the fixed scratch block has counters for", Q,
+                    coral::kStaticMaxQ);
+    if (idx->n > coral::kStaticMaxN)
+        return fail(CORAL_ERR_ARG, "n=%lld exceeds %lld, the nodes the fixed scratch block has overflow bitmaps for",
+                    (long long)idx->n, (long long)coral::kStaticMaxN);
+    if (L <= 0 || L > CORAL_MAX_LDS_BEAM)
+        return fail(CORAL_ERR_ARG, "L=%d is outside 1..%d: longer beams need scratch in global memory", L,
+                    CORAL_MAX_LDS_BEAM);
+    if (k <= 0 || k > L) return fail(CORAL_ERR_ARG, "k=%d must be in 1..L=%d", k, L);
+    if (have_delete && !idx->d_deleted)
+        return fail(CORAL_ERR_STATE, "have_delete set but no tombstone mask was given");
+    HIP_TRY(hipSetDevice(idx->device));
+    unsigned char* base = static_cast<unsigned char*>(coral::static_scratch(idx->device));
+    if (!base) return fail(CORAL_ERR_STATE, "the fixed scratch block of device %d was not set up", idx->device);
+    hipStream_t stream = stream_ ? (hipStream_t)stream_ : idx->stream;
+    coral_tuning t;
+    std::memset(&t, 0, sizeof t);
+    t.policy = policy;  // both policies run on the workgroup-per-query kernel here
+    coral_search_plan plan;
+    if (int rc = plan_search(idx, Q, L, t, 0, &plan)) return rc;
+    // the block: 256 bytes of scalars, the per-query counters, then one overflow bitmap per workgroup
+    int* scal = reinterpret_cast<int*>(base);
+    int32_t* counters = reinterpret_cast<int32_t*>(base + 256);
+    uint32_t* spill = reinterpret_cast<uint32_t*>(base + 256 + (size_t)coral::kStaticMaxQ * 16);
+    const int wgs = (int)std::min<size_t>((size_t)std::min(plan.workgroups, (int)Q),
+                                          coral::kStaticSpillWords / plan.spill_words);
+    // the block keeps what the last call left: the work counter and the bitmaps must start at zero (fill kernels,
+    // which a caller may record into a graph)
+    HIP_TRY(coral::launch_fill_u32(reinterpret_cast<uint32_t*>(scal), 64, 0u, stream));
+    HIP_TRY(coral::launch_fill_u32(spill, plan.spill_words * (size_t)wgs, 0u, stream));
+    coral::SearchArgs a = search_args(idx, plan, d_queries, d_ids, d_dists, Q, k, policy, have_delete);
+    a.counters = counters, a.spill = spill, a.beam_scratch = nullptr;
+    a.next_qid = scal, a.spill_count = scal + 1;
+    HIP_TRY(coral::launch_search(a, false, wgs, plan.threads, plan.lds_bytes, stream));
     return CORAL_OK;
 }
 

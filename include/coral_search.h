@@ -160,6 +160,20 @@ CORAL_API int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t
                      int32_t Q, int32_t k, int32_t policy, int32_t have_delete, void* stream,
                      coral_stats* stats);
 
+/* coral_search_gpu for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference, whose search allocates on every call
+ * (src/index_gpu.cpp:120-124, src/search_gpu.cu:846-852).  No coral_search_prepare is needed and none of its
+ * scratch is used: the work counter, the per-query counters and the per-workgroup overflow bitmaps live in a fixed
+ * 32.3 MiB block of device memory inside the library's code object (each GPU that loads the library holds its
+ * copy until the process ends).  The call makes no allocation of any kind, records only kernels on `stream`
+ * (NULL = the index's own) and returns without waiting for them; both policies run on the workgroup-per-query
+ * kernel, with the results of coral_search_gpu bit for bit.  Limits (CORAL_ERR_ARG beyond them): Q <= 16384,
+ * n <= 4194304, L <= CORAL_MAX_LDS_BEAM.  Every call on a GPU shares that GPU's block: calls that overlap on one
+ * GPU (two streams, two indexes, two threads) race; order them. */
+CORAL_API int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* d_ids, float* d_dists,
+                                       int32_t Q, int32_t k, int32_t L, int32_t policy, int32_t have_delete,
+                                       void* stream);
+
 /* Per-query counters of the last coral_search_gpu call, int32 [Q][4] on the
  * host: hops, expansions, dist_evals, rounds. */
 CORAL_API int coral_search_query_counters(coral_index* idx, int32_t* host_out, int32_t Q);
