@@ -1,20 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the batched graph beam search on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-legs]
 
-Workload (the headline configuration): 1 000 000 x 200 fp32 base vectors N(0,I),
-10 000 queries from the shifted anisotropic law, degree-32 graph built from
-100 000 auxiliary queries, L2, k = 100, all queries in one batch, L in {256, 512}.
-One step = one search of the whole batch (one persistent kernel launch) with the
-index and the queries already resident in HBM.  The JSON line's `value` is
-queries per second at the L named in config.L; the other L is reported under
-"also".  `roofline` prices the search kernel's algorithmic bytes against the
-8 TB/s of HBM; `cpu_baseline` times the reference's CPU search on the host.
-"best_first" is the CPU path's traversal on the GPU, "exact_knn" the library's
-exhaustive search, "structured" the same path on data where recall@100 >= 0.90 exists.
+Workload (the headline configuration): 1 000 000 x 200 fp32 base vectors N(0,I), 10 000 queries from the shifted
+anisotropic law, degree-32 graph built from 100 000 auxiliary queries, L2, k = 100, all queries in one batch.
+
+The metric is QPS at recall@100 >= 0.90.  On this data (isotropic Gaussian, degree-32 graph) the beam that reaches
+that recall is long: the run finds the smallest beam capacity L (a multiple of 512) at which the batch's recall
+against exact ground truth is >= 0.90 for the reference GPU path's traversal (expand-all rounds), and `value` is the
+rate at that L.  One step = one search of the whole batch (one persistent kernel launch) with the index and the
+queries already resident in HBM.  The configuration's own L in {256, 512} are reported under "also" with their
+recall.  `roofline` prices the search kernel's algorithmic bytes against the 8 TB/s of HBM and, beside it, against
+what this GPU's memory delivers to a streaming read and to a random row gather; `cpu_baseline` times the reference's
+CPU search (best-first) on the host at the beam capacity where that traversal reaches the same recall.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -24,13 +26,16 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch seen by the memory-side counters (rocprofv3 --pmc FETCH_SIZE
-# and WRITE_SIZE, scaled by what the same counters read for a plain copy kernel);
-# measured offline (profiles/beam_search_kernel_1Mx200_L*.md; FETCH_SIZE reads half the bytes of a
-# 1 GiB copy on this GPU, so its factor is 2.0; WRITE_SIZE's is 1.0).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {256: 1.3825e+11, 512: 2.6955e+11}
-# the same for the best-first kernel at L = 512 (profiles/best_first_wave_kernel_1Mx200_L512.md)
-BEST_FIRST_TRAFFIC_BYTES = {512: 1.314e+11}
+RECALL_TARGET = 0.90
+L_STEP = 512
+# files whose text decides what the search kernels do; profiles/search_kernels_traffic.txt names their digest
+KERNEL_SOURCES = ("coral_amd/csrc/beam_search.hip", "coral_amd/csrc/beam_search.h", "coral_amd/csrc/best_first.hip",
+                  "coral_amd/csrc/search_device.h", "coral_amd/csrc/coral_search.cpp")
+T0 = time.time()
+
+
+def log(msg):
+    print("[bench %5.0fs] %s" % (time.time() - T0, msg), file=sys.stderr, flush=True)
 
 
 def algorithmic_bytes(expansions, dist_evals, Q, dim, k, R=32):
@@ -38,28 +43,244 @@ def algorithmic_bytes(expansions, dist_evals, Q, dim, k, R=32):
     return expansions * R * 4 + dist_evals * dim * 4 + Q * (dim * 4 + k * 8)
 
 
-def measure(idx, d_q, d_ids, d_gt, Q, k, dim, L, steps, warmup, policy):
-    """`steps` timed searches of the whole batch at beam capacity L (device buffers in and out)."""
-    import torch
-    idx.prepare(Q, L, policy=policy)
-    for _ in range(warmup):
-        idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k, policy=policy)
-    torch.cuda.synchronize()
-    t = time.perf_counter()
-    kernel_s, st = 0.0, None
-    for _ in range(steps):
-        st = idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k, policy=policy)
-        kernel_s += st.kernel_s
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t
-    hits = idx.verify(d_ids.data_ptr(), d_gt.data_ptr(), Q, k)
-    bytes_per_launch = algorithmic_bytes(st.expansions, st.dist_evals, Q, dim, k)
-    avg_kernel = kernel_s / steps
-    return {"L": L, "qps": steps * Q / wall, "ms_per_step": 1e3 * wall / steps,
-            "recall": hits / float(Q * k), "kernel_ms": 1e3 * avg_kernel,
-            "gbps": bytes_per_launch / avg_kernel / 1e9, "bytes_per_launch": bytes_per_launch,
-            "expansions_per_query": st.expansions / Q, "dist_evals_per_query": st.dist_evals / Q,
-            "hops_per_query": st.hops / Q, "rounds_per_query": st.rounds / Q, "spills": st.spills}
+def kernel_sources_digest():
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(kernel, L, policy):
+    """HBM bytes per launch from the rocprofv3 counter runs recorded in profiles/search_kernels_traffic.txt, or None
+    when there is no record for this launch or the kernel sources have changed since it was taken."""
+    path = os.path.join(ROOT, "profiles", "search_kernels_traffic.txt")
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return None
+    rec = {}
+    for ln in lines:
+        if ln.startswith("#") or ":" not in ln:
+            continue
+        key, val = ln.split(":", 1)
+        rec[key.strip()] = val.strip()
+    if rec.get("sources_sha256_16") != kernel_sources_digest():
+        return None
+    val = rec.get("%s %s L=%d" % (kernel, policy, L))
+    if not val:
+        return None
+    f = dict(p.split("=") for p in val.split())
+    return {"bytes": float(f["fetch_bytes"]) + float(f["write_bytes"]), "fetch_bytes": float(f["fetch_bytes"]),
+            "write_bytes": float(f["write_bytes"]), "commit": rec.get("commit"),
+            "source": "profiles/search_kernels_traffic.txt"}
+
+
+class Bench:
+    """One index resident in HBM with its queries, result buffer and ground truth on the device."""
+
+    def __init__(self, w):
+        import torch
+        from coral_amd import capi
+        self.torch, self.capi, self.w = torch, capi, w
+        self.k = w["k"]
+        self.queries = w["queries"]
+        self.Q, self.dim = self.queries.shape
+        m = capi.IP if w["metric"] == "ip" else capi.L2
+        self.idx = capi.Index(w["base"], w["nbrs"], w["starts"], m)
+        self.gt, _, self.gt_s = self.idx.bruteforce(self.queries, self.k, want_dists=False)
+        self.d_q = torch.from_numpy(self.queries).cuda()
+        self.d_ids = torch.empty((self.Q, self.k), dtype=torch.int32, device="cuda")
+        self.d_gt = torch.from_numpy(self.gt).cuda()
+
+    def close(self):
+        self.idx.close()
+
+    def measure(self, L, steps, warmup, policy, Q=None):
+        """`steps` timed searches of the first Q queries (default: the whole batch) at beam capacity L."""
+        torch, idx = self.torch, self.idx
+        Q = Q or self.Q
+        k, dim = self.k, self.dim
+        idx.prepare(Q, L, policy=policy)
+        for _ in range(warmup):
+            idx.search_device(self.d_q.data_ptr(), self.d_ids.data_ptr(), None, Q, k, policy=policy)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        kernel_s, st = 0.0, None
+        for _ in range(steps):
+            st = idx.search_device(self.d_q.data_ptr(), self.d_ids.data_ptr(), None, Q, k, policy=policy)
+            kernel_s += st.kernel_s  # HIP events on the stream the kernel runs on
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t
+        hits = idx.verify(self.d_ids.data_ptr(), self.d_gt.data_ptr(), Q, k)
+        bytes_per_launch = algorithmic_bytes(st.expansions, st.dist_evals, Q, dim, k)
+        avg_kernel = kernel_s / steps
+        return {"L": L, "queries": Q, "qps": steps * Q / wall, "ms_per_step": 1e3 * wall / steps,
+                "recall": hits / float(Q * k), "kernel_ms": 1e3 * avg_kernel,
+                "gbps": bytes_per_launch / avg_kernel / 1e9, "frac": bytes_per_launch / avg_kernel / 1e9 / HBM_PEAK_GBPS,
+                "bytes_per_launch": bytes_per_launch,
+                "expansions_per_query": st.expansions / Q, "dist_evals_per_query": st.dist_evals / Q,
+                "hops_per_query": st.hops / Q, "rounds_per_query": st.rounds / Q, "spills": st.spills}
+
+    def operating_point(self, policy, Q=None, first=512):
+        """The smallest multiple of L_STEP at which recall@k of the first Q queries reaches RECALL_TARGET: doubling
+        from `first`, then bisection between the last beam that fell short and the first that did not.  Returns
+        (L or None, [(L, recall, qps)] of every probe)."""
+        cap = min(self.capi.MAX_BEAM, max(L_STEP, self.idx.n // L_STEP * L_STEP))
+        probes = []
+
+        def probe(L):
+            r = self.measure(L, 1, 0, policy, Q)
+            probes.append((L, r["recall"], r["qps"]))
+            return r["recall"] >= RECALL_TARGET
+
+        lo, hi = None, max(first, (self.k + L_STEP - 1) // L_STEP * L_STEP)
+        while not probe(hi):
+            if hi >= cap:
+                return None, probes
+            lo, hi = hi, min(cap, hi * 2)
+        lo = lo if lo is not None else max(self.k, hi - L_STEP)
+        while hi - lo > L_STEP:
+            mid = (lo + hi) // 2 // L_STEP * L_STEP
+            if mid <= lo:
+                break
+            if probe(mid):
+                hi = mid
+            else:
+                lo = mid
+        return hi, probes
+
+
+def slim(r, keys=("L", "queries", "qps", "recall", "kernel_ms", "gbps", "frac", "dist_evals_per_query",
+                  "expansions_per_query", "spills")):
+    return {k2: r[k2] for k2 in keys if k2 in r}
+
+
+def cpu_reference(w, gt, L, k, budget_s=20.0, stride_first=False):
+    """The reference's CPU search (best-first, sorted queue, AVX-512 squared L2, OpenMP dynamic schedule over
+    queries; src/search_in_cpu.cpp:23-119) on this host's cores, on a bounded sample of the batch.  Uses oracle/_ref
+    (the reference's own queue and distance headers compiled in place) when it is present and the host has AVX-512,
+    otherwise the oracle's restatement."""
+    import oracle
+    prob = oracle.Problem(w["base"], w["nbrs"], w["starts"])
+    q = w["queries"]
+    threads = os.cpu_count() or 1
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    use_ref = oracle.ref() is not None and oracle.lib().oracle_have_avx512()
+    fn = oracle.ref_search_in_cpu if use_ref else oracle.search_A
+    # time a slice first, then as many queries as fit the budget
+    probe = min(4 * threads, q.shape[0])
+    _, _, _, t = fn(prob, q[:probe], k, L, nthreads=threads)
+    n = int(min(q.shape[0], max(probe, budget_s / max(t / probe, 1e-9))))
+    # a sample that falls short of half the budget is timed again (at most 9 passes in all) and the median pass is
+    # quoted: a single pass of under a second on a shared host varies by a third from run to run
+    times = []
+    while not times or (sum(times) < budget_s / 2 and len(times) < 9):
+        ids, _, stats, t = fn(prob, q[:n], k, L, nthreads=threads)
+        times.append(t)
+    t = sorted(times)[len(times) // 2]
+    hits = oracle.recall_hits(ids, gt[:n], k)
+    return {"value": n / t, "unit": "queries/s", "cores": threads, "kind": "reference" if use_ref else "port",
+            "sample": "first %d of %d queries, L=%d, k=%d, M=%d start ids, policy best-first; median of %d passes" %
+                      (n, q.shape[0], L, k, w["starts"].size, len(times)),
+            "L": L, "recall": hits / float(n * k), "time_s": t, "passes_s": [round(x, 4) for x in times],
+            "dist_evals_per_query": float(stats[:, 2].mean()),
+            "expansions_per_query": float(stats[:, 1].mean())}
+
+
+def cpu_operating_point(w, gt, k, start_L, cap):
+    """The smallest multiple of L_STEP at which the CPU reference's recall@k on a 128-query stride of the batch
+    reaches RECALL_TARGET (doubling, then bisection), and the recall it measured at every beam it tried."""
+    import numpy as np
+    import oracle
+    prob = oracle.Problem(w["base"], w["nbrs"], w["starts"])
+    q = w["queries"]
+    sub = np.arange(0, q.shape[0], max(1, q.shape[0] // 128))[:128]
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    use_ref = oracle.ref() is not None and oracle.lib().oracle_have_avx512()
+    fn = oracle.ref_search_in_cpu if use_ref else oracle.search_A
+    seen = []
+
+    def ok(L):
+        ids, _, stats, t = fn(prob, q[sub], k, L, nthreads=threads)
+        r = oracle.recall_hits(ids, gt[sub], k) / float(len(sub) * k)
+        seen.append({"L": L, "recall": r, "dist_evals_per_query": float(stats[:, 2].mean()), "time_s": t})
+        return r >= RECALL_TARGET
+
+    lo, hi = None, start_L
+    while not ok(hi):
+        if hi >= cap:
+            return None, seen
+        lo, hi = hi, min(cap, hi * 2)
+    lo = lo if lo is not None else max(k, hi // 2)
+    while hi - lo > L_STEP:
+        mid = (lo + hi) // 2 // L_STEP * L_STEP
+        if mid <= lo:
+            break
+        if ok(mid):
+            hi = mid
+        else:
+            lo = mid
+    return hi, seen
+
+
+# ------------------------------------------------------------------ legs beside the headline
+
+def control_leg(w, L, steps=2):
+    """The same index searched with queries drawn from the base's own law N(0, I): no shifted region that every
+    query funnels through, so the caches have less to give.  Same kernel, same L as the headline."""
+    import numpy as np
+    from coral_amd import capi, synth
+    w2 = dict(w)
+    w2["queries"] = synth.gaussian_matrix(2099, min(2000, w["queries"].shape[0]), w["queries"].shape[1])
+    b = Bench(w2)
+    out = {"queries": "N(0, I), %d" % w2["queries"].shape[0]}
+    for Lc in sorted({512, L}):
+        out["L=%d" % Lc] = slim(b.measure(Lc, steps, 1, capi.POLICY_ROUNDS))
+    b.close()
+    return out
+
+
+def config1_leg(with_cpu):
+    """Configuration 1 (the reference's CPU-runnable case): 100k x 128, exact 32-NN graph, k = 10, L = 64, M = 1."""
+    from coral_amd import capi, workloads
+    w = workloads.config1()
+    b = Bench(w)
+    out = {"workload": w["name"], "rounds": slim(b.measure(64, 5, 1, capi.POLICY_ROUNDS)),
+           "best_first": slim(b.measure(64, 5, 1, capi.POLICY_BEST_FIRST))}
+    if with_cpu:
+        out["cpu_reference"] = cpu_reference(w, b.gt, 64, w["k"], budget_s=4.0)
+        out["best_first_gpu_over_cpu"] = out["best_first"]["qps"] / out["cpu_reference"]["value"]
+    b.close()
+    return out
+
+
+def config3_leg():
+    """Configuration 3: inner product, 1M x 512 unit vectors, cone-gap queries, built graph, k = 100, L = 256."""
+    from coral_amd import capi, workloads
+    w = workloads.config3()
+    b = Bench(w)
+    out = {"workload": w["name"], "graph_total_s": w["build"]["total_s"],
+           "rounds": slim(b.measure(256, 5, 1, capi.POLICY_ROUNDS))}
+    b.close()
+    return out
+
+
+def config4_leg():
+    """Configuration 4: 10M x 200, built graph, k = 100, L = 256, batches of 1 000 / 10 000 / 100 000 queries."""
+    from coral_amd import capi, synth, workloads
+    n, dim = 10 ** 7, 200
+    base = workloads.gaussian_base(4001, n, dim)
+    aux = synth.shifted_queries(100000, dim, 2002, 2003, 2005)
+    nbrs, starts, info = workloads.build_query_aware_graph(base, aux, "l2")
+    w = dict(name="10000000x200 fp32 L2, R=32 query-aware graph, k=100, L=256", base=base, nbrs=nbrs, starts=starts,
+             metric="l2", k=100, queries=synth.shifted_queries(100000, dim, 2002, 2003, 2004))
+    b = Bench(w)
+    out = {"workload": w["name"], "graph_total_s": info["total_s"], "ground_truth_s": b.gt_s, "rounds": []}
+    for Q in (1000, 10000, 100000):
+        out["rounds"].append(slim(b.measure(256, 3, 1, capi.POLICY_ROUNDS, Q=Q)))
+    b.close()
+    return out
 
 
 def shipped_config_leg(w):
@@ -67,54 +288,41 @@ def shipped_config_leg(w):
     the most-hit nodes through a second search-and-rewire pass after the isolated ones (src/enhance.cu:819-856); the
     headline graph is built with the code's default (0, src/index_gpu.cpp:78).  With n = 1M the reference reads past
     its id array for that value; here the pass covers at most all n nodes."""
-    import torch
     from coral_amd import capi, workloads
-    base, queries, k = w["base"], w["queries"], w["k"]
-    Q, dim = queries.shape
-    nbrs, starts, info = workloads.build_query_aware_graph(base, w["aux"], "l2", top_hit_num=5000000)
-    idx = capi.Index(base, nbrs, starts, capi.L2)
-    gt, _, _ = idx.bruteforce(queries, k, want_dists=False)
-    d_q = torch.from_numpy(queries).cuda()
-    d_ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
-    d_gt = torch.from_numpy(gt).cuda()
+    nbrs, starts, info = workloads.build_query_aware_graph(w["base"], w["aux"], "l2", top_hit_num=5000000)
+    w2 = dict(w, nbrs=nbrs, starts=starts)
+    b = Bench(w2)
     out = {"graph": info}
-    for name, policy, Ls in (("rounds", capi.POLICY_ROUNDS, (256, 512)), ("best_first", capi.POLICY_BEST_FIRST, (512,))):
-        rows = [measure(idx, d_q, d_ids, d_gt, Q, k, dim, L, 3, 1, policy) for L in Ls]
-        out[name] = [{"L": r["L"], "qps": r["qps"], "recall": r["recall"], "frac": r["gbps"] / HBM_PEAK_GBPS,
-                      "dist_evals_per_query": r["dist_evals_per_query"]} for r in rows]
-    idx.close()
+    L, probes = b.operating_point(capi.POLICY_ROUNDS)
+    out["probes"] = [{"L": p[0], "recall": p[1]} for p in probes]
+    if L:
+        out["rounds_at_recall_0.90"] = slim(b.measure(L, 3, 1, capi.POLICY_ROUNDS))
+    out["rounds"] = [slim(b.measure(Lx, 3, 1, capi.POLICY_ROUNDS)) for Lx in (256, 512)]
+    b.close()
     return out
 
 
 def structured_leg(with_cpu=True):
     """The same path on data that has neighbourhood structure (workloads.structured: 1M x 200 near a 16-dimensional
-    subspace, same construction, same k): recall@100 >= 0.90 exists there, and the line reports the best rate at or
-    above it for each policy, with the reference's CPU search at the beam capacity that gets its traversal
+    subspace, same construction, same k), where recall@100 >= 0.90 needs a beam of a few hundred: the best rate at
+    or above it for each policy, with the reference's CPU search at the beam capacity that gets its traversal
     (best-first) there.  Beside the headline, never the headline."""
-    import torch
     from coral_amd import capi, workloads
     w = workloads.structured()
-    queries, k = w["queries"], w["k"]
-    Q, dim = queries.shape
-    idx = capi.Index(w["base"], w["nbrs"], w["starts"], capi.L2)
-    gt, _, _ = idx.bruteforce(queries, k, want_dists=False)
-    d_q = torch.from_numpy(queries).cuda()
-    d_ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
-    d_gt = torch.from_numpy(gt).cuda()
+    b = Bench(w)
     out = {"workload": w["name"], "graph_total_s": w["build"]["total_s"]}
     for name, policy, Ls in (("rounds", capi.POLICY_ROUNDS, (128, 144, 160, 192, 256)),
                              ("best_first", capi.POLICY_BEST_FIRST, (256, 288, 320, 384, 512))):
-        rows = [measure(idx, d_q, d_ids, d_gt, Q, k, dim, L, 3, 1, policy) for L in Ls]
-        out[name] = [{"L": r["L"], "qps": r["qps"], "recall": r["recall"], "frac": r["gbps"] / HBM_PEAK_GBPS,
-                      "dist_evals_per_query": r["dist_evals_per_query"]} for r in rows]
-        ok = [r for r in rows if r["recall"] >= 0.90]
+        rows = [b.measure(L, 3, 1, policy) for L in Ls]
+        out[name] = [slim(r, ("L", "qps", "recall", "frac", "dist_evals_per_query")) for r in rows]
+        ok = [r for r in rows if r["recall"] >= RECALL_TARGET]
         out[name + "_qps_at_recall_0.90"] = max(r["qps"] for r in ok) if ok else None
         if ok and name == "best_first" and with_cpu:
             fastest = max(ok, key=lambda r: r["qps"])
-            cpu = cpu_baseline(w, gt, fastest["L"], k)
+            cpu = cpu_reference(w, b.gt, fastest["L"], w["k"], budget_s=8.0)
             out["cpu_at_recall_0.90"] = cpu
             out["gpu_over_cpu_at_recall_0.90"] = fastest["qps"] / cpu["value"]
-    idx.close()
+    b.close()
     return out
 
 
@@ -123,11 +331,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--L", type=int, default=512, help="beam capacity of the headline number (256 or 512)")
+    ap.add_argument("--L", type=int, default=0,
+                    help="quote the headline at this beam capacity instead of searching for the smallest one that "
+                         "reaches recall@100 >= 0.90 (the line then says whether the recall was met)")
+    ap.add_argument("--policy", default="rounds", choices=("rounds", "best_first"), help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
-    ap.add_argument("--only-L", action="store_true", help="run the headline L only")
-    ap.add_argument("--no-structured", action="store_true",
-                    help="skip the legs beside the headline (second enhancement pass, structured data)")
+    ap.add_argument("--no-legs", action="store_true",
+                    help="headline only: skip the legs beside it (other configurations, second enhancement pass, "
+                         "structured data, control queries, memory rates)")
+    ap.add_argument("--legs-budget-s", type=float, default=330.0,
+                    help="no further leg beside the headline is started once the run is this old")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for memory counters)")
     ap.add_argument("--n", type=int, default=1000000, help=argparse.SUPPRESS)
@@ -138,7 +351,6 @@ def main():
               "runs on a single MI355X; --gpus %d is not supported" % args.gpus, file=sys.stderr)
         return 2
 
-    import numpy as np
     import torch
     from coral_amd import capi, workloads
 
@@ -147,20 +359,28 @@ def main():
         return 2
     capi.lib()  # fails loudly if the HIP library is missing
 
-    t0 = time.time()
+    def optional(fn, *a, **kw):
+        """A leg beside the headline: its failure is reported in the line, it never costs the headline."""
+        if args.no_legs:
+            return None
+        if time.time() - T0 > args.legs_budget_s:
+            return {"skipped": "the run was older than --legs-budget-s when this leg's turn came"}
+        try:
+            t = time.time()
+            out = fn(*a, **kw)
+            log("leg %s: %.1f s" % (getattr(fn, "__name__", fn), time.time() - t))
+            return out
+        except Exception as ex:  # noqa: BLE001
+            print("bench.py: optional leg %s failed: %s" % (getattr(fn, "__name__", fn), ex), file=sys.stderr)
+            return {"error": str(ex)}
+
     w = workloads.config2(n=args.n, Q=args.queries)
-    base, queries, k = w["base"], w["queries"], w["k"]
-    Q, dim = queries.shape
-    idx = capi.Index(base, w["nbrs"], w["starts"], capi.L2)
-    gt, _, gt_s = idx.bruteforce(queries, k, want_dists=False)  # exact ground truth, the library's own kernels
-    prep_s = time.time() - t0
-
-    d_q = torch.from_numpy(queries).cuda()
-    d_ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
-    d_gt = torch.from_numpy(gt).cuda()
-
-    def run(L, steps, warmup, policy=capi.POLICY_ROUNDS):
-        return measure(idx, d_q, d_ids, d_gt, Q, k, dim, L, steps, warmup, policy)
+    k = w["k"]
+    b = Bench(w)
+    Q, dim = b.Q, b.dim
+    prep_s = time.time() - T0
+    log("index resident, ground truth in %.3f s" % b.gt_s)
+    policy = capi.POLICY_ROUNDS if args.policy == "rounds" else capi.POLICY_BEST_FIRST
 
     if args.calibration_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -168,101 +388,131 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    other_L = 256 if args.L == 512 else 512
-    def optional(fn, *a, **kw):
-        """A leg beside the headline: its failure is reported in the line, it never costs the headline."""
-        try:
-            return fn(*a, **kw)
-        except Exception as ex:  # noqa: BLE001
-            print("bench.py: optional leg %s failed: %s" % (getattr(fn, "__name__", fn), ex), file=sys.stderr)
-            return {"error": str(ex)}
 
-    also = None if args.only_L else run(other_L, max(3, args.steps // 2), 1)
-    # the CPU path's traversal (best-first) on the GPU, for the comparison with cpu_baseline at equal policy
-    best_first = None if args.only_L else optional(run, args.L, 3, 1, policy=capi.POLICY_BEST_FIRST)
-    head = run(args.L, args.steps, args.warmup)
+    # ---- where the metric's recall is
+    probes = []
+    if args.L:
+        L_head = args.L
+    else:
+        L_head, probes = b.operating_point(policy)
+        log("operating point: L=%s after probes %s" % (L_head, [(p[0], round(p[1], 4)) for p in probes]))
+    recall_met = L_head is not None
+    if L_head is None:  # no beam the library takes reaches the recall: quote the longest probed, and say so
+        L_head = max(p[0] for p in probes)
+    also = None if args.no_legs else [slim(b.measure(Lx, max(3, args.steps // 4), 1, policy)) for Lx in (256, 512)]
+    head = b.measure(L_head, args.steps, args.warmup, policy)
+    recall_met = recall_met and head["recall"] >= RECALL_TARGET
+    log("headline L=%d: %.0f q/s, recall %.4f" % (L_head, head["qps"], head["recall"]))
 
+    traffic = measured_traffic("beam_search_kernel", head["L"], args.policy) if args.n == 1000000 and \
+        args.queries == 10000 else None
     out = {
         "metric": "QPS at recall@100>=0.90, 1Mx200 fp32 L2, R=32, 1 MI355X; achieved HBM GB/s",
-        "value": head["qps"], "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": w["name"], "L": head["L"], "k": k, "policy": "rounds", "recall@100": head["recall"],
-                   "note": "recall@100 >= 0.90 is not reachable on isotropic 200-d Gaussian data with a "
-                           "degree-32 graph at L <= 512; value is quoted at config.L with its measured recall",
-                   "graph": w.get("build"), "prep_s": prep_s, "ground_truth_s": gt_s},
+        "value": head["qps"] if recall_met else None, "unit": "queries/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w["name"], "L": head["L"], "k": k, "policy": args.policy,
+                   "recall@100": head["recall"], "recall_met": recall_met,
+                   "qps_at_config_L": head["qps"],
+                   "note": "L is the smallest multiple of %d whose recall@100 over the whole batch is >= %.2f on this "
+                           "workload (isotropic 200-d Gaussian base: a degree-32 graph needs a beam this long); the "
+                           "configuration's own L = 256 and 512 are under 'also'" % (L_STEP, RECALL_TARGET),
+                   "operating_point_probes": [{"L": p[0], "recall": p[1], "qps": p[2]} for p in probes],
+                   "graph": w.get("build"), "prep_s": prep_s, "ground_truth_s": b.gt_s},
         "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": head["gbps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(head["L"]),
+                     "frac": head["frac"], "traffic": traffic["bytes"] if traffic else None,
+                     "traffic_record": traffic,
+                     "achieved_is": "algorithmic bytes per launch / average kernel duration (HIP events)",
                      "kernel": "beam_search_kernel", "kernel_ms": head["kernel_ms"],
                      "algorithmic_bytes_per_launch": head["bytes_per_launch"],
                      "expansions_per_query": head["expansions_per_query"],
                      "dist_evals_per_query": head["dist_evals_per_query"]},
     }
     if also:
-        out["also"] = {k2: also[k2] for k2 in ("L", "qps", "recall", "kernel_ms", "gbps", "ms_per_step", "spills")}
-        out["also"]["frac"] = also["gbps"] / HBM_PEAK_GBPS
-    # the library's exhaustive search on the same queries (host buffers in and out): what recall@100 >= 0.90 costs on
-    # this data, since no beam the graph search accepts reaches it
-    out["exact_knn"] = {"qps": Q / gt_s, "recall": 1.0, "time_s": gt_s,
+        out["also"] = also
+
+    # what this GPU's memory delivers: a streaming read and a random gather of vector-sized rows over 8 GiB
+    mem = optional(capi.membench, 8 << 30, dim * 4, 3)
+    if mem and not isinstance(mem, dict):
+        out["roofline"]["practical_peak"] = mem[0]
+        out["roofline"]["practical_peak_is"] = "coral_membench: streaming read of 8 GiB, GB/s"
+        out["roofline"]["gather_peak"] = mem[1]
+        out["roofline"]["gather_peak_is"] = "coral_membench: %d-byte rows from random places of 8 GiB, GB/s" % (dim * 4)
+        out["roofline"]["frac_of_practical_peak"] = head["gbps"] / mem[0]
+        out["roofline"]["note"] = ("achieved counts the bytes the algorithm asks for; the 0.8 GB of vectors are "
+                                   "visited unevenly and part of them is served by L2 and the 256 MB memory-side "
+                                   "cache, which is how it can exceed gather_peak")
+    elif mem:
+        out["roofline"]["practical_peak"] = mem
+
+    # the library's exhaustive search on the same queries (host buffers in and out): what recall 1.0 costs here
+    out["exact_knn"] = {"qps": Q / b.gt_s, "recall": 1.0, "time_s": b.gt_s,
                         "kernels": "approx_tile_mfma_kernel (fp32 MFMA screening) + row_select_kernel + rerank_kernel"}
-    if best_first and "error" in best_first:
-        out["best_first"] = best_first
-    elif best_first:
-        out["best_first"] = {k2: best_first[k2] for k2 in ("L", "qps", "recall", "kernel_ms", "gbps",
-                                                           "dist_evals_per_query", "expansions_per_query")}
-        out["best_first"]["kernel"] = "best_first_wave_kernel"
-        out["best_first"]["frac"] = best_first["gbps"] / HBM_PEAK_GBPS
-        out["best_first"]["traffic"] = BEST_FIRST_TRAFFIC_BYTES.get(best_first["L"])
 
     # the IndexGPU::Search shape: host buffers in and out (query upload to the index's staging buffers,
     # search, id download); reported beside the headline, never as the headline
-    idx.search(queries, k, head["L"], want_dists=False)
+    b.idx.search(b.queries, k, head["L"], want_dists=False)
     t = time.perf_counter()
-    idx.search(queries, k, head["L"], want_dists=False)
+    b.idx.search(b.queries, k, head["L"], want_dists=False)
     out["host_buffers_qps"] = Q / (time.perf_counter() - t)
 
+    # ---- the reference's CPU path beside it, at the beam where ITS traversal (best-first) reaches the recall
     if not args.no_cpu:
-        out["cpu_baseline"] = optional(cpu_baseline, w, gt, head["L"], k)
-        if out["cpu_baseline"].get("value"):
-            out["gpu_over_cpu"] = head["qps"] / out["cpu_baseline"]["value"]
-    idx.close()
-    if not (args.no_structured or args.only_L):
-        out["shipped_config_graph"] = optional(shipped_config_leg, w)
+        def cpu_leg():
+            L_cpu, seen = cpu_operating_point(w, b.gt, k, max(L_STEP, head["L"]), capi.MAX_BEAM)
+            res = cpu_reference(w, b.gt, L_cpu or seen[-1]["L"], k)
+            res["recall_met"] = bool(L_cpu) and res["recall"] >= RECALL_TARGET
+            res["operating_point_probes"] = seen
+            return res
+        try:
+            out["cpu_baseline"] = cpu_leg()
+        except Exception as ex:  # noqa: BLE001
+            print("bench.py: cpu baseline failed: %s" % ex, file=sys.stderr)
+            out["cpu_baseline"] = {"error": str(ex)}
+        cpu = out["cpu_baseline"]
+        if cpu.get("value"):
+            log("cpu reference L=%d: %.1f q/s, recall %.4f" % (cpu["L"], cpu["value"], cpu["recall"]))
+            # both sides at recall@100 >= 0.90, each with its own traversal: the GPU path's rounds, the CPU path's
+            # best-first
+            out["gpu_over_cpu"] = head["qps"] / cpu["value"]
+            out["gpu_over_cpu_is"] = "headline (rounds, L=%d, recall %.4f) / cpu_baseline (best-first, L=%d, recall " \
+                                     "%.4f)" % (head["L"], head["recall"], cpu["L"], cpu["recall"])
+
+            def same_policy():
+                # the CPU path's traversal on the GPU at the CPU's beam, on a slice the kernel finishes in seconds
+                r = b.measure(cpu["L"], 1, 0, capi.POLICY_BEST_FIRST, Q=min(Q, 1024))
+                r["kernel"] = "beam_search_kernel (policy 1, beam in global memory)" if cpu["L"] > capi.MAX_LDS_BEAM \
+                    else "best_first_wave_kernel"
+                return r
+            bf = optional(same_policy)
+            if bf and "qps" in bf:
+                out["best_first"] = slim(bf)
+                out["best_first"]["kernel"] = bf["kernel"]
+                out["gpu_over_cpu_same_policy"] = bf["qps"] / cpu["value"]
+    # equal policy at the configuration's L = 512 (the wavefront-per-query kernel against the CPU at the same beam)
+    bf512 = optional(b.measure, 512, 3, 1, capi.POLICY_BEST_FIRST)
+    if bf512 and "qps" in bf512:
+        out["best_first_L512"] = slim(bf512)
+        out["best_first_L512"]["kernel"] = "best_first_wave_kernel"
+        tr = measured_traffic("best_first_wave_kernel", 512, "best_first")
+        out["best_first_L512"]["traffic"] = tr["bytes"] if tr else None
+        if not args.no_cpu:
+            c512 = optional(cpu_reference, w, b.gt, 512, k, budget_s=6.0)
+            if c512 and c512.get("value"):
+                out["best_first_L512"]["cpu_reference"] = c512
+                out["best_first_L512"]["gpu_over_cpu"] = bf512["qps"] / c512["value"]
+    b.close()
+
+    if not args.no_legs:
+        out["control_queries"] = optional(control_leg, w, head["L"])
         out["structured"] = optional(structured_leg, with_cpu=not args.no_cpu)
+        out["shipped_config_graph"] = optional(shipped_config_leg, w)
+        w = b = None  # (the closures above hold the names, not the arrays)
+        out["configs"] = {"1": optional(config1_leg, not args.no_cpu), "3": optional(config3_leg),
+                          "4": optional(config4_leg)}
+    out["wall_s"] = time.time() - T0
     print(json.dumps(out), flush=True)
     return 0
-
-
-def cpu_baseline(w, gt, L, k):
-    """The reference's CPU search (best-first, sorted queue, AVX-512 squared L2, OpenMP
-    dynamic schedule over queries; src/search_in_cpu.cpp:23-119) on this host's cores.
-    Uses oracle/_ref (the reference's own queue and distance headers compiled in place)
-    when it is present and the host has AVX-512, otherwise the oracle's restatement."""
-    import oracle
-    prob = oracle.Problem(w["base"], w["nbrs"], w["starts"])
-    q = w["queries"]
-    threads = os.cpu_count() or 1
-    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
-    use_ref = oracle.ref() is not None and oracle.lib().oracle_have_avx512()
-    fn = oracle.ref_search_in_cpu if use_ref else oracle.search_A
-    # bounded sample: time a slice first, then as many queries as fit in about 20 s
-    probe = min(256, q.shape[0])
-    _, _, _, t = fn(prob, q[:probe], k, L, nthreads=threads)
-    n = int(min(q.shape[0], max(probe, 20.0 / max(t / probe, 1e-9))))
-    # a sample that short of 10 s is timed again (at most 9 passes in all) and the median pass is
-    # quoted: a single pass of under a second on a shared host varies by a third from run to run
-    times = []
-    while not times or (sum(times) < 10.0 and len(times) < 9):
-        ids, _, stats, t = fn(prob, q[:n], k, L, nthreads=threads)
-        times.append(t)
-    t = sorted(times)[len(times) // 2]
-    hits = oracle.recall_hits(ids, gt[:n], k)
-    return {"value": n / t, "unit": "queries/s", "cores": threads, "kind": "reference" if use_ref else "port",
-            "sample": "first %d of %d queries, L=%d, k=%d, M=%d start ids, policy best-first; median of %d passes" %
-                      (n, q.shape[0], L, k, w["starts"].size, len(times)),
-            "recall": hits / float(n * k), "time_s": t, "passes_s": [round(x, 4) for x in times],
-            "dist_evals_per_query": float(stats[:, 2].mean()),
-            "expansions_per_query": float(stats[:, 1].mean())}
 
 
 if __name__ == "__main__":

@@ -42,7 +42,8 @@ class Stats(C.Structure):
 class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
                 ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("best_first_packed", C.c_int32),
-                ("best_first_table_log2", C.c_int32), ("beam_in_hbm", C.c_int32)]
+                ("best_first_table_log2", C.c_int32), ("beam_in_hbm", C.c_int32), ("prefetch_rows", C.c_int32),
+                ("cand_cap", C.c_int32)]
 
 
 class BuildParams(C.Structure):
@@ -115,6 +116,8 @@ SIGNATURES = {
     "coral_start_ids_fps": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_bruteforce_set_exact_only": (C.c_int, [C.c_void_p, C.c_int32]),
     "coral_bruteforce_last_redone": (C.c_int64, [C.c_void_p]),
+    "coral_membench": (C.c_int, [C.c_int32, C.c_size_t, C.c_int32, C.c_int32, C.POINTER(C.c_double),
+                                 C.POINTER(C.c_double)]),
     "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
                                        C.c_void_p, C.POINTER(C.c_double)]),
 }
@@ -141,6 +144,13 @@ def _check(rc):
 
 def _ptr(a):
     return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def membench(bytes_=8 << 30, row_bytes=800, reps=3, device=0):
+    """(streaming read GB/s, random row gather GB/s) of the device's memory: coral_membench."""
+    a, b = C.c_double(), C.c_double()
+    _check(lib().coral_membench(device, bytes_, row_bytes, reps, C.byref(a), C.byref(b)))
+    return a.value, b.value
 
 
 class Index:
@@ -200,9 +210,10 @@ class Index:
         return m
 
     def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False,
-                best_first_packed=False, best_first_table_log2=0, beam_in_hbm=False):
+                best_first_packed=False, best_first_table_log2=0, beam_in_hbm=False, prefetch_rows=0, cand_cap=0):
         t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)),
-                   int(bool(best_first_packed)), best_first_table_log2, int(bool(beam_in_hbm)))
+                   int(bool(best_first_packed)), best_first_table_log2, int(bool(beam_in_hbm)), prefetch_rows,
+                   cand_cap)
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

@@ -38,9 +38,10 @@ struct SearchArgs {
     // expand live in global memory, beam_stride 64-bit words per workgroup ([2][Lp] keys, then Lp ids).
     uint64_t* beam_scratch;
     size_t beam_stride;
-    // BIG form only: the visited set is a plain bitmap of the n ids in LDS (table_words 32-bit words) instead of
-    // the table of 16-bit cells; no id ever goes to the bitmap in global memory then
+    // the visited set is a plain bitmap of the n ids in LDS (table_words 32-bit words) instead of the table of
+    // 16-bit cells; no id ever goes to the bitmap in global memory then
     int32_t direct_bitmap;
+    int32_t prefetch_rows;     // request a chunk's graph rows one chunk ahead (launches with one workgroup per CU)
     int32_t table_words;       // 32-bit words of LDS the visited structure takes (cells / 2, or ceil(n / 32) rounded up to 4)
 };
 

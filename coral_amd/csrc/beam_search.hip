@@ -79,7 +79,7 @@ struct VisitedSet {
     uint32_t* bitmap;  // global
     uint32_t smask, bmask, rmask;
     int rb, xs, dmax, ocap;
-    bool direct;       // words is a bitmap of all ids (BIG launches over few enough nodes)
+    bool direct;       // words is a bitmap of all ids (launches over few enough nodes that have LDS to spare)
 
     __device__ __forceinline__ uint32_t mix(uint32_t id) const {
         uint32_t h = (id * 0x9E3779B1u) & bmask;
@@ -90,9 +90,8 @@ struct VisitedSet {
     }
 
     // 1 if id was not yet in the set (and now is), 0 if it was
-    template <bool BIG>
     __device__ __forceinline__ int test_and_set(uint32_t id, bool frozen) {
-        if (BIG && direct) {
+        if (direct) {
             const uint32_t b = 1u << (id & 31);
             return (atomicOr(&words[id >> 5], b) & b) == 0u;
         }
@@ -173,7 +172,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     vs.smask = (uint32_t)slots - 1u, vs.bmask = a.id_bits >= 32 ? 0xffffffffu : (1u << a.id_bits) - 1u;
     vs.rb = a.rem_bits, vs.rmask = (1u << a.rem_bits) - 1u;
     vs.xs = a.id_bits > 1 ? a.id_bits / 2 : 1, vs.dmax = a.dmax, vs.ocap = a.ocap;
-    vs.direct = BIG && a.direct_bitmap != 0;
+    vs.direct = a.direct_bitmap != 0;
     (void)slots;
 
     constexpr int GPW = 64 / G;                    // row groups per wave
@@ -386,7 +385,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         const int M = a.M;
         for (int i = tid; i < M; i += NT) {
             const uint32_t id = (uint32_t)a.start_ids[i];
-            vs.template test_and_set<BIG>(id, false);
+            vs.test_and_set(id, false);
             todo[i] = id;
         }
         __syncthreads();
@@ -456,12 +455,21 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 break;
             }
 
-            // The round's rows are taken in chunks of `ech` beam entries (what the todo
-            // list holds).  Requesting graph rows ahead of time (the next chunk's, or for
-            // best-first the likely next entry's) was measured twice and lost to this plain
-            // form: the other workgroup on the CU already covers that wait.
+            // The round's rows are taken in chunks of `ech` beam entries (what the todo list holds).  Where one
+            // pass of the workgroup covers a chunk's ids (ech * R <= threads) and the launch asks for it, a chunk's
+            // ids are requested one chunk ahead -- and the entry whose row they come from two chunks ahead -- so
+            // that both waits pass while the chunk before is being measured.  With two workgroups per CU the other
+            // workgroup covers those waits and the look-ahead only costs (measured); with one it pays.
             const int ech = TCAP / R;
             ne += nexp;
+            const bool ahead = a.prefetch_rows != 0 && ech * R <= NT;
+            const int pe = tid / R, pj = tid - pe * R;  // this thread's entry of a chunk and neighbour slot
+            int vpre = -1;
+            uint32_t epre = 0;
+            if (ahead) {
+                if (pe < min(ech, nexp)) vpre = a.nbrs[(size_t)elist[pe] * R + pj];
+                if (pe < ech && ech + pe < nexp) epre = elist[ech + pe];
+            }
             for (int e0 = 0; e0 < nexp; e0 += ech) {
                 if (!spill && s_nvis > a.vis_limit) spill = true;
                 if (tid == 0) s_ntodo = 0;
@@ -470,12 +478,14 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 for (int f0 = 0; f0 < total; f0 += NT) {
                     const int f = f0 + tid;
                     int v = -1;
-                    if (f < total) {
+                    if (ahead) {
+                        v = vpre;
+                    } else if (f < total) {
                         const int e = f / R;
                         v = a.nbrs[(size_t)elist[e0 + e] * R + (f - e * R)];
                     }
                     bool isnew = false;
-                    if (v >= 0) isnew = vs.template test_and_set<BIG>((uint32_t)v, spill) != 0;
+                    if (v >= 0) isnew = vs.test_and_set((uint32_t)v, spill) != 0;
                     const uint64_t m = __ballot(isnew);
                     if (m) {
                         int pos = 0;
@@ -491,6 +501,13 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 if (s_ncand + T > CCAP) merge();  // merge() starts and ends with a barrier
                 PHASE_MARK(5);
                 if (tid == 0) s_nvis += T;
+                if (ahead) {
+                    // the next chunk's ids (their entries arrived a chunk ago) and the entries of the chunk after
+                    vpre = -1;
+                    const int e1 = e0 + ech, e2 = e0 + 2 * ech;
+                    if (pe < ech && e1 + pe < nexp) vpre = a.nbrs[(size_t)epre * R + pj];
+                    if (pe < ech && e2 + pe < nexp) epre = elist[e2 + pe];
+                }
                 distance_phase(T);
                 __syncthreads();
                 PHASE_MARK(4);

@@ -253,7 +253,7 @@ int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* 
 // Launch geometry of the workgroup-per-query kernel for a beam of capacity L: arithmetic, the kernel's LDS
 // attribute and an occupancy query; nothing is allocated.  bump_log2 raises the library's own choice of table size.
 static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral_tuning& t, int bump_log2,
-                       coral_search_plan* out) {
+                       bool lds_beam_only, coral_search_plan* out) {
     if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
     if (L <= 0 || L > kMaxL) return fail(CORAL_ERR_ARG, "L must be in 1..%d (got %d)", kMaxL, L);
     if (idx->M <= 0) return fail(CORAL_ERR_STATE, "the graph has no start ids yet (rows under construction)");
@@ -265,41 +265,61 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     coral_search_plan p;
     p.L = L;
     p.big = L > CORAL_MAX_LDS_BEAM || t.beam_in_hbm != 0;
-    // todo / candidate buffers: sized below, once the visited structure is known
+    // todo / candidate buffers: at least what the start ids and four graph rows need
     int min_cap = 256;
     while (min_cap < idx->M || min_cap < idx->R * 4) min_cap <<= 1;
-    int tcap = min_cap;
-    int ocap = 256;
     int id_bits = 1;
     while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
-    int slots_log2 = t.visited_slots_log2;
-    auto table_lds = [&](int lg, int cap) {
-        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, ocap, p.big) + 64;
+    const size_t lds_max = (size_t)kMaxLdsBytes;
+    // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
+    // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
+    // -1, or the library's choice): one LDS atomic per test and nothing ever overflows, at n / 8 bytes -- 125 KB for
+    // a million nodes, which leaves a CU one workgroup.
+    const int bitmap_words = (int)(((idx->n + 31) / 32 + 3) & ~(int64_t)3);
+    auto lds_bitmap = [&](bool big, int cap) {
+        return coral::search_lds_bytes(L, idx->dim, bitmap_words, cap, cap, 4, big) + 64;
     };
-    if (p.big) {
-        // The beams are out of LDS.  What they leave takes the visited set as a bitmap of all n ids where that fits
-        // (a million nodes = 125 KB), else the largest table of cells; one workgroup of 1024 threads per CU.
-        if (!best_first) tcap = std::max(tcap, 1024);
-        const int bitmap_words = (int)(((idx->n + 31) / 32 + 3) & ~(int64_t)3);
-        if (slots_log2 == 0 && idx->n <= ((int64_t)1 << 21) &&
-            coral::search_lds_bytes(L, idx->dim, bitmap_words, tcap, tcap, 4, true) + 64 <= (size_t)kMaxLdsBytes) {
-            p.direct = 1, p.table_words = bitmap_words, ocap = 4;
-        } else if (slots_log2 == 0) {
-            slots_log2 = 16;
-            while (slots_log2 > 12 && table_lds(slots_log2, tcap) > (size_t)kMaxLdsBytes) --slots_log2;
+    auto lds_table = [&](bool big, int lg, int cap) {
+        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, 256, big) + 64;
+    };
+    const bool bitmap_possible = idx->n <= ((int64_t)1 << 21);
+    int slots_log2 = t.visited_slots_log2;
+    if (slots_log2 == -1) {
+        if (!bitmap_possible || lds_bitmap(p.big, min_cap) > lds_max)
+            return fail(CORAL_ERR_ARG, "a bitmap of %lld ids does not fit LDS beside a beam of %d", (long long)idx->n, L);
+        p.direct = 1;
+    } else if (slots_log2 == 0 && !best_first) {
+        // the table the rounds policy wants: a degree-32 graph over a million nodes sees about 75 first visits per
+        // beam entry, 112 cells per entry keep the load factor near 0.65; `bump_log2` doubles that after batches
+        // that overflowed (see coral_search_gpu)
+        int want = 12;
+        while ((1 << want) < 112 * L && want < 20) ++want;
+        want += bump_log2;
+        const bool table_holds = !p.big && want <= 16 && lds_table(false, want, min_cap) <= lds_max;
+        const bool table_alone_on_cu = table_holds && lds_table(false, want, min_cap) > lds_max / 2;
+        if (bitmap_possible && !p.big && lds_bitmap(false, min_cap) <= lds_max && (!table_holds || table_alone_on_cu)) {
+            p.direct = 1;  // one workgroup per CU either way: the bitmap is the cheaper test and cannot overflow
+        } else if (bitmap_possible && !table_holds && !lds_beam_only && lds_bitmap(true, 1024) <= lds_max) {
+            p.direct = 1, p.big = true;  // the beam gives its LDS to the bitmap (measured: +30 % at L = 1024 and 2048)
+        } else {
+            slots_log2 = std::min(16, want);
+            while (slots_log2 > 12 && lds_table(p.big, slots_log2, min_cap) > lds_max) --slots_log2;
         }
     } else if (slots_log2 == 0) {
-        // a degree-32 graph over a million nodes sees about 75 first visits per beam
-        // entry; 112 cells per entry keep the load factor near 0.65
-        // (best-first: about 31 first visits per entry, 48 cells)
-        slots_log2 = 12;
-        while ((1 << slots_log2) < (best_first ? 48 : 112) * L && slots_log2 < 16) ++slots_log2;
-        slots_log2 = std::min(16, slots_log2 + bump_log2);  // see coral_search_gpu
-        while (slots_log2 > 12 && table_lds(slots_log2, tcap) > (size_t)kMaxLdsBytes) --slots_log2;
+        // best-first on this kernel: about 31 first visits per beam entry, 48 cells
+        if (p.big && bitmap_possible && lds_bitmap(true, min_cap) <= lds_max) {
+            p.direct = 1;
+        } else {
+            slots_log2 = 12;
+            while ((1 << slots_log2) < 48 * L && slots_log2 < 16) ++slots_log2;
+            slots_log2 = std::min(16, slots_log2 + bump_log2);
+            while (slots_log2 > 12 && lds_table(p.big, slots_log2, min_cap) > lds_max) --slots_log2;
+        }
     }
+    int ocap = 256;
     if (!p.direct) {
         if (slots_log2 < 10 || slots_log2 > 16)
-            return fail(CORAL_ERR_ARG, "visited_slots_log2 must be in 10..16");
+            return fail(CORAL_ERR_ARG, "visited_slots_log2 must be -1 or in 10..16");
         const int slots = 1 << slots_log2;
         p.slots_log2 = slots_log2, p.table_words = slots >> 1;
         p.rem_bits = std::max(0, id_bits - slots_log2);
@@ -308,38 +328,50 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         p.vis_limit = p.dmax < 0 ? 0 : slots - slots / 4;
         p.spill_words = ((size_t)idx->n + 31) / 32;
     } else {
+        p.table_words = bitmap_words, ocap = 4;
         p.dmax = -1, p.vis_limit = 0x7fffffff;
     }
-    // Larger chunks mean fewer latency-bound steps per round: take the largest todo /
-    // candidate capacity that does not lower the number of workgroups a CU can hold.
-    auto lds_for = [&](int cap) {
-        return coral::search_lds_bytes(L, idx->dim, p.table_words, cap, cap, ocap, p.big) + 64;
+    // ---- todo and candidate buffers (powers of two: the candidates are bitonic-sorted in place).  Larger chunks
+    // mean fewer latency-bound steps per round: the largest that does not lower the number of workgroups a CU can
+    // hold; a launch that is alone on its CU anyway takes a candidate buffer of twice the size where there is room
+    // (half as many merges of a long beam).  Best-first expands one row at a time and needs neither.
+    auto lds_for = [&](int tc, int cc) {
+        return coral::search_lds_bytes(L, idx->dim, p.table_words, tc, cc, ocap, p.big) + 64;
     };
-    if (lds_for(min_cap) > (size_t)kMaxLdsBytes)
+    if (lds_for(min_cap, min_cap) > lds_max)
         return fail(CORAL_ERR_ARG, "L=%d with %d words of visited state needs %zu bytes of LDS", L, p.table_words,
-                    lds_for(min_cap));
-    while (tcap > min_cap && lds_for(tcap) > (size_t)kMaxLdsBytes) tcap >>= 1;
-    const int wg_fit = (int)((size_t)kMaxLdsBytes / lds_for(min_cap));
-    // (capacities are powers of two: the candidate buffer is bitonic-sorted in place)
+                    lds_for(min_cap, min_cap));
+    int tcap = min_cap;
+    const int wg_fit = (int)(lds_max / lds_for(min_cap, min_cap));
     for (int cap : {1024, 512}) {
-        if (cap <= tcap || best_first) break;  // best-first expands one row at a time
-        if (lds_for(cap) <= (size_t)kMaxLdsBytes && (int)((size_t)kMaxLdsBytes / lds_for(cap)) >= std::min(wg_fit, 2)) {
+        if (cap <= tcap || best_first) break;
+        if (lds_for(cap, cap) <= lds_max && (int)(lds_max / lds_for(cap, cap)) >= std::min(wg_fit, 2)) {
             tcap = cap;
             break;
         }
     }
+    int ccap = tcap;
+    if (t.cand_cap > 0) {
+        if ((t.cand_cap & (t.cand_cap - 1)) != 0 || t.cand_cap < tcap || lds_for(tcap, t.cand_cap) > lds_max)
+            return fail(CORAL_ERR_ARG, "cand_cap must be a power of two, at least %d, that fits LDS", tcap);
+        ccap = t.cand_cap;
+    } else if (!best_first && p.big && lds_for(tcap, 2 * tcap) <= lds_max) {
+        ccap = 2 * tcap;
+    }
     int threads = t.threads;
     if (threads == 0)
-        threads = p.big ? 1024 : best_first ? 256 : (lds_for(tcap) > (size_t)kMaxLdsBytes / 2 ? 1024 : 512);
+        threads = p.big ? 1024 : best_first ? 256 : (lds_for(tcap, ccap) > lds_max / 2 ? 1024 : 512);
     if (threads != 128 && threads != 256 && threads != 512 && threads != 1024)
         return fail(CORAL_ERR_ARG, "threads must be 128, 256, 512 or 1024");
-    p.lds_bytes = coral::search_lds_bytes(L, idx->dim, p.table_words, tcap, tcap, ocap, p.big);
+    p.lds_bytes = coral::search_lds_bytes(L, idx->dim, p.table_words, tcap, ccap, ocap, p.big);
     int wg_per_cu = 0;
     HIP_TRY(coral::search_kernel_prepare(idx->dim, p.big, p.lds_bytes, threads, &wg_per_cu));
     if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
     int workgroups = t.workgroups > 0 ? t.workgroups : wg_per_cu * idx->num_cu;
     p.workgroups = std::min(workgroups, (int)Q);
-    p.tcap = tcap, p.ccap = tcap, p.threads = threads, p.id_bits = id_bits, p.ocap = ocap;
+    p.tcap = tcap, p.ccap = ccap, p.threads = threads, p.id_bits = id_bits, p.ocap = ocap;
+    // graph rows a chunk ahead: pays where a workgroup is alone on its CU (nothing else covers the wait)
+    p.prefetch = t.prefetch_rows > 0 || (t.prefetch_rows == 0 && wg_per_cu == 1 && !best_first);
     p.beam_stride = p.big ? coral::search_beam_stride(L) : 0;
     *out = p;
     return CORAL_OK;
@@ -353,7 +385,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     if (tuning) t = *tuning;
     HIP_TRY(hipSetDevice(idx->device));
     coral_search_plan plan;
-    if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, &plan)) return rc;
+    if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, false, &plan)) return rc;
     HIP_TRY(hipStreamSynchronize(idx->stream));
     const bool best_first = t.policy == CORAL_POLICY_BEST_FIRST;
     const int id_bits = plan.id_bits;
@@ -473,6 +505,7 @@ static coral::SearchArgs search_args(const coral_index* idx, const coral_search_
     a.tcap = p.tcap, a.ccap = p.ccap;
     a.id_bits = p.id_bits, a.rem_bits = p.rem_bits, a.dmax = p.dmax, a.ocap = p.ocap;
     a.beam_stride = p.beam_stride, a.direct_bitmap = p.direct, a.table_words = p.table_words;
+    a.prefetch_rows = p.prefetch;
     return a;
 }
 
@@ -608,13 +641,14 @@ int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* 
     std::memset(&t, 0, sizeof t);
     t.policy = policy;  // both policies run on the workgroup-per-query kernel here
     coral_search_plan plan;
-    if (int rc = plan_search(idx, Q, L, t, 0, &plan)) return rc;
+    if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, &plan)) return rc;
     // the block: 256 bytes of scalars, the per-query counters, then one overflow bitmap per workgroup
     int* scal = reinterpret_cast<int*>(base);
     int32_t* counters = reinterpret_cast<int32_t*>(base + 256);
     uint32_t* spill = reinterpret_cast<uint32_t*>(base + 256 + (size_t)coral::kStaticMaxQ * 16);
-    const int wgs = (int)std::min<size_t>((size_t)std::min(plan.workgroups, (int)Q),
-                                          coral::kStaticSpillWords / plan.spill_words);
+    int wgs = std::min(plan.workgroups, (int)Q);
+    if (plan.spill_words)  // (none when the visited set is a bitmap of all ids in LDS)
+        wgs = (int)std::min<size_t>((size_t)wgs, coral::kStaticSpillWords / plan.spill_words);
     // the block keeps what the last call left: the work counter and the bitmaps must start at zero (fill kernels,
     // which a caller may record into a graph)
     HIP_TRY(coral::launch_fill_u32(reinterpret_cast<uint32_t*>(scal), 64, 0u, stream));

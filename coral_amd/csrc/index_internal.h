@@ -22,7 +22,8 @@
 struct coral_search_plan {
     int L = 0;
     bool big = false;         // beams in global memory (the kernel's BIG form)
-    int direct = 0;           // BIG only: the visited set is a bitmap of all ids in LDS
+    int direct = 0;           // the visited set is a bitmap of all ids in LDS
+    int prefetch = 0;         // a chunk's graph rows are requested one chunk ahead
     int slots_log2 = 0, table_words = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
     int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0;
     size_t lds_bytes = 0;

@@ -91,7 +91,9 @@ typedef struct {
 
 /* Optional launch tuning; zero-initialise for defaults. */
 typedef struct {
-    int32_t visited_slots_log2; /* LDS visited table: log2 of its 16-bit cells, 10..16; 0 = chosen from L */
+    int32_t visited_slots_log2; /* visited set in LDS: log2 of the 16-bit cells of its table, 10..16 (what outgrows the
+                                   table goes to a bitmap in global memory); -1 = a plain bitmap of all n ids instead
+                                   (n / 8 bytes: up to about a million nodes); 0 = chosen from L and n */
     int32_t workgroups;         /* persistent workgroups (of four query slots each on the wavefront-per-query
                                    best-first kernel); 0 = chosen from Q and the device */
     int32_t threads;            /* threads per workgroup: 128, 256, 512 or 1024; 0 = chosen from the LDS need */
@@ -110,7 +112,12 @@ typedef struct {
                                    where 8192 cells hold most of a query's visits (L <= 409 at up to 2^25 nodes),
                                    none otherwise; -1 = none */
     int32_t beam_in_hbm;        /* 1 = keep the beam in global memory whatever L is (the form beams longer than
-                                   CORAL_MAX_LDS_BEAM always take) */
+                                   CORAL_MAX_LDS_BEAM always take, and shorter ones when that frees the LDS a bitmap of
+                                   all ids needs) */
+    int32_t prefetch_rows;      /* graph rows of a chunk of beam entries requested one chunk ahead: 1 = yes, -1 = no,
+                                   0 = where a workgroup has its CU to itself */
+    int32_t cand_cap;           /* capacity of the candidate buffer in LDS (a power of two, at least the todo list's);
+                                   0 = chosen */
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);
@@ -324,6 +331,15 @@ CORAL_API int coral_build_graph_from_clusters(coral_index* idx, const int32_t* h
  * [n][R] and degrees [n] (the dists and deg fields of the reference's Slot).  Any pointer may be NULL. */
 CORAL_API int coral_index_get_graph(coral_index* idx, int32_t* h_nbrs, float* h_dists, int32_t* h_deg,
                                     int32_t* h_start_ids);
+
+/* What the device's memory delivers, for setting the search kernels' rates against (no counterpart in the
+ * reference): allocates `bytes` of device memory (use far more than the 256 MB memory-side cache), reads all of it
+ * once in 16-byte coalesced requests (*stream_gbps) and then as many bytes as rows of row_bytes from pseudo-random
+ * places, one wavefront per row, eight rows in flight per wavefront (*gather_gbps: the access pattern of the distance
+ * phase, one vector row per visited node, with no reuse for a cache to find).  Best of `reps` timed passes each
+ * (HIP events), GB/s = 1e9 bytes per second.  Either pointer may be NULL. */
+CORAL_API int coral_membench(int32_t device, size_t bytes, int32_t row_bytes, int32_t reps, double* stream_gbps,
+                             double* gather_gbps);
 
 #ifdef __cplusplus
 }

@@ -103,8 +103,9 @@ def test_exact_against_same_order_oracle(orc, case):
 
 
 BIG_CASES = [
-    # n, dim, R, metric, policy, L, k, M, ragged, slots_log2 (0: the library's choice, a bitmap of all ids in LDS at
-    # these sizes; else the table of cells that size with the overflow bitmap in global memory), workgroups, tombstones
+    # n, dim, R, metric, policy, L, k, M, ragged, slots_log2 (0: the library's choice, which is -1, a bitmap of all ids
+    # in LDS, at these sizes; else the table of cells that size with the overflow bitmap in global memory), workgroups,
+    # tombstones
     (20000, 200, 32, "l2", 0, 4096, 100, 16, None, 0, 0, False),
     (20000, 200, 32, "l2", 0, 6656, 100, 16, None, 0, 0, False),   # the reference driver's last step (128 * 52)
     (20000, 200, 32, "l2", 1, 4096, 100, 16, None, 0, 0, False),
@@ -227,8 +228,12 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         big = rng.rand() < 0.25  # the beam in global memory, at up to eight times the length drawn above
         if big:
             L = min(n, L * int(rng.choice([1, 3, 8])))
+        if rng.rand() < 0.2:
+            slots = -1  # the visited set as a bitmap of all ids in LDS
+        ahead = int(rng.choice([0, 1, -1]))  # graph rows requested a chunk ahead: the library's choice, yes, no
         print("case", dict(c=c, n=n, dim=dim, R=R, metric=metric, policy=policy, L=L, k=k, M=M, Q=Q, slots=slots,
-                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl, big=big), flush=True)
+                           threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl, big=big, ahead=ahead),
+              flush=True)
         m = capi.IP if metric == "ip" else capi.L2
         base = synth.gaussian_matrix(1000 + c, n, dim)
         if metric == "ip":
@@ -254,7 +259,7 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
             idx.prepare(Q, L, visited_slots_log2=slots, threads=threads, workgroups=wgs, policy=policy,
                         best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=tbl,
-                        beam_in_hbm=big)
+                        beam_in_hbm=big, prefetch_rows=ahead)
             ids, dists, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
             assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
             assert np.array_equal(idx.query_counters(Q), os_)

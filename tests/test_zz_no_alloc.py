@@ -51,14 +51,29 @@ def test_no_alloc_entry_point_equals_the_allocating_one():
                 want = _reference(idx, d_q, Q, k, L, policy, have_delete, torch)
                 assert np.array_equal(got[0], want[0])
                 assert got[1].tobytes() == want[1].tobytes()
-    # a table too small for a query's visits: ids go to the per-workgroup overflow bitmaps of the block
-    # (L = 2048 at 30 000 nodes visits most of the graph) -- and the next, smaller call finds them clean
-    for Q, k, L in ((300, 100, 2048), (64, 5, 32)):
-        d_q = torch.from_numpy(q_all[:Q]).cuda()
-        got = _noalloc(idx, d_q, Q, k, L, capi.POLICY_ROUNDS, False, torch)
-        want = _reference(idx, d_q, Q, k, L, capi.POLICY_ROUNDS, False, torch)
-        assert np.array_equal(got[0], want[0]) and got[1].tobytes() == want[1].tobytes()
-    # a second index on the same GPU uses the same block
+    # a second index on the same GPU uses the same block.  More nodes than a bitmap in LDS can cover (1.3 M), so the
+    # visited set is the table of cells, and at L = 2048 a query outgrows it: ids go to the per-workgroup overflow
+    # bitmaps of the block (fewer workgroups than usual, so that each has one) -- and the next, smaller call finds
+    # them clean.  (A graph of random neighbours; the check is against coral_search_gpu, no oracle needed.)
+    rng = np.random.RandomState(8)
+    n3, dim3 = 1300000, 8
+    base3 = rng.standard_normal((n3, dim3)).astype(np.float32)
+    nbrs3 = rng.randint(0, n3, (n3, 16)).astype(np.int32)
+    idx3 = capi.Index(base3, nbrs3, np.array([1, 70000, 1299999], np.int32))
+    q3 = make_queries(300, dim3, 903)
+    for Q, k, L in ((300, 100, 2048), (16, 5, 32)):
+        print("noalloc case on 1.3 M nodes", dict(Q=Q, k=k, L=L), flush=True)
+        d_q = torch.from_numpy(q3[:Q]).cuda()
+        got = _noalloc(idx3, d_q, Q, k, L, capi.POLICY_ROUNDS, False, torch)
+        ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
+        dists = torch.empty((Q, k), dtype=torch.float32, device="cuda")
+        idx3.prepare(Q, L)
+        st = idx3.search_device(d_q.data_ptr(), ids.data_ptr(), dists.data_ptr(), Q, k)
+        torch.cuda.synchronize()
+        assert st.spills > 0 if L == 2048 else st.spills == 0
+        assert np.array_equal(got[0], ids.cpu().numpy()) and got[1].tobytes() == dists.cpu().numpy().tobytes()
+    idx3.close()
+    # and a small one
     n2, dim2 = 5000, 64
     base2 = synth.gaussian_matrix(92, n2, dim2)
     nbrs2 = synth.exact_knn_graph(base2, 16, device="cuda")
