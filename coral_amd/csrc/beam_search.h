@@ -41,6 +41,7 @@ struct SearchArgs {
     // the visited set is a plain bitmap of the n ids in LDS (table_words 32-bit words) instead of the table of
     // 16-bit cells; no id ever goes to the bitmap in global memory then
     int32_t direct_bitmap;
+    int32_t scap;              // BIG form: keys of the LDS sample of the beam that the merge searches first
     int32_t prefetch_rows;     // request a chunk's graph rows one chunk ahead (launches with one workgroup per CU)
     int32_t table_words;       // 32-bit words of LDS the visited structure takes (cells / 2, or ceil(n / 32) rounded up to 4)
 };
@@ -82,6 +83,8 @@ hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, i
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice
 hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream);
+
+constexpr int kBeamSampleKeys = 512;  // LDS sample of a beam in global memory (4 KB)
 
 // LDS bytes of one workgroup.  big: the beams and the expand list are in global memory, LDS holds the candidate
 // buffer, the visited structure (table_words 32-bit words), the todo list, the overflow list and the query.

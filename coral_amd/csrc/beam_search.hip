@@ -143,13 +143,14 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     const int slots = 1 << a.slots_log2;
     const int TCAP = a.tcap, CCAP = a.ccap;
 
-    uint64_t *beam0, *beam1, *cand;
+    uint64_t *beam0, *beam1, *cand, *samp = nullptr;
     uint32_t *table, *todo, *elist, *olist;
     if constexpr (BIG) {
         uint64_t* g = a.beam_scratch + (size_t)blockIdx.x * a.beam_stride;
         beam0 = g, beam1 = g + Lp, elist = (uint32_t*)(g + 2 * (size_t)Lp);
         cand = (uint64_t*)smem;
-        table = (uint32_t*)(cand + CCAP);  // 16-bit cells, or the bitmap of all ids
+        samp = cand + CCAP;                     // a sample of the beam's keys for the merge's searches
+        table = (uint32_t*)(samp + a.scap);     // 16-bit cells, or the bitmap of all ids
         todo = table + a.table_words;
         olist = todo + TCAP;
     } else {
@@ -361,16 +362,57 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             const uint64_t* src = st.cur ? beam1 : beam0;
             uint64_t* dst = st.cur ? beam0 : beam1;
             const int nb = st.nb;
-            for (int i = tid; i < nb; i += NT) {
-                const uint64_t key = src[i];
-                const int pos = i + lower_bound_u64(cand, nc, key);
-                if (pos < L) dst[pos] = key;
-            }
-            for (int j = tid; j < nc; j += NT) {
-                const uint64_t key = cand[j];
-                const int pos = j + lower_bound_u64(src, nb, key);
-                if (pos < L) dst[pos] = key;
-                if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
+            if constexpr (BIG) {
+                // The beam is in global memory: every access is a trip to L2.  Beam keys are fetched four per
+                // thread before the first is placed, and keys outside the candidates' range need no search; a
+                // candidate's search through the beam starts in an LDS sample of every 2^ss-th beam key, so that
+                // only its last few steps (inside one or two cache lines) go to memory.
+                int ss = 0;
+                while (((nb - 1) >> ss) + 1 > a.scap) ++ss;
+                const int ns = nb > 0 ? ((nb - 1) >> ss) + 1 : 0;
+                for (int j = tid; j < ns; j += NT) samp[j] = src[(size_t)j << ss];
+                const uint64_t c_lo = cand[0], c_hi = cand[nc - 1];
+                for (int i0 = tid; i0 < nb; i0 += 4 * NT) {
+                    uint64_t key[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) key[u] = i0 + u * NT < nb ? src[i0 + u * NT] : kKeyMax;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int i = i0 + u * NT;
+                        if (i < nb) {
+                            const int below = key[u] < c_lo ? 0 : key[u] > c_hi ? nc : lower_bound_u64(cand, nc, key[u]);
+                            if (i + below < L) dst[i + below] = key[u];
+                        }
+                    }
+                }
+                __syncthreads();  // the sample is complete
+                for (int j = tid; j < nc; j += NT) {
+                    const uint64_t key = cand[j];
+                    const int js = lower_bound_u64(samp, ns, key);
+                    int lo = js == 0 ? 0 : ((js - 1) << ss) + 1, hi = js == ns ? nb : (js << ss);
+                    while (lo < hi) {
+                        const int mid = (lo + hi) >> 1;
+                        if (src[mid] < key)
+                            lo = mid + 1;
+                        else
+                            hi = mid;
+                    }
+                    const int pos = j + lo;
+                    if (pos < L) dst[pos] = key;
+                    if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
+                }
+            } else {
+                for (int i = tid; i < nb; i += NT) {
+                    const uint64_t key = src[i];
+                    const int pos = i + lower_bound_u64(cand, nc, key);
+                    if (pos < L) dst[pos] = key;
+                }
+                for (int j = tid; j < nc; j += NT) {
+                    const uint64_t key = cand[j];
+                    const int pos = j + lower_bound_u64(src, nb, key);
+                    if (pos < L) dst[pos] = key;
+                    if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
+                }
             }
             __syncthreads();
             st.nb = min(L, nb + nc);
@@ -646,7 +688,7 @@ static kernel_fn pick_kernel(int dim, bool big) {
 
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big) {
     const size_t Lp = (size_t)((L + 3) & ~3);
-    const size_t beams = big ? 0 : Lp * 8 * 2 + Lp * 4;  // two key buffers and the expand list
+    const size_t beams = big ? (size_t)kBeamSampleKeys * 8 : Lp * 8 * 2 + Lp * 4;  // (big: the merge's sample) two key buffers and the expand list
     return beams + (size_t)ccap * 8 + (size_t)table_words * 4 + (size_t)tcap * 4 + (size_t)ocap * 4 +
            (size_t)((dim + 3) & ~3) * 4;
 }

@@ -506,6 +506,7 @@ static coral::SearchArgs search_args(const coral_index* idx, const coral_search_
     a.id_bits = p.id_bits, a.rem_bits = p.rem_bits, a.dmax = p.dmax, a.ocap = p.ocap;
     a.beam_stride = p.beam_stride, a.direct_bitmap = p.direct, a.table_words = p.table_words;
     a.prefetch_rows = p.prefetch;
+    a.scap = p.big ? coral::kBeamSampleKeys : 0;
     return a;
 }
 

@@ -34,11 +34,34 @@ def build_query_aware_graph(base, aux, metric="l2", **params):
     return nbrs, starts, info
 
 
+def exact_knn_graph(base, R=32, metric="l2", batch=1 << 17):
+    """Exact R-nearest-neighbour graph of the base, int32 [n][R], by the library's own brute-force kernels
+    (coral_bruteforce_knn, the stand-in for the reference's faiss calls, tests/comp_gt.cpp:119-176): every vector's
+    R + 1 nearest under (distance, id), the vector itself dropped.  n <= R gives rows padded with -1."""
+    from . import capi
+    base = np.ascontiguousarray(base, dtype=np.float32)
+    n = base.shape[0]
+    idx = capi.Index(base, None, None, metric=capi.IP if metric == "ip" else capi.L2)
+    kk = min(R + 1, n)
+    out = np.full((n, R), -1, np.int32)
+    for s in range(0, n, batch):
+        ids, _, _ = idx.bruteforce(base[s:s + batch], kk, want_dists=False)
+        own = np.arange(s, s + ids.shape[0], dtype=np.int32)[:, None]
+        # the vector itself is among its R + 1 nearest (first, unless an exact duplicate with a lower id comes before
+        # it); where it is not -- more than R duplicates -- the last entry goes instead
+        is_self = ids == own
+        is_self[~is_self.any(1), -1] = True
+        keep = ids[~is_self].reshape(ids.shape[0], kk - 1)
+        out[s:s + ids.shape[0], :kk - 1] = keep
+    idx.close()
+    return out
+
+
 def config1(device="cuda"):
     """100k x 128 N(0,I); 1k shifted queries; exact 32-NN graph; entry = medoid; k=10, L=64, L2."""
     base = gaussian_base(1001, 100000, 128)
     queries = synth.shifted_queries(1000, 128, 1002, 1003, 1004)
-    nbrs = synth.exact_knn_graph(base, 32, device=device)
+    nbrs = exact_knn_graph(base, 32)
     starts = np.array([synth.medoid_start(base)], np.int32)
     return dict(name="100k x 128 fp32 L2, exact 32-NN graph, k=10, L=64", base=base, queries=queries, nbrs=nbrs,
                 starts=starts, metric="l2", k=10, Ls=(64,))

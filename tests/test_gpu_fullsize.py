@@ -19,8 +19,9 @@ def test_full_size_properties(orc):
         list(ex.map(lambda r: synth.gaussian_matrix(2001, min(step, n - r), dim, row0=r, out=base[r:r + step]),
                     range(0, n, step)))
     q = synth.shifted_queries(Q, dim, 2002, 2003, 2004)
-    print("building the 1M exact 32-NN graph on the GPU", flush=True)
-    nbrs = synth.exact_knn_graph(base, 32, device="cuda", block=4096)
+    print("building the 1M exact 32-NN graph with the library's brute-force kernels", flush=True)
+    from coral_amd import workloads
+    nbrs = workloads.exact_knn_graph(base, 32)
     starts = np.random.RandomState(1).choice(n, 16, replace=False).astype(np.int32)
     idx = capi.Index(base, nbrs, starts)
     print("searching", flush=True)

@@ -14,7 +14,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from coral_amd import capi, formats, synth
+from coral_amd import capi, formats, synth, workloads
 from util import explain_divergence, make_queries, near_tie_equal, ragged, rounds_hand_case
 
 pytestmark = pytest.mark.gpu
@@ -24,7 +24,8 @@ WAVE64 = 3
 
 
 def gpu_graph(base, R, metric="l2"):
-    return synth.exact_knn_graph(base, R, metric=metric, device="cuda")
+    """exact R-NN graph by the library's brute-force kernels"""
+    return workloads.exact_knn_graph(base, R, metric=metric)
 
 
 def problem(n, dim, R, seed, metric="l2", n_start=16, ragged_seed=None, isolate=0):
@@ -512,7 +513,7 @@ def test_cli_end_to_end(orc, tmp_path):
     # --index_type roar replaces the graph by a RoarGraph file and searches from its entry point
     # (tests/test_search_pipeline.cpp:247-252: ../data/<dataset>/indexes/roar.index)
     os.makedirs(work / "data" / "syn" / "indexes")
-    roar = ragged(synth.exact_knn_graph(base, 32, device="cuda"), 9, keep_min=4)
+    roar = ragged(gpu_graph(base, 32), 9, keep_min=4)
     formats.roargraph_write(work / "data" / "syn" / "indexes" / "roar.index", roar, 123)
     r = subprocess.run(args + ["--index_type", "roar"], cwd=work / "cwd", capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr

@@ -5,7 +5,7 @@ shares the same block; sizes beyond the block are turned away."""
 import numpy as np
 import pytest
 
-from coral_amd import capi, synth
+from coral_amd import capi, synth, workloads
 from util import make_queries, ragged
 
 pytestmark = pytest.mark.gpu
@@ -34,7 +34,7 @@ def test_no_alloc_entry_point_equals_the_allocating_one():
     import torch
     n, dim, R = 30000, 200, 32
     base = synth.gaussian_matrix(91, n, dim)
-    nbrs = ragged(synth.exact_knn_graph(base, R, device="cuda"), 17, keep_min=1)
+    nbrs = ragged(workloads.exact_knn_graph(base, R), 17, keep_min=1)
     starts = np.random.RandomState(5).choice(n, 16, replace=False).astype(np.int32)
     mask = synth.tombstone_mask(n, 77, modulo=7)
     idx = capi.Index(base, nbrs, starts)
@@ -76,7 +76,7 @@ def test_no_alloc_entry_point_equals_the_allocating_one():
     # and a small one
     n2, dim2 = 5000, 64
     base2 = synth.gaussian_matrix(92, n2, dim2)
-    nbrs2 = synth.exact_knn_graph(base2, 16, device="cuda")
+    nbrs2 = workloads.exact_knn_graph(base2, 16)
     idx2 = capi.Index(base2, nbrs2, np.array([3, 999], np.int32))
     d_q2 = torch.from_numpy(make_queries(50, dim2, 902)).cuda()
     got = _noalloc(idx2, d_q2, 50, 20, 100, capi.POLICY_ROUNDS, False, torch)
