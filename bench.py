@@ -30,7 +30,7 @@ RECALL_TARGET = 0.90
 L_STEP = 512
 # files whose text decides what the search kernels do; profiles/search_kernels_traffic.txt names their digest
 KERNEL_SOURCES = ("coral_amd/csrc/beam_search.hip", "coral_amd/csrc/beam_search.h", "coral_amd/csrc/best_first.hip",
-                  "coral_amd/csrc/search_device.h", "coral_amd/csrc/coral_search.cpp")
+                  "coral_amd/csrc/search_device.h")
 T0 = time.time()
 
 

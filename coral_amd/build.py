@@ -24,7 +24,7 @@ DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-pa
 # host-only translation units: plain C++ that may call the HIP runtime API
 HOST = ["-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include"]
 
-LIB_SOURCES = ["beam_search.hip", "best_first.hip", "bruteforce.hip", "bruteforce_mfma.hip", "coral_search.cpp", "bruteforce_api.cpp", "start_nodes.hip",
+LIB_SOURCES = ["beam_search.hip", "best_first.hip", "best_first_long.hip", "bruteforce.hip", "bruteforce_mfma.hip", "coral_search.cpp", "bruteforce_api.cpp", "start_nodes.hip",
                "start_nodes_api.cpp", "graph_build.hip", "graph_build_api.cpp", "formats.cpp", "index_gpu.cpp", "membench.hip"]
 CLI_SOURCES = ["test_search_pipeline.cpp", "test_build_pipeline.cpp", "comp_gt.cpp", "update_compute_gt.cpp",
                "test_update.cpp"]

@@ -88,6 +88,30 @@ constexpr int kBeamSampleKeys = 512;  // LDS sample of a beam in global memory (
 
 // LDS bytes of one workgroup.  big: the beams and the expand list are in global memory, LDS holds the candidate
 // buffer, the visited structure (table_words 32-bit words), the todo list, the overflow list and the query.
+// What the wavefront-per-query best-first kernel for long beams (best_first_long.hip) needs beyond SearchArgs: the
+// visited state of BestFirstArgs, and per query slot two buffers of Lp keys in global memory for the long sorted run.
+struct BestFirstLongArgs {
+    uint8_t* visited;    // [slots][stride], as BestFirstArgs
+    uint32_t* epochs;    // [slots]
+    size_t stride;
+    uint64_t* beams;     // [slots][beam_stride]: two runs of Lp keys each
+    size_t beam_stride;  // 64-bit words per slot
+    int32_t slots;
+    int32_t rows_unique;
+    int32_t packed;
+    int32_t bcap;        // keys of the sorted insert buffer in LDS, a multiple of 64
+    int32_t scap;        // keys of the LDS sample of the long run
+    int32_t sshift;      // the sample holds every 2^sshift-th key: ((L - 1) >> sshift) + 1 <= scap
+};
+// LDS bytes of one wavefront: the insert buffer, a copy of the long run's last bcap + 32 keys, two samples, 32 candidate
+// keys, 32 ids, bcap byte counters
+__host__ __device__ inline size_t best_first_long_lds_bytes(int bcap, int scap) {
+    return ((size_t)bcap * 8 + (size_t)(bcap + 32) * 8 + (size_t)scap * 16 + 32 * 8 + 32 * 4 + (size_t)bcap + 15) &
+           ~(size_t)15;
+}
+hipError_t best_first_long_prepare(int dim, bool packed, int bcap, int scap, int* max_wg_per_cu);
+hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& b, hipStream_t stream);
+
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big);
 // 64-bit words of global scratch one workgroup of a BIG launch needs for a beam of capacity L
 size_t search_beam_stride(int L);

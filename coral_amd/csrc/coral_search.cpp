@@ -39,6 +39,7 @@ using coral::fail;
 
 constexpr int kMaxL = CORAL_MAX_BEAM;  // beams beyond CORAL_MAX_LDS_BEAM live in global memory
 constexpr int kMaxLdsBytes = 160 * 1024;
+constexpr int kLongBeamFrom = 1280;  // best-first: beams longer than this take the long-beam kernel
 
 // bits of a mixed id that a cell of the wavefront kernel's table stores: what the bucket index (a quarter of the
 // cells) does not imply; a cell has room for 14
@@ -188,6 +189,7 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_phase);
     (void)hipFree(idx->d_bf_visited);
     (void)hipFree(idx->d_bf_epochs);
+    (void)hipFree(idx->d_bf_beams);
     (void)hipFree(idx->d_bnorm);
     (void)hipFree(idx->d_bnorm_max);
     (void)hipFree(idx->d_io_q);
@@ -391,8 +393,15 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     const int id_bits = plan.id_bits;
     const int workgroups = plan.workgroups;
 
-    // the wavefront-per-query best-first kernel keeps its beam in LDS: four wavefronts of a workgroup must fit
-    const bool wave_form = best_first && !t.best_first_in_lds && !plan.big &&
+    // Best-first on one wavefront per query: with the beam in LDS (best_first.hip; four wavefronts of a workgroup must
+    // fit) or, for longer beams, with a sorted insert buffer in LDS in front of a long run in global memory
+    // (best_first_long.hip).  best_first_in_lds = 1 keeps the policy on the workgroup-per-query kernel.
+    if (t.best_first_buffer != 0 && (t.best_first_buffer < 64 || t.best_first_buffer > 4096 || t.best_first_buffer % 64))
+        return fail(CORAL_ERR_ARG, "best_first_buffer must be a multiple of 64 in 64..4096");
+    // (measured at a million nodes: the two forms cross between L = 1024 and 1536)
+    const bool long_form = best_first && !t.best_first_in_lds &&
+                           (t.best_first_long > 0 || (t.best_first_long == 0 && L > kLongBeamFrom));
+    const bool wave_form = best_first && !t.best_first_in_lds && !long_form && !plan.big &&
                            coral::best_first_wave_lds_bytes(L, 0, 0) * 4 <= (size_t)kMaxLdsBytes;
     int table_log2 = 0;
     if (wave_form)
@@ -423,25 +432,11 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         HIP_TRY(hipHostMalloc(&idx->h_counters, need_counters * sizeof(int32_t)));
         idx->counters_alloc = need_counters;
     }
-    // Best-first: one wavefront per query with the visited state in HBM (best_first.hip), when the memory for it
-    // is there: n bytes per wavefront (n / 6 in the packed form), up to a third of what is free and 64 GiB.
-    idx->bf_ready = false;
-    if (wave_form) {
-        int bf_wg_per_cu = 0;
-        const int chunks = idx->dim / 4;
-        idx->bf_table_log2 = table_log2;
-        idx->bf_table_rem_bits = table_log2 ? bf_table_rem_bits(id_bits, table_log2) : 0;
-        // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling; a
-        // launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a step
-        int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
-        if (table_log2 && coral::best_first_wave_lds_bytes(L, 0, table_log2) * 12 > (size_t)kMaxLdsBytes && chunks > 16 &&
-            chunks <= 64)
-            rif = 32;
-        idx->bf_rows_in_flight = rif;
-        // with a table the filter would only cover what outgrew it, and its LDS is worth more as cells
-        const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L);
-        idx->bf_bloom_log2 = bloom_log2;
-        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, bloom_log2, table_log2, &bf_wg_per_cu));
+    // Best-first, one wavefront per query: the visited state lives in HBM, n bytes per wavefront (n / 6 in the packed
+    // form), up to a third of what is free and 64 GiB.  wg_per_cu: what the chosen kernel's occupancy allows;
+    // reprepare(packed): sets that kernel up in the packed form and returns its occupancy.
+    idx->bf_ready = false, idx->bf_long = false;
+    auto visited_slots = [&](int bf_wg_per_cu, auto reprepare, int64_t other_bytes_per_slot) -> int {
         size_t free_b = 0, total_b = 0;
         HIP_TRY(hipMemGetInfo(&free_b, &total_b));
         const size_t budget = std::min<size_t>((free_b + idx->bf_alloc_bytes) / 3, (size_t)64 << 30);
@@ -450,12 +445,12 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const size_t stride_packed = ((((size_t)idx->n + 23) / 24 * 4) + 15) & ~(size_t)15;
         // a byte per node while that leaves every wavefront its slot, else the packed words
         const int64_t need = std::min<int64_t>(want, (int64_t)Q);
-        const int packed = t.best_first_packed || (int64_t)(budget / stride_bytes) < need ? 1 : 0;
+        const int packed = t.best_first_packed || (int64_t)(budget / (stride_bytes + other_bytes_per_slot)) < need ? 1 : 0;
         const size_t stride = packed ? stride_packed : stride_bytes;
         if (packed != idx->bf_packed) idx->bf_stride = 0;  // forces a fresh, zeroed allocation
         idx->bf_packed = packed;
-        if (packed) HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, true, bloom_log2, table_log2, &bf_wg_per_cu));
-        int slots = (int)std::min<size_t>((size_t)need, budget / stride);
+        if (packed) HIP_TRY(reprepare(&bf_wg_per_cu));
+        int slots = (int)std::min<size_t>((size_t)need, budget / (stride + other_bytes_per_slot));
         // below about four wavefronts per CU the workgroup-per-query kernel is the faster one
         if (bf_wg_per_cu > 0 && (slots >= 4 * idx->num_cu || slots >= Q || t.workgroups > 0) && slots > 0) {
             bool have = stride == idx->bf_stride && slots <= idx->bf_alloc_slots;
@@ -480,6 +475,58 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
             }
             if (have) idx->bf_slots = slots, idx->bf_ready = true;
         }
+        return CORAL_OK;
+    };
+    if (wave_form) {
+        int bf_wg_per_cu = 0;
+        const int chunks = idx->dim / 4;
+        idx->bf_table_log2 = table_log2;
+        idx->bf_table_rem_bits = table_log2 ? bf_table_rem_bits(id_bits, table_log2) : 0;
+        // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling; a
+        // launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a step
+        int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
+        if (table_log2 && coral::best_first_wave_lds_bytes(L, 0, table_log2) * 12 > (size_t)kMaxLdsBytes && chunks > 16 &&
+            chunks <= 64)
+            rif = 32;
+        idx->bf_rows_in_flight = rif;
+        // with a table the filter would only cover what outgrew it, and its LDS is worth more as cells
+        const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L);
+        idx->bf_bloom_log2 = bloom_log2;
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, bloom_log2, table_log2, &bf_wg_per_cu));
+        auto reprepare = [&](int* occ) {
+            return coral::best_first_prepare(idx->dim, L, rif, true, bloom_log2, table_log2, occ);
+        };
+        if (int rc = visited_slots(bf_wg_per_cu, reprepare, 0)) return rc;
+    } else if (long_form) {
+        // the insert buffer: 512 keys unless the caller names a size; a sample of at most 128 keys of the long run
+        const int bcap = t.best_first_buffer ? t.best_first_buffer : 512;
+        const int scap = 128;
+        int sshift = 0;
+        while ((((int64_t)L - 1) >> sshift) + 1 > scap) ++sshift;
+        if (coral::best_first_long_lds_bytes(bcap, scap) * 4 > (size_t)kMaxLdsBytes)
+            return fail(CORAL_ERR_ARG, "best_first_buffer = %d does not fit LDS", bcap);
+        int bf_wg_per_cu = 0;
+        HIP_TRY(coral::best_first_long_prepare(idx->dim, false, bcap, scap, &bf_wg_per_cu));
+        auto reprepare = [&](int* occ) { return coral::best_first_long_prepare(idx->dim, true, bcap, scap, occ); };
+        const size_t Lp = (size_t)((L + 3) & ~3);
+        const size_t beam_stride = (2 * Lp + 15) & ~(size_t)15;  // two runs of Lp keys, a multiple of 128 bytes
+        if (int rc = visited_slots(bf_wg_per_cu, reprepare, (int64_t)beam_stride * 8)) return rc;
+        if (idx->bf_ready) {
+            const size_t need = beam_stride * (size_t)idx->bf_slots;
+            if (need > idx->bf_beam_alloc_words) {
+                (void)hipFree(idx->d_bf_beams);
+                idx->d_bf_beams = nullptr, idx->bf_beam_alloc_words = 0;
+                const hipError_t e = hipMalloc(&idx->d_bf_beams, need * sizeof(uint64_t));
+                if (e == hipSuccess) {
+                    idx->bf_beam_alloc_words = need;
+                } else {
+                    (void)hipGetLastError();
+                    idx->bf_ready = false;  // the workgroup-per-query kernel serves the policy
+                }
+            }
+        }
+        idx->bf_long = idx->bf_ready;
+        idx->bf_bcap = bcap, idx->bf_scap = scap, idx->bf_sshift = sshift, idx->bf_beam_stride = beam_stride;
     }
     HIP_TRY(hipStreamSynchronize(idx->stream));
     idx->Q = Q, idx->L = L, idx->plan = plan;
@@ -552,7 +599,16 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
 #endif
     // timed region, same scope as the reference: kernel + counter read-back
     HIP_TRY(hipEventRecord(ev0, stream));
-    if (wave_kernel) {
+    if (wave_kernel && idx->bf_long) {
+        coral::BestFirstLongArgs b;
+        std::memset(&b, 0, sizeof b);
+        b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
+        b.beams = idx->d_bf_beams, b.beam_stride = idx->bf_beam_stride;
+        b.slots = std::min(idx->bf_slots, (int)Q);
+        b.rows_unique = idx->rows_unique == 1, b.packed = idx->bf_packed;
+        b.bcap = idx->bf_bcap, b.scap = idx->bf_scap, b.sshift = idx->bf_sshift;
+        HIP_TRY(coral::launch_best_first_long(a, b, stream));
+    } else if (wave_kernel) {
         coral::BestFirstArgs b;
         b.rows_unique = idx->rows_unique == 1;
         b.packed = idx->bf_packed;

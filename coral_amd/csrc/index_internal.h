@@ -78,6 +78,11 @@ struct coral_index {
     size_t bf_stride = 0, bf_alloc_bytes = 0;
     int bf_slots = 0, bf_alloc_slots = 0, bf_rows_in_flight = 8, bf_packed = 0, bf_bloom_log2 = 0;
     int bf_table_log2 = 0, bf_table_rem_bits = 0;
+    // ... or, for long beams, with an insert buffer in LDS and the long sorted run of every slot in global memory
+    bool bf_long = false;
+    uint64_t* d_bf_beams = nullptr;
+    size_t bf_beam_alloc_words = 0, bf_beam_stride = 0;
+    int bf_bcap = 0, bf_scap = 0, bf_sshift = 0;
     int rows_unique = -1;  // 1: no graph row lists an id twice, 0: some do, -1: not looked at since the rows changed
     // the tuning of the last prepare, and what the searches since have taught about the visited table:
     // at beam capacity bump_L the library's own choice of table size is raised by bump_log2

@@ -118,6 +118,11 @@ typedef struct {
                                    0 = where a workgroup has its CU to itself */
     int32_t cand_cap;           /* capacity of the candidate buffer in LDS (a power of two, at least the todo list's);
                                    0 = chosen */
+    int32_t best_first_long;    /* best-first with a wavefront per query keeps beams up to 1280 entries in LDS and longer
+                                   ones as a sorted insert buffer in LDS in front of a long run in global memory (two
+                                   runs of L keys per query slot): 1 = that form whatever L is, -1 = never (beams
+                                   beyond CORAL_MAX_LDS_BEAM then run on the workgroup-per-query kernel), 0 = by L */
+    int32_t best_first_buffer;  /* keys of that insert buffer, a multiple of 64 in 64..4096; 0 = 512 */
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);

@@ -22,7 +22,8 @@ pytestmark = pytest.mark.gpu
 
 # every form the best-first policy takes on the GPU
 FORMS = (dict(), dict(best_first_packed=True), dict(best_first_in_lds=True), dict(best_first_table_log2=-1),
-         dict(best_first_table_log2=8), dict(beam_in_hbm=True))
+         dict(best_first_table_log2=8), dict(best_first_in_lds=True, beam_in_hbm=True), dict(best_first_long=1),
+         dict(best_first_long=1, best_first_buffer=64))
 
 
 @pytest.mark.parametrize("name", golden_cases())

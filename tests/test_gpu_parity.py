@@ -83,15 +83,18 @@ def test_exact_against_same_order_oracle(orc, case):
     else:
         oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=m, order=WAVE64)
     idx = capi.Index(base, nbrs, starts, m)
-    # best-first has two kernels: a wavefront per query (visited state in HBM, a byte per node or packed words) and a
-    # workgroup per query (LDS table)
-    # workgroup per query (LDS table); the wavefront form keeps the first visits in an exact table in LDS where the
-    # beam leaves room (chosen by the library, none, or a small one that overflows into the state in HBM)
-    forms = ((False, False, 0), (False, True, 0), (True, False, 0), (False, False, -1), (False, True, 8),
-             (False, False, 9)) if policy == 1 else ((False, False, 0),)
-    for in_lds, packed, table in forms:
-        idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy,
-                    best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=table)
+    # best-first has three kernels: a wavefront per query with the beam in LDS (visited state in HBM, a byte per node
+    # or packed words; the first visits in an exact table in LDS where the beam leaves room -- chosen by the library,
+    # none, or a small one that overflows into the state in HBM), a wavefront per query with an insert buffer in LDS
+    # in front of a long run in global memory (the form of long beams; a tiny buffer merges into the run all the
+    # time), and a workgroup per query (visited set in LDS)
+    forms = (dict(), dict(best_first_packed=True), dict(best_first_in_lds=True), dict(best_first_table_log2=-1),
+             dict(best_first_packed=True, best_first_table_log2=8), dict(best_first_table_log2=9),
+             dict(best_first_long=1), dict(best_first_long=1, best_first_buffer=64, best_first_packed=True),
+             dict(best_first_long=1, best_first_buffer=192)) if policy == 1 else (dict(),)
+    for form in forms:
+        in_lds = form.get("best_first_in_lds", False)
+        idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy, **form)
         ids, dists, st = idx.search(q, k, L, policy=policy)
         cnt = idx.query_counters(q.shape[0])
         assert np.array_equal(ids, oi)
@@ -143,17 +146,23 @@ def test_beams_in_global_memory_equal_the_oracle(orc, case):
     idx = capi.Index(base, nbrs, starts, m)
     if dele:
         idx.set_deleted(mask)
-    idx.prepare(Q, L, visited_slots_log2=slots, workgroups=wgs, policy=policy, beam_in_hbm=True)
-    ids, dists, st = idx.search(q, k, L, policy=policy, have_delete=dele)
-    cnt = idx.query_counters(Q)
-    assert np.array_equal(ids, oi)
-    assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist()
-    assert np.array_equal(cnt, os_)
-    if slots:
-        assert st.spills > 0
-    # the same call again on the workgroups' used beam blocks and bitmaps
-    ids2, dists2, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
-    assert np.array_equal(ids2, oi) and dists2.tobytes() == od.tobytes()
+    # the workgroup-per-query kernel with its beams in global memory; for best-first also the wavefront-per-query
+    # kernel of long beams (an insert buffer in LDS in front of a long run in global memory), which is what the library
+    # picks for that policy beyond CORAL_MAX_LDS_BEAM
+    forms = (dict(best_first_in_lds=True), dict(best_first_long=1), dict(best_first_long=1, best_first_buffer=128)) \
+        if policy == 1 else (dict(),)
+    for form in forms:
+        idx.prepare(Q, L, visited_slots_log2=slots, workgroups=wgs, policy=policy, beam_in_hbm=True, **form)
+        ids, dists, st = idx.search(q, k, L, policy=policy, have_delete=dele)
+        cnt = idx.query_counters(Q)
+        assert np.array_equal(ids, oi), form
+        assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), form
+        assert np.array_equal(cnt, os_), form
+        if slots and not form.get("best_first_long"):
+            assert st.spills > 0
+        # the same call again on the used beam blocks and bitmaps
+        ids2, dists2, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
+        assert np.array_equal(ids2, oi) and dists2.tobytes() == od.tobytes(), form
     if L <= capi.MAX_LDS_BEAM:  # and the form with the beam in LDS agrees
         idx.prepare(Q, L, policy=policy, best_first_in_lds=True)
         ids3, dists3, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
@@ -257,10 +266,12 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         idx = capi.Index(base, nbrs, starts, m)
         if dele:
             idx.set_deleted(mask)
-        for in_lds, packed in (((False, False), (False, True), (True, False)) if policy == 1 else ((False, False),)):
+        longb = int(rng.choice([64, 128, 512]))  # insert buffer of the long-beam form of best-first
+        for in_lds, packed, long_ in (((False, False, 0), (False, True, 0), (True, False, 0), (False, False, 1),
+                                       (False, True, 1)) if policy == 1 else ((False, False, 0),)):
             idx.prepare(Q, L, visited_slots_log2=slots, threads=threads, workgroups=wgs, policy=policy,
                         best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=tbl,
-                        beam_in_hbm=big, prefetch_rows=ahead)
+                        beam_in_hbm=big, prefetch_rows=ahead, best_first_long=long_, best_first_buffer=longb)
             ids, dists, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
             assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
             assert np.array_equal(idx.query_counters(Q), os_)
