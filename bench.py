@@ -30,7 +30,7 @@ RECALL_TARGET = 0.90
 L_STEP = 512
 # files whose text decides what the search kernels do; profiles/search_kernels_traffic.txt names their digest
 KERNEL_SOURCES = ("coral_amd/csrc/beam_search.hip", "coral_amd/csrc/beam_search.h", "coral_amd/csrc/best_first.hip",
-                  "coral_amd/csrc/search_device.h")
+                  "coral_amd/csrc/best_first_long.hip", "coral_amd/csrc/search_device.h")
 T0 = time.time()
 
 
@@ -479,16 +479,19 @@ def main():
                                      "%.4f)" % (head["L"], head["recall"], cpu["L"], cpu["recall"])
 
             def same_policy():
-                # the CPU path's traversal on the GPU at the CPU's beam, on a slice the kernel finishes in seconds
-                r = b.measure(cpu["L"], 1, 0, capi.POLICY_BEST_FIRST, Q=min(Q, 1024))
-                r["kernel"] = "beam_search_kernel (policy 1, beam in global memory)" if cpu["L"] > capi.MAX_LDS_BEAM \
-                    else "best_first_wave_kernel"
+                # the CPU path's traversal on the GPU at the CPU's beam, the whole batch
+                r = b.measure(cpu["L"], 2, 1, capi.POLICY_BEST_FIRST)
+                r["kernel"] = "best_first_long_kernel" if cpu["L"] > 1280 else "best_first_wave_kernel"
                 return r
             bf = optional(same_policy)
             if bf and "qps" in bf:
                 out["best_first"] = slim(bf)
                 out["best_first"]["kernel"] = bf["kernel"]
+                tr = measured_traffic(bf["kernel"], bf["L"], "best_first")
+                out["best_first"]["traffic"] = tr["bytes"] if tr else None
                 out["gpu_over_cpu_same_policy"] = bf["qps"] / cpu["value"]
+                out["gpu_over_cpu_same_policy_is"] = "best_first (GPU, L=%d, recall %.4f) / cpu_baseline (same beam)" % \
+                                                     (bf["L"], bf["recall"])
     # equal policy at the configuration's L = 512 (the wavefront-per-query kernel against the CPU at the same beam)
     bf512 = optional(b.measure, 512, 3, 1, capi.POLICY_BEST_FIRST)
     if bf512 and "qps" in bf512:
