@@ -43,7 +43,8 @@ class Tuning(C.Structure):
     _fields_ = [("visited_slots_log2", C.c_int32), ("workgroups", C.c_int32), ("threads", C.c_int32),
                 ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("best_first_packed", C.c_int32),
                 ("best_first_table_log2", C.c_int32), ("beam_in_hbm", C.c_int32), ("prefetch_rows", C.c_int32),
-                ("cand_cap", C.c_int32), ("best_first_long", C.c_int32), ("best_first_buffer", C.c_int32)]
+                ("cand_cap", C.c_int32), ("best_first_long", C.c_int32), ("best_first_buffer", C.c_int32),
+                ("screening", C.c_int32)]
 
 
 class BuildParams(C.Structure):
@@ -211,10 +212,10 @@ class Index:
 
     def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False,
                 best_first_packed=False, best_first_table_log2=0, beam_in_hbm=False, prefetch_rows=0, cand_cap=0,
-                best_first_long=0, best_first_buffer=0):
+                best_first_long=0, best_first_buffer=0, screening=0):
         t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)),
                    int(bool(best_first_packed)), best_first_table_log2, int(bool(beam_in_hbm)), prefetch_rows,
-                   cand_cap, best_first_long, best_first_buffer)
+                   cand_cap, best_first_long, best_first_buffer, screening)
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

@@ -41,6 +41,11 @@ struct SearchArgs {
     // the visited set is a plain bitmap of the n ids in LDS (table_words 32-bit words) instead of the table of
     // 16-bit cells; no id ever goes to the bitmap in global memory then
     int32_t direct_bitmap;
+    // screening: a half-precision copy of the vectors (rows stride16 bytes apart, the row's norm behind its halves), or
+    // nullptr; tcap2 = entries of the list of rows it leaves for the exact pass (tcap, or 0 without screening)
+    const unsigned char* vec16;
+    size_t stride16;
+    int32_t tcap2;
     int32_t scap;              // BIG form: keys of the LDS sample of the beam that the merge searches first
     int32_t prefetch_rows;     // request a chunk's graph rows one chunk ahead (launches with one workgroup per CU)
     int32_t table_words;       // 32-bit words of LDS the visited structure takes (cells / 2, or ceil(n / 32) rounded up to 4)
@@ -112,7 +117,10 @@ __host__ __device__ inline size_t best_first_long_lds_bytes(int bcap, int scap) 
 hipError_t best_first_long_prepare(int dim, bool packed, int bcap, int scap, int* max_wg_per_cu);
 hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& b, hipStream_t stream);
 
-size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big);
+size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening);
+// the half-precision copy of the vectors that the screening phase reads: bytes per row, and its construction
+size_t half_row_stride(int dim);
+hipError_t launch_half_rows(const float* vec, int64_t n, int dim, unsigned char* out, hipStream_t stream);
 // 64-bit words of global scratch one workgroup of a BIG launch needs for a beam of capacity L
 size_t search_beam_stride(int L);
 hipError_t search_kernel_prepare(int dim, bool big, size_t lds_bytes, int threads, int* max_wg_per_cu);

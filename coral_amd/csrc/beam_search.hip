@@ -26,6 +26,7 @@
 // group of G lanes accumulates float4 chunks l, l+G, ... with four fused
 // multiply-adds per chunk in x,y,z,w order; partials are combined by a butterfly
 // p[l] += p[l^off], off = 1, 2, 4, ..., G/2.
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     const int TCAP = a.tcap, CCAP = a.ccap;
 
     uint64_t *beam0, *beam1, *cand, *samp = nullptr;
-    uint32_t *table, *todo, *elist, *olist;
+    uint32_t *table, *todo, *todo2, *elist, *olist;
     if constexpr (BIG) {
         uint64_t* g = a.beam_scratch + (size_t)blockIdx.x * a.beam_stride;
         beam0 = g, beam1 = g + Lp, elist = (uint32_t*)(g + 2 * (size_t)Lp);
@@ -152,19 +153,21 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         samp = cand + CCAP;                     // a sample of the beam's keys for the merge's searches
         table = (uint32_t*)(samp + a.scap);     // 16-bit cells, or the bitmap of all ids
         todo = table + a.table_words;
-        olist = todo + TCAP;
+        todo2 = todo + TCAP;
+        olist = todo2 + a.tcap2;
     } else {
         beam0 = (uint64_t*)smem;
         beam1 = beam0 + Lp;
         cand = beam1 + Lp;
         table = (uint32_t*)(cand + CCAP);  // slots 16-bit cells
         todo = table + a.table_words;
-        elist = todo + TCAP;
+        todo2 = todo + TCAP;
+        elist = todo2 + a.tcap2;
         olist = elist + Lp;
     }
     float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ncand, s_nexp, s_cntf, s_nvis, s_cursor, s_nover;
+    __shared__ int s_qid, s_ntodo, s_ntodo2, s_ncand, s_nexp, s_cntf, s_nvis, s_cursor, s_nover;
     __shared__ int s_wcnt[16];
 
     VisitedSet vs;
@@ -207,15 +210,123 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         int hops = 0, nd = 0, ne = 0, rounds = 0;
         bool spill = false;
 
-        // ---- distance phase: todo[0..T) -> cand[], counting passes of the frozen threshold
-        auto distance_phase = [&](int T) {
+        // ---- screening phase (launches with a half-precision copy of the vectors): todo[0..T) -> todo2[0..s_ntodo2)
+        //
+        // Most ids a long search measures fail the round's frozen threshold.  Each row is first measured in its
+        // half-precision copy (half the bytes; 512-byte rows that start on a cache line).  From that distance d16, the
+        // norm of the row |x| (stored behind it) and the rounding bound of the format, |x - half(x)| <= 2^-11 |x|,
+        // the exact distance d lies in [(sqrt(d16) - r)^2, (sqrt(d16) + r)^2], r = 2^-11 |x| (taken a little larger,
+        // and both ends widened by 1e-4 to cover the fp32 rounding of either computation).  A row whose whole
+        // interval lies beyond the frozen threshold is no candidate whatever its exact distance; one whose interval
+        // lies below the threshold and beyond the beam's current worst entry is a candidate that is counted and
+        // cannot enter the beam.  Only the rest -- possible beam entries and rows within 0.1 % of the threshold --
+        // have their fp32 row read, by the distance phase below; results and counters are what they are without
+        // the screening, bit for bit.
+        auto screening_phase = [&](int T) {
+            if constexpr (G == 64) {
+                constexpr int RPIH = 2 * U;  // two groups of 32 lanes per wave, U rows in flight per group
+                const int glh = lane & 31, grph = lane >> 5;
+                const int chunksH = (dim + 7) >> 3;  // 16-byte chunks of eight halves
+                float4 qa[CPL][2];
+#pragma unroll
+                for (int t = 0; t < CPL; ++t) {
+                    const int c = 2 * (glh + 32 * t);
+                    qa[t][0] = c < chunks ? reinterpret_cast<const float4*>(qs)[c] : make_float4(0, 0, 0, 0);
+                    qa[t][1] = c + 1 < chunks ? reinterpret_cast<const float4*>(qs)[c + 1] : make_float4(0, 0, 0, 0);
+                }
+                const float s_live = st.live == kKeyMax ? 3.402823466e+38f : key_s(st.live);
+                int cnt = 0;
+                for (int base = wave * RPIH; base < T; base += NW * RPIH) {
+                    int vid[U];
+                    const int r0 = base + grph * U;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if (r0 + u >= T) vid[u] = -1;
+                    uint4 h[U][CPL];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const uint4* row = reinterpret_cast<const uint4*>(
+                            a.vec16 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * a.stride16);
+#pragma unroll
+                        for (int t = 0; t < CPL; ++t) {
+                            const int c = glh + 32 * t;
+                            h[u][t] = (vid[u] >= 0 && c < chunksH) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
+                        }
+                    }
+                    // the row this lane will file, and its norm
+                    int myid = vid[0];
+#pragma unroll
+                    for (int u = 1; u < U; ++u)
+                        if ((lane & (U - 1)) == u) myid = vid[u];
+                    const bool valid = glh < U && myid >= 0;
+                    float nx = 0.0f;
+                    if (valid)
+                        nx = *reinterpret_cast<const float*>(a.vec16 + (uint64_t)(uint32_t)myid * a.stride16 +
+                                                             (size_t)chunksH * 16);
+                    float acc[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < CPL; ++t) {
+                            const __half2* hp = reinterpret_cast<const __half2*>(&h[u][t]);
+                            const float2 x0 = __half22float2(hp[0]), x1 = __half22float2(hp[1]);
+                            const float2 x2 = __half22float2(hp[2]), x3 = __half22float2(hp[3]);
+                            float d;
+                            d = qa[t][0].x - x0.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][0].y - x0.y, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][0].z - x1.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][0].w - x1.y, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].x - x2.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].y - x2.y, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].z - x3.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].w - x3.y, sum = __fmaf_rn(d, d, sum);
+                        }
+                        acc[u] = sum;
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        acc[u] = acc[u] + dpp_mov<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
+                        acc[u] = acc[u] + dpp_mov<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
+                        acc[u] = acc[u] + dpp_mov<0x141>(acc[u]);  // row_half_mirror
+                        acc[u] = acc[u] + dpp_mov<0x140>(acc[u]);  // row_mirror
+                    }
+                    float mine = acc[0];
+#pragma unroll
+                    for (int u = 1; u < U; ++u)
+                        if ((lane & (U - 1)) == u) mine = acc[u];
+                    mine = mine + __shfl_xor(mine, 16, 64);
+                    const float root = sqrtf(mine), r = 5.0e-4f * nx + 1.0e-6f;
+                    const float lo_root = fmaxf(root - r, 0.0f), hi_root = root + r;
+                    const float lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
+                    // (a row with a component beyond the half format has an infinite norm: lo = 0, hi = inf)
+                    const bool gone = valid && lo > thr;
+                    const bool counted = valid && !gone && hi < thr && lo > s_live;
+                    const bool exact = valid && !gone && !counted;
+                    cnt += __popcll(__ballot(counted));
+                    const uint64_t m = __ballot(exact);
+                    if (m) {
+                        int pos = 0;
+                        if (lane == 0) pos = atomicAdd(&s_ntodo2, __popcll(m));
+                        pos = __shfl(pos, 0, 64);
+                        if (exact) todo2[pos + prefix_popc(m)] = (uint32_t)myid;
+                    }
+                }
+                if (lane == 0 && cnt) atomicAdd(&s_cntf, cnt);
+            }
+        };
+
+        // ---- distance phase: list[0..T) -> cand[], counting passes of the frozen threshold
+        auto distance_phase = [&](const uint32_t* list, int T) {
             int cntf = 0;
             for (int base = wave * RPI; base < T; base += NW * RPI) {
                 // all ids of this iteration first (one LDS wait), then all row requests back to back
                 int vid[U];
                 const int r0 = base + grp * U;
 #pragma unroll
-                for (int u = 0; u < U; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
+                for (int u = 0; u < U; ++u) vid[u] = (int)list[r0 + u];  // inside the list's capacity
 #pragma unroll
                 for (int u = 0; u < U; ++u)
                     if (r0 + u >= T) vid[u] = -1;
@@ -431,7 +542,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             todo[i] = id;
         }
         __syncthreads();
-        distance_phase(M);
+        distance_phase(todo, M);
         merge();
         PHASE_MARK(1);
         if (tid == 0) s_nvis = M, s_cntf = 0;
@@ -550,7 +661,16 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     if (pe < ech && e1 + pe < nexp) vpre = a.nbrs[(size_t)epre * R + pj];
                     if (pe < ech && e2 + pe < nexp) epre = elist[e2 + pe];
                 }
-                distance_phase(T);
+                if (a.vec16 != nullptr && a.policy == 0) {
+                    if (tid == 0) s_ntodo2 = 0;
+                    __syncthreads();
+                    screening_phase(T);
+                    __syncthreads();
+                    PHASE_MARK(7);
+                    distance_phase(todo2, s_ntodo2);
+                } else {
+                    distance_phase(todo, T);
+                }
                 __syncthreads();
                 PHASE_MARK(4);
             }
@@ -686,8 +806,9 @@ static kernel_fn pick_kernel(int dim, bool big) {
     return big ? pick_kernel_form<true>(dim / 4) : pick_kernel_form<false>(dim / 4);
 }
 
-size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big) {
+size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening) {
     const size_t Lp = (size_t)((L + 3) & ~3);
+    if (screening) tcap *= 2;  // the list of rows the screening leaves for the exact pass
     const size_t beams = big ? (size_t)kBeamSampleKeys * 8 : Lp * 8 * 2 + Lp * 4;  // (big: the merge's sample) two key buffers and the expand list
     return beams + (size_t)ccap * 8 + (size_t)table_words * 4 + (size_t)tcap * 4 + (size_t)ocap * 4 +
            (size_t)((dim + 3) & ~3) * 4;
@@ -745,6 +866,41 @@ hipError_t static_scratch_init(int device) {
 void* static_scratch(int device) {
     if (device < 0 || device >= kMaxDevices) return nullptr;
     return __atomic_load_n(&g_scratch_ptr[device], __ATOMIC_ACQUIRE);
+}
+
+// Half-precision copy of the vectors for the screening phase: row i = dim halves (round to nearest), zero padding up
+// to a whole 16-byte chunk, then |x_i| as a float (rounded up a little; infinite when a component does not fit the
+// format, which sends the row to the exact pass every time), rows `stride` bytes apart.
+__global__ __launch_bounds__(256) void half_rows_kernel(const float* __restrict__ vec, int64_t n, int dim,
+                                                        unsigned char* __restrict__ out, size_t stride) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    const int padded = (dim + 7) & ~7;
+    for (int64_t row = wave; row < n; row += nwaves) {
+        const float* x = vec + row * dim;
+        __half* h = reinterpret_cast<__half*>(out + (size_t)row * stride);
+        float sum = 0.0f;
+        bool bad = false;
+        for (int j = lane; j < padded; j += 64) {
+            const float v = j < dim ? x[j] : 0.0f;
+            h[j] = __float2half_rn(v);
+            sum = __fmaf_rn(v, v, sum);
+            bad |= !(fabsf(v) <= 65504.0f);
+        }
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        bad = __ballot(bad) != 0ull;
+        if (lane == 0)
+            *reinterpret_cast<float*>(out + (size_t)row * stride + (size_t)padded * 2) =
+                bad ? __int_as_float(0x7f800000) : sqrtf(sum) * (1.0f + 1.0e-5f);
+    }
+}
+
+size_t half_row_stride(int dim) { return ((size_t)((dim + 7) & ~7) * 2 + 4 + 127) & ~(size_t)127; }
+
+hipError_t launch_half_rows(const float* vec, int64_t n, int dim, unsigned char* out, hipStream_t stream) {
+    hipLaunchKernelGGL(half_rows_kernel, dim3(4096), dim3(256), 0, stream, vec, n, dim, out, half_row_stride(dim));
+    return hipGetLastError();
 }
 
 hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,

@@ -183,6 +183,7 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_deleted);
     (void)hipFree(idx->d_spill);
     (void)hipFree(idx->d_beam);
+    (void)hipFree(idx->d_vec16);
     (void)hipFree(idx->d_counters);
     (void)hipFree(idx->d_scalars);
     (void)hipFree(idx->d_hit);
@@ -255,7 +256,7 @@ int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* 
 // Launch geometry of the workgroup-per-query kernel for a beam of capacity L: arithmetic, the kernel's LDS
 // attribute and an occupancy query; nothing is allocated.  bump_log2 raises the library's own choice of table size.
 static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral_tuning& t, int bump_log2,
-                       bool lds_beam_only, coral_search_plan* out) {
+                       bool lds_beam_only, bool no_screen, coral_search_plan* out) {
     if (Q <= 0) return fail(CORAL_ERR_ARG, "Q must be positive");
     if (L <= 0 || L > kMaxL) return fail(CORAL_ERR_ARG, "L must be in 1..%d (got %d)", kMaxL, L);
     if (idx->M <= 0) return fail(CORAL_ERR_STATE, "the graph has no start ids yet (rows under construction)");
@@ -273,16 +274,22 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     int id_bits = 1;
     while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
     const size_t lds_max = (size_t)kMaxLdsBytes;
+    // ---- screening in half precision (rounds policy, L2, rows of 132 .. 2048 floats): see beam_search.hip
+    const bool screen_possible = !best_first && idx->metric == CORAL_L2 && idx->dim / 4 > 32;
+    if (t.screening > 0 && !screen_possible)
+        return fail(CORAL_ERR_ARG, "screening needs the rounds policy, the L2 metric and more than 128 dimensions");
+    const bool screen = t.screening > 0 || (t.screening == 0 && screen_possible && !no_screen);
+    p.screen = screen;
     // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
     // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
     // -1, or the library's choice): one LDS atomic per test and nothing ever overflows, at n / 8 bytes -- 125 KB for
     // a million nodes, which leaves a CU one workgroup.
     const int bitmap_words = (int)(((idx->n + 31) / 32 + 3) & ~(int64_t)3);
     auto lds_bitmap = [&](bool big, int cap) {
-        return coral::search_lds_bytes(L, idx->dim, bitmap_words, cap, cap, 4, big) + 64;
+        return coral::search_lds_bytes(L, idx->dim, bitmap_words, cap, cap, 4, big, screen) + 64;
     };
     auto lds_table = [&](bool big, int lg, int cap) {
-        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, 256, big) + 64;
+        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, 256, big, screen) + 64;
     };
     const bool bitmap_possible = idx->n <= ((int64_t)1 << 21);
     int slots_log2 = t.visited_slots_log2;
@@ -338,7 +345,7 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     // hold; a launch that is alone on its CU anyway takes a candidate buffer of twice the size where there is room
     // (half as many merges of a long beam).  Best-first expands one row at a time and needs neither.
     auto lds_for = [&](int tc, int cc) {
-        return coral::search_lds_bytes(L, idx->dim, p.table_words, tc, cc, ocap, p.big) + 64;
+        return coral::search_lds_bytes(L, idx->dim, p.table_words, tc, cc, ocap, p.big, screen) + 64;
     };
     if (lds_for(min_cap, min_cap) > lds_max)
         return fail(CORAL_ERR_ARG, "L=%d with %d words of visited state needs %zu bytes of LDS", L, p.table_words,
@@ -365,7 +372,7 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         threads = p.big ? 1024 : best_first ? 256 : (lds_for(tcap, ccap) > lds_max / 2 ? 1024 : 512);
     if (threads != 128 && threads != 256 && threads != 512 && threads != 1024)
         return fail(CORAL_ERR_ARG, "threads must be 128, 256, 512 or 1024");
-    p.lds_bytes = coral::search_lds_bytes(L, idx->dim, p.table_words, tcap, ccap, ocap, p.big);
+    p.lds_bytes = coral::search_lds_bytes(L, idx->dim, p.table_words, tcap, ccap, ocap, p.big, screen);
     int wg_per_cu = 0;
     HIP_TRY(coral::search_kernel_prepare(idx->dim, p.big, p.lds_bytes, threads, &wg_per_cu));
     if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
@@ -387,7 +394,32 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     if (tuning) t = *tuning;
     HIP_TRY(hipSetDevice(idx->device));
     coral_search_plan plan;
-    if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, false, &plan)) return rc;
+    // The screening phase needs a half-precision copy of the vectors (5/8 of their memory at dim 200), made once per
+    // index; where the library chooses by itself and the memory is not to be had, the search runs without.
+    auto ensure_vec16 = [&]() -> hipError_t {
+        if (idx->d_vec16) return hipSuccess;
+        const size_t bytes = coral::half_row_stride(idx->dim) * (size_t)idx->n;
+        unsigned char* p = nullptr;
+        hipError_t e = hipMalloc(&p, bytes);
+        if (e != hipSuccess) return e;
+        e = hipMemsetAsync(p, 0, bytes, idx->stream);
+        if (e == hipSuccess) e = coral::launch_half_rows(idx->d_vec, idx->n, idx->dim, p, idx->stream);
+        if (e == hipSuccess)
+            idx->d_vec16 = p;
+        else
+            (void)hipFree(p);
+        return e;
+    };
+    if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, false, false, &plan)) return rc;
+    if (plan.screen) {
+        const hipError_t e = ensure_vec16();
+        if (e == hipErrorOutOfMemory && t.screening == 0) {
+            (void)hipGetLastError();
+            if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, false, true, &plan)) return rc;
+        } else {
+            HIP_TRY(e);
+        }
+    }
     HIP_TRY(hipStreamSynchronize(idx->stream));
     const bool best_first = t.policy == CORAL_POLICY_BEST_FIRST;
     const int id_bits = plan.id_bits;
@@ -553,6 +585,8 @@ static coral::SearchArgs search_args(const coral_index* idx, const coral_search_
     a.id_bits = p.id_bits, a.rem_bits = p.rem_bits, a.dmax = p.dmax, a.ocap = p.ocap;
     a.beam_stride = p.beam_stride, a.direct_bitmap = p.direct, a.table_words = p.table_words;
     a.prefetch_rows = p.prefetch;
+    a.vec16 = p.screen ? idx->d_vec16 : nullptr, a.stride16 = coral::half_row_stride(idx->dim);
+    a.tcap2 = p.screen ? p.tcap : 0;
     a.scap = p.big ? coral::kBeamSampleKeys : 0;
     return a;
 }
@@ -640,9 +674,10 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         HIP_TRY(hipMemcpy(t, idx->d_phase, sizeof t, hipMemcpyDeviceToHost));
         double sum = 0;
         for (int i = 0; i < 7; ++i) sum += (double)t[i];
-        std::fprintf(stderr, "[phase %%] init %.1f seeds %.1f elist %.1f expand %.1f distance %.1f merge %.1f output %.1f\n",
-                     100 * t[0] / sum, 100 * t[1] / sum, 100 * t[2] / sum, 100 * t[3] / sum, 100 * t[4] / sum,
-                     100 * t[5] / sum, 100 * t[6] / sum);
+        sum += (double)t[7];
+        std::fprintf(stderr, "[phase %%] init %.1f seeds %.1f elist %.1f expand %.1f screening %.1f distance %.1f merge %.1f output %.1f\n",
+                     100 * t[0] / sum, 100 * t[1] / sum, 100 * t[2] / sum, 100 * t[3] / sum, 100 * t[7] / sum,
+                     100 * t[4] / sum, 100 * t[5] / sum, 100 * t[6] / sum);
     }
 #endif
     idx->last_Q = Q;
@@ -697,8 +732,9 @@ int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* 
     coral_tuning t;
     std::memset(&t, 0, sizeof t);
     t.policy = policy;  // both policies run on the workgroup-per-query kernel here
+    t.screening = -1;   // (the half-precision copy of the vectors is made by coral_search_prepare)
     coral_search_plan plan;
-    if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, &plan)) return rc;
+    if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, /*no_screen*/ true, &plan)) return rc;
     // the block: 256 bytes of scalars, the per-query counters, then one overflow bitmap per workgroup
     int* scal = reinterpret_cast<int*>(base);
     int32_t* counters = reinterpret_cast<int32_t*>(base + 256);
