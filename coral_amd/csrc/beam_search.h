@@ -65,15 +65,18 @@ struct BestFirstArgs {
     // buckets of four; rem_bits = the bits of the mixed id (id_bits wide) that a cell stores, at most 14; what
     // finds its two buckets full goes to the state in HBM
     int32_t table_log2, id_bits, rem_bits;
+    // screening: the half-precision copy of the vectors (see SearchArgs), or nullptr
+    const unsigned char* vec16;
+    size_t stride16;
 };
 
-// LDS bytes of one wavefront: a beam of L keys, 32 candidate keys, 32 ids, L byte counters, a Bloom filter of
+// LDS bytes of one wavefront: a beam of L keys, 32 candidate keys, two lists of 32 ids, L byte counters, a Bloom filter of
 // 2^bloom_log2 bits over the visited ids in HBM (bloom_log2 = 0: none) and a table of 2^table_log2 16-bit cells
 // (table_log2 = 0: none)
 __host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2, int table_log2 = 0) {
     const size_t bloom = bloom_log2 ? ((size_t)1 << bloom_log2) / 8 : 0;
     const size_t table = table_log2 ? (size_t)2 << table_log2 : 0;
-    return ((size_t)((L + 3) & ~3) * 9 + 32 * 8 + 32 * 4 + bloom + table + 15) & ~(size_t)15;
+    return ((size_t)((L + 3) & ~3) * 9 + 32 * 8 + 2 * 32 * 4 + bloom + table + 15) & ~(size_t)15;
 }
 // the filter size for a beam of L: 128 bits per beam entry rounded up to a power of two, halved while that would leave
 // a CU fewer than sixteen wavefronts; none below 4096 bits
@@ -83,8 +86,8 @@ __host__ inline int best_first_bloom_log2(int L) {
     while (lg >= 12 && best_first_wave_lds_bytes(L, lg) > (size_t)10 * 1024) --lg;
     return lg >= 12 ? lg : 0;
 }
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int table_log2,
-                              int* max_wg_per_cu);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, bool screen, int bloom_log2,
+                              int table_log2, int* max_wg_per_cu);
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice
 hipError_t launch_find_repeated_ids(const int32_t* nbrs, int64_t n, int R, uint32_t* flag, hipStream_t stream);

@@ -24,6 +24,7 @@
 //
 // The arithmetic is that of beam_search.hip (same lane-strided accumulation, same butterfly, same 64-bit keys), so
 // results and counters are identical bit for bit; a wavefront needs no workgroup barrier anywhere.
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -36,6 +37,7 @@ namespace {
 
 constexpr int kWavesPerWg = 4;
 constexpr int kBatch = 32;  // ids measured and merged at a time (a graph row has at most 32)
+constexpr int kScreenRows = 8;  // half-precision rows in flight per group of 32 lanes in the screening phase
 
 __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -57,7 +59,8 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
 
 // PACKED: the visited state of a slot is one 32-bit word per 24 nodes (8 bits of epoch, 24 flags) instead of one
 // byte per node: a sixth of the memory, the same one line per test.
-template <int G, int CPL, int RIF, bool PACKED>
+// SCREEN: rows are measured in the half-precision copy of the vectors first (b.vec16; rows of more than 128 floats).
+template <int G, int CPL, int RIF, bool PACKED, bool SCREEN>
 __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -69,7 +72,8 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
     uint64_t* beam = reinterpret_cast<uint64_t*>(mine_lds);      // L keys, sorted
     uint64_t* cand = beam + Lp;                                   // kBatch keys
     uint32_t* todo = reinterpret_cast<uint32_t*>(cand + kBatch);  // kBatch ids
-    uint32_t* table = todo + kBatch;                              // 2^table_log2 16-bit cells, or none (8-byte aligned)
+    uint32_t* todo2 = todo + kBatch;                              // kBatch ids: what the screening leaves to measure
+    uint32_t* table = todo2 + kBatch;                             // 2^table_log2 16-bit cells, or none (8-byte aligned)
     uint32_t* marks = table + (b.table_log2 ? (1 << b.table_log2) >> 1 : 0);  // Lp byte counters, zero between merges
     uint32_t* bloom = marks + (Lp >> 2);                          // 2^bloom_log2 bits, or none
     for (int i = lane; i < (Lp >> 2); i += 64) marks[i] = 0u;
@@ -202,12 +206,105 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
 
         // todo[0..T) -> distances -> the beam
         auto measure_and_merge = [&](int T) {
+            const uint32_t* list = todo;
+            // Screening (see beam_search.hip): each row is first measured in the half-precision copy of the vectors;
+            // a row whose exact distance is certainly beyond the beam's worst entry is dropped without reading its
+            // fp32 row -- most of what a search measures once its beam is full.
+            if (SCREEN && G == 64 && nb == L) {
+                constexpr int UH = U > kScreenRows ? kScreenRows : U;
+                constexpr int RPIH = 2 * UH;
+                const int glh = lane & 31, grph = lane >> 5;
+                const int chunksH = (dim + 7) >> 3;
+                const float s_live = key_s(live);
+                // the lane's share of the query: the eight dimensions of each 16-byte chunk of halves it reads
+                // (fetched with the rows rather than kept in registers for the whole query)
+                float4 qa[CPL][2];
+                {
+                    const float4* q4 = reinterpret_cast<const float4*>(a.queries + (size_t)qid * dim);
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        const int c = 2 * (glh + 32 * t);
+                        qa[t][0] = c < chunks ? q4[c] : make_float4(0, 0, 0, 0);
+                        qa[t][1] = c + 1 < chunks ? q4[c + 1] : make_float4(0, 0, 0, 0);
+                    }
+                }
+                int n2 = 0;
+                for (int base = 0; base < T; base += RPIH) {
+                    int vid[UH];
+                    const int r0 = base + grph * UH;
+#pragma unroll
+                    for (int u = 0; u < UH; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
+                    uint4 h[UH][CPL];
+#pragma unroll
+                    for (int u = 0; u < UH; ++u) {
+                        const uint4* row = reinterpret_cast<const uint4*>(
+                            b.vec16 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * b.stride16);
+#pragma unroll
+                        for (int t = 0; t < CPL; ++t) {
+                            const int c = glh + 32 * t;
+                            h[u][t] = (vid[u] >= 0 && c < chunksH) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
+                        }
+                    }
+                    int myid = vid[0];
+#pragma unroll
+                    for (int u = 1; u < UH; ++u)
+                        if ((lane & (UH - 1)) == u) myid = vid[u];
+                    const bool valid = glh < UH && myid >= 0;
+                    float nx = 0.0f;
+                    if (valid)
+                        nx = *reinterpret_cast<const float*>(b.vec16 + (uint64_t)(uint32_t)myid * b.stride16 +
+                                                             (size_t)chunksH * 16);
+                    float acc[UH];
+#pragma unroll
+                    for (int u = 0; u < UH; ++u) {
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < CPL; ++t) {
+                            const __half2* hp = reinterpret_cast<const __half2*>(&h[u][t]);
+                            const float2 x0 = __half22float2(hp[0]), x1 = __half22float2(hp[1]);
+                            const float2 x2 = __half22float2(hp[2]), x3 = __half22float2(hp[3]);
+                            float d;
+                            d = qa[t][0].x - x0.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][0].y - x0.y, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][0].z - x1.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][0].w - x1.y, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].x - x2.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].y - x2.y, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].z - x3.x, sum = __fmaf_rn(d, d, sum);
+                            d = qa[t][1].w - x3.y, sum = __fmaf_rn(d, d, sum);
+                        }
+                        acc[u] = sum;
+                    }
+#pragma unroll
+                    for (int u = 0; u < UH; ++u) {
+                        acc[u] = acc[u] + dpp_mov<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
+                        acc[u] = acc[u] + dpp_mov<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
+                        acc[u] = acc[u] + dpp_mov<0x141>(acc[u]);  // row_half_mirror
+                        acc[u] = acc[u] + dpp_mov<0x140>(acc[u]);  // row_mirror
+                    }
+                    float mine = acc[0];
+#pragma unroll
+                    for (int u = 1; u < UH; ++u)
+                        if ((lane & (UH - 1)) == u) mine = acc[u];
+                    mine = mine + __shfl_xor(mine, 16, 64);
+                    const float root = sqrtf(mine), r = 5.0e-4f * nx + 1.0e-6f;
+                    const float lo_root = fmaxf(root - r, 0.0f);
+                    const float lo = lo_root * lo_root * (1.0f - 1.0e-4f);
+                    const bool exact = valid && !(lo > s_live);
+                    const uint64_t m = __ballot(exact);
+                    if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;
+                    n2 += __popcll(m);
+                }
+                wave_sync();
+                list = todo2;
+                T = n2;
+            }
             int nc = 0;
             for (int base = 0; base < T; base += RPI) {
                 int vid[U];
                 const int r0 = base + grp * U;
 #pragma unroll
-                for (int u = 0; u < U; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
+                for (int u = 0; u < U; ++u) vid[u] = r0 + u < T ? (int)list[r0 + u] : -1;
                 float4 v[U][CPL];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -457,30 +554,36 @@ using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 // RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
 // dependent memory waits of a step against 8 and needs 128 registers; 32 (a whole step at once, 212 registers) is
 // for launches whose LDS holds a CU to eight wavefronts anyway (+2..3 %)
-template <int RIF, bool PACKED>
+template <int RIF, bool PACKED, bool SCREEN>
 bf_kernel_fn pick_bf_kernel_rif(int chunks) {
-    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED>;
-    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED>;
-    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED>;
-    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED>;
-    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED>;
-    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED>;
+    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED, false>;
+    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, false>;
+    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED, SCREEN>;
+    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED, SCREEN>;
+    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED, SCREEN>;
+    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED, SCREEN>;
     return nullptr;
 }
 
-bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed) {
+template <bool SCREEN>
+bf_kernel_fn pick_bf_kernel_screen(int dim, int rif, bool packed) {
     // 32: for launches that hold eight wavefronts per CU or fewer (256 registers per lane); rows of 17..64 chunks
     if (rif >= 32 && dim / 4 > 16 && dim / 4 <= 64)
-        return packed ? pick_bf_kernel_rif<32, true>(dim / 4) : pick_bf_kernel_rif<32, false>(dim / 4);
-    if (packed) return rif >= 16 ? pick_bf_kernel_rif<16, true>(dim / 4) : pick_bf_kernel_rif<8, true>(dim / 4);
-    return rif >= 16 ? pick_bf_kernel_rif<16, false>(dim / 4) : pick_bf_kernel_rif<8, false>(dim / 4);
+        return packed ? pick_bf_kernel_rif<32, true, SCREEN>(dim / 4) : pick_bf_kernel_rif<32, false, SCREEN>(dim / 4);
+    if (packed)
+        return rif >= 16 ? pick_bf_kernel_rif<16, true, SCREEN>(dim / 4) : pick_bf_kernel_rif<8, true, SCREEN>(dim / 4);
+    return rif >= 16 ? pick_bf_kernel_rif<16, false, SCREEN>(dim / 4) : pick_bf_kernel_rif<8, false, SCREEN>(dim / 4);
+}
+
+bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed, bool screen) {
+    return screen ? pick_bf_kernel_screen<true>(dim, rif, packed) : pick_bf_kernel_screen<false>(dim, rif, packed);
 }
 
 }  // namespace
 
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int bloom_log2, int table_log2,
-                              int* max_wg_per_cu) {
-    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed);
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, bool screen, int bloom_log2,
+                              int table_log2, int* max_wg_per_cu) {
+    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed, screen);
     if (!fn) return hipErrorInvalidValue;
     const size_t lds = best_first_wave_lds_bytes(L, bloom_log2, table_log2) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -494,7 +597,7 @@ hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, i
 }
 
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream) {
-    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0);
+    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0, b.vec16 != nullptr);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64),

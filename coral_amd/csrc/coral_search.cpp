@@ -275,10 +275,11 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
     const size_t lds_max = (size_t)kMaxLdsBytes;
     // ---- screening in half precision (rounds policy, L2, rows of 132 .. 2048 floats): see beam_search.hip
+    // (best-first: the wavefront-per-query kernel with the beam in LDS screens too, see coral_search_prepare)
     const bool screen_possible = !best_first && idx->metric == CORAL_L2 && idx->dim / 4 > 32;
-    if (t.screening > 0 && !screen_possible)
-        return fail(CORAL_ERR_ARG, "screening needs the rounds policy, the L2 metric and more than 128 dimensions");
-    const bool screen = t.screening > 0 || (t.screening == 0 && screen_possible && !no_screen);
+    if (t.screening > 0 && !(idx->metric == CORAL_L2 && idx->dim / 4 > 32))
+        return fail(CORAL_ERR_ARG, "screening needs the L2 metric and more than 128 dimensions");
+    const bool screen = screen_possible && (t.screening > 0 || (t.screening == 0 && !no_screen));
     p.screen = screen;
     // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
     // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
@@ -467,7 +468,22 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // Best-first, one wavefront per query: the visited state lives in HBM, n bytes per wavefront (n / 6 in the packed
     // form), up to a third of what is free and 64 GiB.  wg_per_cu: what the chosen kernel's occupancy allows;
     // reprepare(packed): sets that kernel up in the packed form and returns its occupancy.
-    idx->bf_ready = false, idx->bf_long = false;
+    idx->bf_ready = false, idx->bf_long = false, idx->bf_screen = false;
+    // Best-first with the beam in LDS screens rows in half precision too, where a CU holds sixteen wavefronts (beams
+    // without the LDS table: L > 409): +12 % at L = 512 and 1024.  With the table (eight wavefronts per CU) the extra
+    // wait per step costs more than the bytes it spares (L = 256 / 320: -27 %), so those launches go without unless
+    // the caller asks for it by name.
+    if (wave_form && idx->metric == CORAL_L2 && idx->dim / 4 > 32 &&
+        (t.screening > 0 || (t.screening == 0 && table_log2 == 0))) {
+        const hipError_t e = ensure_vec16();
+        if (e == hipSuccess) {
+            idx->bf_screen = true;
+        } else if (e == hipErrorOutOfMemory && t.screening == 0) {
+            (void)hipGetLastError();
+        } else {
+            HIP_TRY(e);
+        }
+    }
     auto visited_slots = [&](int bf_wg_per_cu, auto reprepare, int64_t other_bytes_per_slot) -> int {
         size_t free_b = 0, total_b = 0;
         HIP_TRY(hipMemGetInfo(&free_b, &total_b));
@@ -524,9 +540,9 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         // with a table the filter would only cover what outgrew it, and its LDS is worth more as cells
         const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L);
         idx->bf_bloom_log2 = bloom_log2;
-        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, bloom_log2, table_log2, &bf_wg_per_cu));
+        HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, idx->bf_screen, bloom_log2, table_log2, &bf_wg_per_cu));
         auto reprepare = [&](int* occ) {
-            return coral::best_first_prepare(idx->dim, L, rif, true, bloom_log2, table_log2, occ);
+            return coral::best_first_prepare(idx->dim, L, rif, true, idx->bf_screen, bloom_log2, table_log2, occ);
         };
         if (int rc = visited_slots(bf_wg_per_cu, reprepare, 0)) return rc;
     } else if (long_form) {
@@ -652,6 +668,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;
+        b.vec16 = idx->bf_screen ? idx->d_vec16 : nullptr, b.stride16 = coral::half_row_stride(idx->dim);
         HIP_TRY(coral::launch_best_first(a, b, stream));
     } else {
         const int wgs = std::min(plan.workgroups, (int)Q);

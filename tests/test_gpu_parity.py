@@ -207,10 +207,22 @@ def test_screening_in_half_precision_changes_nothing(orc, kind):
         assert np.array_equal(ids, oi), form
         assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), form
         assert np.array_equal(idx.query_counters(Q), os_), form
-    # where it does not apply it is refused when asked for by name, and left out otherwise
-    with pytest.raises(capi.CoralError):
-        idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, screening=1)
+    # best-first on the wavefront-per-query kernel screens against the beam's worst entry
+    oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
+    for form in (dict(screening=-1), dict(screening=1), dict(screening=1, best_first_table_log2=-1),
+                 dict(screening=1, best_first_packed=True)):
+        idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, **form)
+        ids, dists, _ = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)
+        assert np.array_equal(ids, oi), form
+        assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), form
+        assert np.array_equal(idx.query_counters(Q), os_), form
     idx.close()
+    # where it does not apply it is refused when asked for by name, and left out otherwise
+    small = capi.Index(base[:, :64].copy(), nbrs, starts)
+    with pytest.raises(capi.CoralError):
+        small.prepare(Q, L, screening=1)
+    small.prepare(Q, L)
+    small.close()
 
 
 def test_beam_capacity_limits():
