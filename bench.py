@@ -458,7 +458,8 @@ def main():
 
     # the library's exhaustive search on the same queries (host buffers in and out): what recall 1.0 costs here
     out["exact_knn"] = {"qps": Q / b.gt_s, "recall": 1.0, "time_s": b.gt_s,
-                        "kernels": "approx_tile_mfma_kernel (fp32 MFMA screening) + row_select_kernel + rerank_kernel"}
+                        "kernels": "approx_tile_mfma_kernel (fp32 MFMA screening, candidates selected in its epilogue) + "
+                                   "list_select_kernel + rerank_kernel"}
 
     # the IndexGPU::Search shape: host buffers in and out (query upload to the index's staging buffers,
     # search, id download); reported beside the headline, never as the headline

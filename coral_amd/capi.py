@@ -117,6 +117,7 @@ SIGNATURES = {
     "coral_start_ids_fps": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_bruteforce_set_exact_only": (C.c_int, [C.c_void_p, C.c_int32]),
     "coral_bruteforce_last_redone": (C.c_int64, [C.c_void_p]),
+    "coral_bruteforce_last_fused": (C.c_int32, [C.c_void_p]),
     "coral_membench": (C.c_int, [C.c_int32, C.c_size_t, C.c_int32, C.c_int32, C.POINTER(C.c_double),
                                  C.POINTER(C.c_double)]),
     "coral_bruteforce_knn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
@@ -261,8 +262,12 @@ class Index:
         return ids, dists, t.value
 
     def bruteforce_exact_only(self, on=True):
-        """Skip (or restore) the matrix-core screening pass of the exact kNN."""
-        _check(lib().coral_bruteforce_set_exact_only(self._h, int(bool(on))))
+        """Skip (True / 1) or restore (False / 0) the matrix-core screening pass of the exact kNN; 2 keeps the
+        screening and selects the candidates from the full distance matrix instead of inside the kernel."""
+        _check(lib().coral_bruteforce_set_exact_only(self._h, int(on)))
+
+    def bruteforce_last_fused(self):
+        return int(lib().coral_bruteforce_last_fused(self._h))
 
     def bruteforce_last_redone(self):
         return int(lib().coral_bruteforce_last_redone(self._h))

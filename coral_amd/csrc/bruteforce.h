@@ -16,9 +16,21 @@ hipError_t launch_merge_segments(const unsigned long long* part, int nq, int nse
 // out[r] = |x_r|^2; *max_bits (optional, zero before) = bit pattern of the largest of them
 hipError_t launch_row_norms(const float* x, int64_t n, int dim, float* out, uint32_t* max_bits, hipStream_t stream);
 // as launch_distance_tile, with D[q][b] = |q|^2 + |b|^2 - 2 q.b (L2) or -q.b (IP) from fp32 MFMA inner products
+// sample_tiles > 0: only that many tiles of 128 base points, every tile_stride-th of the base, side by side in D
 hipError_t launch_approx_tile(const float* queries, const float* base, int nq, int64_t nb, int dim, int metric,
                               const float* qn, const float* bn, const uint32_t* deleted, int64_t base_id0, float* D,
-                              int64_t ldD, hipStream_t stream);
+                              int64_t ldD, hipStream_t stream, int64_t sample_tiles = 0, int64_t tile_stride = 1);
+// the same distances, no matrix: every entry <= tau[q] is appended to lists[q * cap ...] as ord(value) << 32 | id
+// (cnt[q] counts them, also those beyond cap that were dropped; zero before)
+hipError_t launch_approx_filter(const float* queries, const float* base, int nq, int64_t nb, int dim, int metric,
+                                const float* qn, const float* bn, const uint32_t* deleted, const float* tau,
+                                unsigned long long* lists, int64_t cap, unsigned int* cnt, hipStream_t stream);
+// tau[q] = value of keys[q * stride + j], +inf where that key is the "none" key
+hipError_t launch_bound_from_keys(const unsigned long long* keys, int64_t stride, int j, int nq, float* tau,
+                                  hipStream_t stream);
+// the k (<= 1024) smallest keys of every list, sorted; *overflow (zero before) counts the lists that could not be done
+hipError_t launch_list_select(const unsigned long long* lists, int64_t cap, const unsigned int* cnt, int nq, int k,
+                              unsigned long long* out, int64_t out_stride, int* overflow, hipStream_t stream);
 // cand_ids / cand_d [nq][kc] (ascending approximate signed distance, -1 = none) -> the exact k best per query in the
 // reference's summation order; redo[q] = 1 where the candidates cannot vouch for the result
 hipError_t launch_rerank(const float* queries, const float* base, int nq, int dim, int metric, const int32_t* cand_ids,

@@ -262,6 +262,77 @@ __global__ __launch_bounds__(kSelThreads) void row_select_kernel(const float* __
     }
 }
 
+// One workgroup per query: the k smallest of the cnt[q] keys in lists[q * cap ...] (distinct: every key carries its
+// id), sorted, into out.  The scheme of row_select_kernel on keys: the k-th smallest of the per-thread minima bounds
+// the k-th smallest key from above, a second pass collects what lies up to it, a sort finishes.  *overflow is raised
+// when a list lost entries (cnt[q] > cap) or the collection outgrows LDS; the caller then takes another path.
+__global__ __launch_bounds__(kSelThreads) void list_select_kernel(const unsigned long long* __restrict__ lists,
+                                                                  int64_t cap, const unsigned int* __restrict__ cnt,
+                                                                  int k, unsigned long long* __restrict__ out,
+                                                                  int64_t out_stride, int* __restrict__ overflow) {
+    __shared__ unsigned long long skeys[kSelCap];
+    __shared__ unsigned long long smin[kSelThreads];
+    __shared__ unsigned int s_count;
+    const int tid = threadIdx.x;
+    const unsigned int have = cnt[blockIdx.x];
+    if (have > (unsigned)cap) {
+        if (tid == 0) atomicAdd(overflow, 1);
+        return;
+    }
+    const int n = (int)have;
+    const unsigned long long* list = lists + (size_t)blockIdx.x * cap;
+    const int kk = min(k, n);
+    unsigned long long m = ~0ull;
+    for (int i = tid; i < n; i += kSelThreads) m = min(m, list[i]);
+    smin[tid] = m;
+    if (tid == 0) s_count = 0u;
+    __syncthreads();
+    for (int k2 = 2; k2 <= kSelThreads; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1) {
+            if (tid < kSelThreads / 2) {
+                const int i = 2 * tid - (tid & (j - 1)), x = i + j;
+                const bool asc = (i & k2) == 0;
+                const unsigned long long a = smin[i], b = smin[x];
+                if ((a > b) == asc) smin[i] = b, smin[x] = a;
+            }
+            __syncthreads();
+        }
+    const unsigned long long thr = kk > 0 ? smin[kk - 1] : 0ull;  // k <= kSelThreads (launcher)
+    for (int i = tid; i < n; i += kSelThreads) {
+        const unsigned long long key = list[i];
+        if (kk > 0 && key <= thr) {
+            const unsigned pos = atomicAdd(&s_count, 1u);
+            if (pos < (unsigned)kSelCap) skeys[pos] = key;
+        }
+    }
+    __syncthreads();
+    const unsigned count = s_count;
+    if (count > (unsigned)kSelCap) {
+        if (tid == 0) atomicAdd(overflow, 1);
+        return;
+    }
+    int P = 2;
+    while (P < (int)count) P <<= 1;
+    for (int i = (int)count + tid; i < P; i += kSelThreads) skeys[i] = ~0ull;
+    __syncthreads();
+    for (int k2 = 2; k2 <= P; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1) {
+            for (int t = tid; t < (P >> 1); t += kSelThreads) {
+                const int i = 2 * t - (t & (j - 1)), x = i + j;
+                const bool asc = (i & k2) == 0;
+                const unsigned long long ka = skeys[i], kb = skeys[x];
+                if ((ka > kb) == asc) skeys[i] = kb, skeys[x] = ka;
+            }
+            __syncthreads();
+        }
+    unsigned long long* dst = out + (size_t)blockIdx.x * out_stride;
+    for (int i = tid; i < k; i += kSelThreads) {
+        unsigned long long key = i < kk ? skeys[i] : ~0ull;
+        if ((uint32_t)(key >> 32) == bf_ord32(__int_as_float(0x7f800000))) key = ~0ull;  // tombstoned
+        dst[i] = key;
+    }
+}
+
 // The general path: exact k-th smallest by an 8-bit radix select, then ordered compaction.  Only rows flagged in
 // redo (or all rows when redo is null) are processed.
 __global__ __launch_bounds__(256) void row_select_radix_kernel(const float* __restrict__ D, int64_t ldD,
@@ -447,6 +518,14 @@ hipError_t launch_row_select(const float* D, int64_t ldD, int nq, int64_t n, int
                            redo);
     hipLaunchKernelGGL(row_select_radix_kernel, dim3(nq), dim3(256), (size_t)P * 8, stream, D, ldD, n, k, id0, out,
                        out_stride, fast ? redo : nullptr);
+    return hipGetLastError();
+}
+
+hipError_t launch_list_select(const unsigned long long* lists, int64_t cap, const unsigned int* cnt, int nq, int k,
+                              unsigned long long* out, int64_t out_stride, int* overflow, hipStream_t stream) {
+    if (k > kSelThreads) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(list_select_kernel, dim3(nq), dim3(kSelThreads), 0, stream, lists, cap, cnt, k, out, out_stride,
+                       overflow);
     return hipGetLastError();
 }
 

@@ -90,6 +90,74 @@ int ensure_base_norms(coral_index* idx, hipStream_t stream) {
 }
 
 constexpr int kScreenSlack = 32;  // candidates kept beyond k
+constexpr int64_t kListCap = 16384;  // keys a query's candidate list holds in the fused screening
+
+// The screening with the selection inside the matrix-core kernel: no distance matrix goes to memory.  Per block of
+// queries: (1) the distances to a sample of the base (every stride-th tile of 128 points) as a small matrix, whose
+// kc-th smallest entry per row is a bound tau[q] that at least kc entries of the whole row do not exceed; (2) one
+// pass over the whole base that appends the entries up to tau[q] to the query's list (about kc * n / sample of
+// them); (3) the kc smallest keys of every list.  The kept candidates are those of knn_passes(screen = true): the
+// same approximate values, the kc smallest under (value, id).  *used = false when the shape does not suit (kc beyond
+// what list_select_kernel takes, a base too small to sample) or a list overflowed (sample unlike the base, rows of
+// equal values, too few live points in the sample): the caller then goes through the matrix.
+int knn_screen_fused(coral_index* idx, const float* d_queries, int32_t Q, int32_t kc, int32_t have_delete,
+                     const float* d_qn, int32_t* d_cid, float* d_cd, hipStream_t stream, bool* used) {
+    *used = false;
+    const int64_t n = idx->n, full_tiles = n / 128;
+    int64_t tiles = (2 * (int64_t)kc * full_tiles + kListCap - 1) / kListCap;
+    tiles = std::max<int64_t>(8, (tiles + 7) & ~(int64_t)7);
+    if (kc > 1024 || tiles * 8 > full_tiles || n > 0x7fffffff) return CORAL_OK;
+    const int64_t stride = full_tiles / tiles, ns = tiles * 128;
+    int64_t qc = std::min<int64_t>(kListCap, (kBufferFloats / ns) & ~(int64_t)127);
+    qc = std::min<int64_t>(qc, ((int64_t)Q + 127) & ~(int64_t)127);
+    float *D = nullptr, *tau = nullptr;
+    unsigned long long *keys = nullptr, *lists = nullptr;
+    unsigned int* cnt = nullptr;
+    int *redo = nullptr, *overflow = nullptr;
+    auto release = [&]() {
+        (void)hipFree(D), (void)hipFree(tau), (void)hipFree(keys), (void)hipFree(lists);
+        (void)hipFree(cnt), (void)hipFree(redo), (void)hipFree(overflow);
+    };
+#define HIP_TRY_R(expr)                                                                  \
+    do {                                                                                 \
+        hipError_t e_ = (expr);                                                          \
+        if (e_ != hipSuccess) {                                                          \
+            release();                                                                   \
+            return fail(e_ == hipErrorOutOfMemory ? CORAL_ERR_MEMORY : CORAL_ERR_DEVICE, \
+                        "%s failed: %s", #expr, hipGetErrorString(e_));                  \
+        }                                                                                \
+    } while (0)
+    HIP_TRY_R(hipMalloc(&D, (size_t)qc * ns * sizeof(float)));
+    HIP_TRY_R(hipMalloc(&tau, (size_t)qc * sizeof(float)));
+    HIP_TRY_R(hipMalloc(&keys, (size_t)qc * kc * sizeof(unsigned long long)));
+    HIP_TRY_R(hipMalloc(&lists, (size_t)qc * kListCap * sizeof(unsigned long long)));
+    HIP_TRY_R(hipMalloc(&cnt, (size_t)qc * sizeof(unsigned int)));
+    HIP_TRY_R(hipMalloc(&redo, (size_t)qc * sizeof(int)));
+    HIP_TRY_R(hipMalloc(&overflow, sizeof(int)));
+    HIP_TRY_R(coral::launch_fill_u32(reinterpret_cast<uint32_t*>(overflow), 1, 0u, stream));
+    const uint32_t* del = have_delete ? idx->d_deleted : nullptr;
+    for (int64_t q0 = 0; q0 < Q; q0 += qc) {
+        const int nq = (int)std::min<int64_t>(qc, Q - q0);
+        const float* qp = d_queries + (size_t)q0 * idx->dim;
+        HIP_TRY_R(coral::launch_approx_tile(qp, idx->d_vec, nq, n, idx->dim, idx->metric, d_qn + q0, idx->d_bnorm, del, 0, D,
+                                            ns, stream, tiles, stride));
+        HIP_TRY_R(coral::launch_row_select(D, ns, nq, ns, kc, 0, keys, kc, redo, stream));
+        HIP_TRY_R(coral::launch_bound_from_keys(keys, kc, kc - 1, nq, tau, stream));
+        HIP_TRY_R(coral::launch_fill_u32(cnt, (size_t)nq, 0u, stream));
+        HIP_TRY_R(coral::launch_approx_filter(qp, idx->d_vec, nq, n, idx->dim, idx->metric, d_qn + q0, idx->d_bnorm, del, tau,
+                                              lists, kListCap, cnt, stream));
+        HIP_TRY_R(coral::launch_list_select(lists, kListCap, cnt, nq, kc, keys, kc, overflow, stream));
+        HIP_TRY_R(coral::launch_merge_segments(keys, nq, 1, kc, /*signed distances*/ 0, d_cid + (size_t)q0 * kc,
+                                               d_cd + (size_t)q0 * kc, stream));
+    }
+    int lost = 0;
+    HIP_TRY_R(hipMemcpyAsync(&lost, overflow, sizeof(int), hipMemcpyDeviceToHost, stream));
+    HIP_TRY_R(hipStreamSynchronize(stream));
+#undef HIP_TRY_R
+    release();
+    *used = lost == 0;
+    return CORAL_OK;
+}
 
 }  // namespace
 
@@ -97,11 +165,14 @@ extern "C" {
 
 int coral_bruteforce_set_exact_only(coral_index* idx, int32_t on) {
     if (!idx) return fail(CORAL_ERR_ARG, "null index");
-    idx->knn_exact_only = on != 0;
+    if (on < 0 || on > 2) return fail(CORAL_ERR_ARG, "on must be 0, 1 or 2 (got %d)", on);
+    idx->knn_mode = on;
     return CORAL_OK;
 }
 
 int64_t coral_bruteforce_last_redone(coral_index* idx) { return idx ? idx->knn_last_redone : -1; }
+
+int32_t coral_bruteforce_last_fused(coral_index* idx) { return idx ? (int32_t)idx->knn_last_fused : -1; }
 
 int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q, int32_t k,
                              int32_t have_delete, int32_t* d_ids, float* d_dists, void* stream_,
@@ -120,7 +191,8 @@ int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q
     int rc = CORAL_OK;
     const int kc = k + kScreenSlack;
     idx->knn_last_redone = 0;
-    if (idx->knn_exact_only || kc > 2048 || idx->n <= kc) {
+    idx->knn_last_fused = false;
+    if (idx->knn_mode == 1 || kc > 2048 || idx->n <= kc) {
         rc = knn_passes(idx, d_queries, Q, k, have_delete, false, nullptr, idx->metric, d_ids, d_dists, stream);
     } else {
         // screening on the matrix cores, exact distances for the kc candidates of each query, the exact passes for
@@ -145,8 +217,14 @@ int coral_bruteforce_knn_gpu(coral_index* idx, const float* d_queries, int32_t Q
             ok(hipMalloc(&d_cid, (size_t)Q * kc * sizeof(int32_t)), "hipMalloc") &&
             ok(hipMalloc(&d_cd, (size_t)Q * kc * sizeof(float)), "hipMalloc") &&
             ok(hipMalloc(&d_redo, (size_t)Q * sizeof(int)), "hipMalloc") &&
-            ok(coral::launch_row_norms(d_queries, Q, idx->dim, d_qn, nullptr, stream), "query norms"))
-            rc = knn_passes(idx, d_queries, Q, kc, have_delete, true, d_qn, /*signed distances*/ 0, d_cid, d_cd, stream);
+            ok(coral::launch_row_norms(d_queries, Q, idx->dim, d_qn, nullptr, stream), "query norms")) {
+            bool fused = false;
+            if (idx->knn_mode == 0)
+                rc = knn_screen_fused(idx, d_queries, Q, kc, have_delete, d_qn, d_cid, d_cd, stream, &fused);
+            idx->knn_last_fused = fused;
+            if (rc == CORAL_OK && !fused)
+                rc = knn_passes(idx, d_queries, Q, kc, have_delete, true, d_qn, /*signed distances*/ 0, d_cid, d_cd, stream);
+        }
         if (rc == CORAL_OK &&
             ok(coral::launch_rerank(d_queries, idx->d_vec, Q, idx->dim, idx->metric, d_cid, d_cd, kc, k, d_qn,
                                     idx->d_bnorm_max, d_ids, d_dists, d_redo, stream), "rerank") &&

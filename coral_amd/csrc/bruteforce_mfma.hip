@@ -29,7 +29,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 #define CORAL_MFMA_BK 8
 #endif
 constexpr int MT = 128, NT = 128, BK = CORAL_MFMA_BK;  // tile of queries x base points per workgroup, dimensions per LDS stage
-constexpr int NLD = BK / 8;                             // float4 loads per thread, operand and stage
+constexpr int NS = BK / 8;                              // 16-byte pieces per thread, operand and stage
+constexpr int RS = BK == 8 ? 8 : BK + 4;                // floats from one row to the next in LDS
+
 
 __device__ __forceinline__ uint32_t mf_ord32(float s) {
     const uint32_t u = __float_as_uint(s);
@@ -67,44 +69,56 @@ __global__ __launch_bounds__(256) void row_norms_kernel(const float* __restrict_
 #ifndef CORAL_MFMA_WAVES
 #define CORAL_MFMA_WAVES 4
 #endif
+// FUSED = false writes the tile into D (column bt * 128 + ..., where bt counts the tiles this launch computes:
+// tile_stride > 1 takes every tile_stride-th tile of the base, a sample whose columns lie side by side in D).
+// FUSED = true writes no matrix: an entry goes, as the key ord(value) << 32 | id, to the list of its query if it does
+// not exceed the query's bound tau[q] -- cnt[q] entries so far, at most cap kept (a count beyond cap tells the
+// caller that the list is incomplete).  A tile's entries are first gathered in LDS, so that the global counters see
+// one round of atomics per tile instead of one per accumulator register.
+template <bool FUSED, bool L2>
 __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel(const float* __restrict__ queries,
                                                               const float* __restrict__ base, int nq, int64_t nb,
-                                                              int dim, int metric, const float* __restrict__ qn,
+                                                              int dim, const float* __restrict__ qn,
                                                               const float* __restrict__ bn,
                                                               const uint32_t* __restrict__ deleted, int64_t base_id0,
-                                                              float* __restrict__ D, int64_t ldD) {
-    __shared__ float sa[2][BK][MT + 4];
-    __shared__ float sb[2][BK][NT + 4];
+                                                              int64_t ntiles, int64_t tile_stride, int hq,
+                                                              float* __restrict__ D, int64_t ldD,
+                                                              const float* __restrict__ tau,
+                                                              unsigned long long* __restrict__ lists, int64_t cap,
+                                                              unsigned int* __restrict__ cnt) {
+    // Operands in LDS row-major, the BK = 8 dimensions of a row side by side (32 bytes): a thread parks the 16 bytes
+    // it fetched with one write, and the 16 bytes a lane reads hold its operands of four multiplications -- lane
+    // (kh, m) supplies row m's dimension kh * 4 + j to step j, so a step multiplies the dimension pair (j, 4 + j) of
+    // the stage.  The 64 lanes of either access cover consecutive addresses: no bank conflicts, no padding.
+    __shared__ __align__(16) float sa[2][MT][RS];
+    __shared__ __align__(16) float sb[2][NT][RS];
+    static_assert(BK % 8 == 0, "a stage is made of 16-byte pieces, one per thread, operand and eight dimensions");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1;
-    // Workgroups go to the eight XCDs in turn, each with an L2 of its own: the workgroups that share a tile of
-    // base points (one per tile of queries) are given consecutive places on one XCD, so that the base tile comes
-    // from memory once and from that L2 afterwards.  grid.x = 8 x ceil(base tiles / 8) x query tiles.
+    // Workgroups go to the eight XCDs in turn, each with an L2 of its own (4 MB).  An XCD takes every eighth tile of
+    // base points and walks, for one block of hq query tiles after the other, through all its base tiles: the
+    // workgroups in flight on it share those hq query tiles (hq x 100 KB at dim 200) and a handful of base tiles,
+    // so both operands come from that L2 and each base tile from memory once per block of queries.
+    // grid.x = 8 x ceil(base tiles / 8) x query blocks x hq.
     const int nqt = (nq + MT - 1) / MT;
     const unsigned xcd = blockIdx.x & 7u, place = blockIdx.x >> 3;
-    const int64_t bt = (int64_t)(place / (unsigned)nqt) * 8 + xcd;
-    const int64_t b0 = bt * NT;
-    const int q0 = (int)(place % (unsigned)nqt) * MT;
-    if (b0 >= nb) return;  // the padding of the last group of eight base tiles
+    const unsigned nbt8 = (unsigned)((ntiles + 7) >> 3);
+    const unsigned qb = place / (nbt8 * (unsigned)hq), rem = place - qb * nbt8 * (unsigned)hq;
+    const int64_t bt = (int64_t)(rem / (unsigned)hq) * 8 + xcd;
+    const int qt = (int)(qb * (unsigned)hq + rem % (unsigned)hq);
+    const int64_t b0 = bt * tile_stride * NT;
+    const int q0 = qt * MT;
+    if (bt >= ntiles || b0 >= nb || qt >= nqt) return;  // padding: the last group of eight base tiles, the last query block
     const int lrow = tid >> 1, lk = (tid & 1) * 4;  // staging: thread t loads row t/2, dimensions (t&1)*4 .. +4
-    float4 va[NLD], vb[NLD];
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            va[u] = make_float4(0, 0, 0, 0), vb[u] = make_float4(0, 0, 0, 0);
-            const int kd = k0 + lk + 8 * u;
-            if (kd < dim) {
-                if (q0 + lrow < nq) va[u] = *reinterpret_cast<const float4*>(queries + (size_t)(q0 + lrow) * dim + kd);
-                if (b0 + lrow < nb) vb[u] = *reinterpret_cast<const float4*>(base + (size_t)(b0 + lrow) * dim + kd);
-            }
-        }
-    };
+    // rows beyond the end read the last row instead: their results are never written
+    const float* pa = queries + (size_t)min(q0 + lrow, nq - 1) * dim + lk;
+    const float* pb = base + (size_t)min(b0 + lrow, nb - 1) * dim + lk;
+    float4 va[NS], vb[NS];
     auto park = [&](int buf) {
 #pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            const int r = lk + 8 * u;
-            sa[buf][r + 0][lrow] = va[u].x, sa[buf][r + 1][lrow] = va[u].y, sa[buf][r + 2][lrow] = va[u].z, sa[buf][r + 3][lrow] = va[u].w;
-            sb[buf][r + 0][lrow] = vb[u].x, sb[buf][r + 1][lrow] = vb[u].y, sb[buf][r + 2][lrow] = vb[u].z, sb[buf][r + 3][lrow] = vb[u].w;
+        for (int u = 0; u < NS; ++u) {
+            *reinterpret_cast<float4*>(&sa[buf][lrow][8 * u + lk]) = va[u];
+            *reinterpret_cast<float4*>(&sb[buf][lrow][8 * u + lk]) = vb[u];
         }
     };
     v16f acc[2][2];
@@ -115,30 +129,59 @@ __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
     const int kh = lane >> 5, m = lane & 31;  // an MFMA operand: lane = row (or column) m of dimension kh
-    fetch(0);
+    // the last stage may hold half a row (dim is a multiple of 4): its missing half is zero
+    const int full = dim / BK, tail = dim % BK;
+    auto fetch = [&](int st) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            va[u] = *reinterpret_cast<const float4*>(pa + st * BK + 8 * u);
+            vb[u] = *reinterpret_cast<const float4*>(pb + st * BK + 8 * u);
+        }
+    };
+    auto fetch_tail = [&]() {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            va[u] = make_float4(0, 0, 0, 0), vb[u] = make_float4(0, 0, 0, 0);
+            if (8 * u + lk < tail) {
+                va[u] = *reinterpret_cast<const float4*>(pa + full * BK + 8 * u);
+                vb[u] = *reinterpret_cast<const float4*>(pb + full * BK + 8 * u);
+            }
+        }
+    };
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            const float4 a0 = *reinterpret_cast<const float4*>(&sa[buf][wr * 64 + m][8 * u + kh * 4]);
+            const float4 a1 = *reinterpret_cast<const float4*>(&sa[buf][wr * 64 + 32 + m][8 * u + kh * 4]);
+            const float4 c0 = *reinterpret_cast<const float4*>(&sb[buf][wc * 64 + m][8 * u + kh * 4]);
+            const float4 c1 = *reinterpret_cast<const float4*>(&sb[buf][wc * 64 + 32 + m][8 * u + kh * 4]);
+#define CORAL_MFMA_STEP(X)                                                                  \
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.X, c0.X, acc[0][0], 0, 0, 0); \
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.X, c1.X, acc[0][1], 0, 0, 0); \
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.X, c0.X, acc[1][0], 0, 0, 0); \
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.X, c1.X, acc[1][1], 0, 0, 0);
+            CORAL_MFMA_STEP(x)
+            CORAL_MFMA_STEP(y)
+            CORAL_MFMA_STEP(z)
+            CORAL_MFMA_STEP(w)
+#undef CORAL_MFMA_STEP
+        }
+    };
+    const int stages = full + (tail ? 1 : 0);
+    if (full > 0)
+        fetch(0);
+    else
+        fetch_tail();
     park(0);
     __syncthreads();
     int cur = 0;
-    for (int k0 = 0; k0 < dim; k0 += BK) {
-        const bool more = k0 + BK < dim;
-        if (more) fetch(k0 + BK);
-        // the operands of a pair of dimensions are read while the pair before is multiplied
-        float a0 = sa[cur][kh][wr * 64 + m], a1 = sa[cur][kh][wr * 64 + 32 + m];
-        float c0 = sb[cur][kh][wc * 64 + m], c1 = sb[cur][kh][wc * 64 + 32 + m];
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float a0n = 0.0f, a1n = 0.0f, c0n = 0.0f, c1n = 0.0f;
-            if (kk + 2 < BK) {
-                a0n = sa[cur][kk + 2 + kh][wr * 64 + m], a1n = sa[cur][kk + 2 + kh][wr * 64 + 32 + m];
-                c0n = sb[cur][kk + 2 + kh][wc * 64 + m], c1n = sb[cur][kk + 2 + kh][wc * 64 + 32 + m];
-            }
-            __builtin_amdgcn_sched_barrier(0);  // keeps the reads above ahead of the multiplications below
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, c0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, c1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, c0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, c1, acc[1][1], 0, 0, 0);
-            a0 = a0n, a1 = a1n, c0 = c0n, c1 = c1n;
-        }
+    for (int st = 0; st < stages; ++st) {
+        const bool more = st + 1 < stages;
+        if (st + 1 < full)
+            fetch(st + 1);
+        else if (more)
+            fetch_tail();
+        multiply(cur);
         if (more) park(cur ^ 1);
         __syncthreads();
         cur ^= 1;
@@ -148,15 +191,24 @@ __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel
     // workgroup instead of by 64 dependent global loads per lane.
     float* srow = &sa[0][0][0];  // the operand buffers are free after the last barrier of the loop
     float* scol = &sb[0][0][0];
-    const float inf = __int_as_float(0x7f800000);
+    float* stau = srow + MT;
+    // (FUSED) the tile's entries that pass: ord(value) << 32 | place, where place = accumulator register << 8 |
+    // thread names the entry's row and column; they lie behind the norms
+    unsigned long long* shit = reinterpret_cast<unsigned long long*>(scol + NT);
+    constexpr int kHitCap = (2 * NT * RS - NT) / 2;
+    unsigned int& s_nhit = *reinterpret_cast<unsigned int*>(stau + MT);
+    const float inf = __int_as_float(0x7f800000), nan = __int_as_float(0x7fc00000);
     if (tid < MT) {
         const int r = q0 + tid;
-        srow[tid] = (metric == 0 && r < nq) ? qn[r] : 0.0f;
+        srow[tid] = (L2 && r < nq) ? qn[r] : 0.0f;
+        if constexpr (FUSED) stau[tid] = r < nq ? tau[r] : -inf;
     } else if (tid < MT + NT) {
+        // what a column adds to its entries: |b|^2 (L2) or 0, +inf for a tombstoned id; (FUSED) NaN beyond the end of
+        // the base, which no comparison passes
         const int64_t c = b0 + (tid - MT);
-        float v = 0.0f;
+        float v = FUSED ? nan : 0.0f;
         if (c < nb) {
-            if (metric == 0) v = bn[c];
+            v = L2 ? bn[c] : 0.0f;
             if (deleted) {
                 const int64_t id = base_id0 + c;
                 if ((deleted[id >> 5] >> (id & 31)) & 1u) v = inf;
@@ -164,12 +216,26 @@ __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel
         }
         scol[tid - MT] = v;
     }
+    if (tid == 0) s_nhit = 0u;
     __syncthreads();
+    // register v of block (ti, tj) in thread t: row and column inside the tile
+    auto row_of = [&](int t, int ti, int v) { return ((t >> 6) >> 1) * 64 + ti * 32 + 8 * (v >> 2) + 4 * ((t & 63) >> 5) + (v & 3); };
+    auto col_of = [&](int t, int tj) { return ((t >> 6) & 1) * 64 + tj * 32 + (t & 31); };
+    auto emit = [&](int rl, int cl, float sv) {
+        const int r = q0 + rl;
+        const unsigned pos = atomicAdd(&cnt[r], 1u);
+        if (pos < (unsigned)cap)
+            lists[(size_t)r * cap + pos] = ((unsigned long long)mf_ord32(sv) << 32) | (uint32_t)(base_id0 + b0 + cl);
+    };
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti) {
         float4 rown[4];  // |q|^2 of the 16 rows this lane holds of a block: four runs of four
+        float4 taun[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) rown[g] = *reinterpret_cast<const float4*>(srow + wr * 64 + ti * 32 + 8 * g + 4 * kh);
+        for (int g = 0; g < 4; ++g) {
+            rown[g] = *reinterpret_cast<const float4*>(srow + wr * 64 + ti * 32 + 8 * g + 4 * kh);
+            if constexpr (FUSED) taun[g] = *reinterpret_cast<const float4*>(stau + wr * 64 + ti * 32 + 8 * g + 4 * kh);
+        }
 #pragma unroll
         for (int tj = 0; tj < 2; ++tj) {
             const int cl = wc * 64 + tj * 32 + m;
@@ -177,16 +243,47 @@ __global__ __launch_bounds__(256, CORAL_MFMA_WAVES) void approx_tile_mfma_kernel
             const float bnc = scol[cl];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int r = q0 + wr * 64 + ti * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
                 const float4 rn4 = rown[v >> 2];
                 const float rn = (v & 3) == 0 ? rn4.x : (v & 3) == 1 ? rn4.y : (v & 3) == 2 ? rn4.z : rn4.w;
                 const float dot = acc[ti][tj][v];
-                // (|q|^2 + |b|^2) - 2 q.b; a tombstoned column's +inf survives both forms
-                const float s = metric == 0 ? (rn + bnc) - 2.0f * dot : (bnc == inf ? inf : 0.0f - dot);
-                if (r < nq && c < nb) D[(size_t)r * ldD + c] = s;
+                // (|q|^2 + |b|^2) - 2 q.b, or -q.b; a tombstoned column's +inf survives both forms
+                const float sv = L2 ? __fmaf_rn(-2.0f, dot, rn + bnc) : bnc - dot;
+                if constexpr (FUSED) {
+                    const float4 t4 = taun[v >> 2];
+                    const float tq = (v & 3) == 0 ? t4.x : (v & 3) == 1 ? t4.y : (v & 3) == 2 ? t4.z : t4.w;
+                    if (sv <= tq) {  // rows beyond nq have tau = -inf, columns beyond nb give NaN
+                        const unsigned pos = atomicAdd(&s_nhit, 1u);
+                        if (pos < (unsigned)kHitCap)
+                            shit[pos] = ((unsigned long long)mf_ord32(sv) << 32) | (unsigned)(((ti * 2 + tj) * 16 + v) << 8) | (unsigned)tid;
+                        else  // more hits than the tile's buffer holds: straight to the list
+                            emit(row_of(tid, ti, v), cl, sv);
+                    }
+                } else {
+                    const int r = q0 + row_of(tid, ti, v);
+                    if (r < nq && c < nb) D[(size_t)r * ldD + bt * NT + cl] = sv;
+                }
             }
         }
     }
+    if constexpr (FUSED) {
+        __syncthreads();
+        const int nhit = (int)min(s_nhit, (unsigned)kHitCap);
+        for (int i = tid; i < nhit; i += 256) {
+            const unsigned long long h = shit[i];
+            const int t = (int)(h & 0xffu), reg = (int)((h >> 8) & 0x3fu);
+            emit(row_of(t, reg >> 5, reg & 15), col_of(t, (reg >> 4) & 1), mf_unord32((uint32_t)(h >> 32)));
+        }
+    }
+}
+
+// tau[q] = value of the key keys[q * stride + j] (the j-th smallest of a sample of the row), +inf where the sample
+// has no j-th entry
+__global__ void bound_from_keys_kernel(const unsigned long long* __restrict__ keys, int64_t stride, int j, int nq,
+                                       float* __restrict__ tau) {
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= nq) return;
+    const unsigned long long key = keys[(size_t)q * stride + j];
+    tau[q] = key == ~0ull ? __int_as_float(0x7f800000) : mf_unord32((uint32_t)(key >> 32));
 }
 
 // One workgroup per query: the kc candidates (ids, -1 = none; approximate signed distances, ascending) are measured
@@ -288,15 +385,43 @@ hipError_t launch_row_norms(const float* x, int64_t n, int dim, float* out, uint
     return hipGetLastError();
 }
 
+#ifndef CORAL_MFMA_HQ
+#define CORAL_MFMA_HQ 16
+#endif
+constexpr int64_t kQueryTilesPerBlock = CORAL_MFMA_HQ;  // query tiles an XCD keeps in its L2 while it walks the base
+
 hipError_t launch_approx_tile(const float* queries, const float* base, int nq, int64_t nb, int dim, int metric,
                               const float* qn, const float* bn, const uint32_t* deleted, int64_t base_id0, float* D,
-                              int64_t ldD, hipStream_t stream) {
-    const int64_t nbt = (nb + NT - 1) / NT, nqt = (nq + MT - 1) / MT;
-    const int64_t wgs = (nbt + 7) / 8 * 8 * nqt;
-    if (wgs <= 0 || wgs > 0x7fffffff) return hipErrorInvalidValue;
+                              int64_t ldD, hipStream_t stream, int64_t sample_tiles, int64_t tile_stride) {
+    const int64_t nbt = sample_tiles > 0 ? sample_tiles : (nb + NT - 1) / NT, nqt = (nq + MT - 1) / MT;
+    const int64_t qblocks = (nqt + kQueryTilesPerBlock - 1) / kQueryTilesPerBlock, hq = (nqt + qblocks - 1) / qblocks;
+    const int64_t wgs = (nbt + 7) / 8 * 8 * qblocks * hq;
+    if (wgs <= 0 || wgs > 0x7fffffff || tile_stride < 1) return hipErrorInvalidValue;
     dim3 grid((unsigned)wgs);
-    hipLaunchKernelGGL(approx_tile_mfma_kernel, grid, dim3(256), 0, stream, queries, base, nq, nb, dim, metric, qn, bn,
-                       deleted, base_id0, D, ldD);
+    auto kernel = metric == 0 ? approx_tile_mfma_kernel<false, true> : approx_tile_mfma_kernel<false, false>;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, queries, base, nq, nb, dim, qn, bn, deleted, base_id0, nbt,
+                       tile_stride, (int)hq, D, ldD, (const float*)nullptr, (unsigned long long*)nullptr, (int64_t)0,
+                       (unsigned int*)nullptr);
+    return hipGetLastError();
+}
+
+hipError_t launch_approx_filter(const float* queries, const float* base, int nq, int64_t nb, int dim, int metric,
+                                const float* qn, const float* bn, const uint32_t* deleted, const float* tau,
+                                unsigned long long* lists, int64_t cap, unsigned int* cnt, hipStream_t stream) {
+    const int64_t nbt = (nb + NT - 1) / NT, nqt = (nq + MT - 1) / MT;
+    const int64_t qblocks = (nqt + kQueryTilesPerBlock - 1) / kQueryTilesPerBlock, hq = (nqt + qblocks - 1) / qblocks;
+    const int64_t wgs = (nbt + 7) / 8 * 8 * qblocks * hq;
+    if (wgs <= 0 || wgs > 0x7fffffff || nb > 0x7fffffff) return hipErrorInvalidValue;
+    dim3 grid((unsigned)wgs);
+    auto kernel = metric == 0 ? approx_tile_mfma_kernel<true, true> : approx_tile_mfma_kernel<true, false>;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, queries, base, nq, nb, dim, qn, bn, deleted, (int64_t)0, nbt,
+                       (int64_t)1, (int)hq, (float*)nullptr, (int64_t)0, tau, lists, cap, cnt);
+    return hipGetLastError();
+}
+
+hipError_t launch_bound_from_keys(const unsigned long long* keys, int64_t stride, int j, int nq, float* tau,
+                                  hipStream_t stream) {
+    hipLaunchKernelGGL(bound_from_keys_kernel, dim3((nq + 255) / 256), dim3(256), 0, stream, keys, stride, j, nq, tau);
     return hipGetLastError();
 }
 

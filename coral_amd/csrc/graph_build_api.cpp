@@ -388,7 +388,7 @@ static int build_impl(coral_index* idx, const float* h_aux, const int32_t* h_clu
     HIP_TRY(hipSetDevice(idx->device));
     const int dim = idx->dim, kb = prm->k_b;
     // the exact k_b-NN of a chunk of auxiliary queries at a time (KNNTask), then its batches in order (GraphTask)
-    const int64_t chunk = std::min<int64_t>(A, (int64_t)prm->batch * 8);
+    const int64_t chunk = std::min<int64_t>(A, (int64_t)prm->batch * 16);
     float* d_aux = nullptr;
     int32_t* d_knn = nullptr;
     int rc = CORAL_OK;

@@ -70,7 +70,8 @@ struct coral_index {
     // matrix-core screening pass is skipped
     float* d_bnorm = nullptr;
     uint32_t* d_bnorm_max = nullptr;
-    bool knn_exact_only = false;
+    int knn_mode = 0;             // 0: fused screening, 1: no screening, 2: screening through the distance matrix
+    bool knn_last_fused = false;  // the last call's candidates came from the fused screening
     int64_t knn_last_redone = 0;  // queries of the last call that went through the exact passes after screening
 
     // best-first on one wavefront per query: per-slot visited epochs in global memory

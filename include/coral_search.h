@@ -221,10 +221,16 @@ CORAL_API int coral_bruteforce_knn(coral_index* idx, const float* h_queries, int
                                    int32_t have_delete, int32_t* h_ids, float* h_dists, double* time_s);
 /* The search first screens all pairs with approximate distances from the matrix cores, keeps k + 32 candidates per
  * query, measures those in the reference's summation order and sends the rare query whose candidates cannot vouch
- * for the result through the plain passes: same ids and distance bits either way.  on = 1 skips the screening
- * (every pair in the reference's order on the vector units).  No counterpart in the reference (faiss does this work
- * there). */
+ * for the result through the plain passes: same ids and distance bits either way.  The candidates are selected
+ * inside the matrix-core kernel (entries up to a per-query bound, taken from a sample of the base, go to a short
+ * list per query; no distance matrix is written); where that does not apply -- k + 32 > 1024, a base of fewer than
+ * 64 sample tiles, a list that overflows -- the screening goes through the distance matrix instead.  on = 1 skips
+ * the screening (every pair in the reference's order on the vector units); on = 2 keeps the screening and always
+ * goes through the distance matrix; on = 0 restores the default.  No counterpart in the reference (faiss does this
+ * work there). */
 CORAL_API int coral_bruteforce_set_exact_only(coral_index* idx, int32_t on);
+/* 1 if the candidates of the last coral_bruteforce_knn* call were selected inside the matrix-core kernel */
+CORAL_API int32_t coral_bruteforce_last_fused(coral_index* idx);
 /* queries of the last coral_bruteforce_knn* call that went through the plain passes after the screening */
 CORAL_API int64_t coral_bruteforce_last_redone(coral_index* idx);
 

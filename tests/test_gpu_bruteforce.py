@@ -71,11 +71,16 @@ def test_bruteforce_exact_against_oracle(orc, n, dim, Q, k, metric, tomb):
     if tomb:
         idx.set_deleted(mask)
     ids, dists, _ = idx.bruteforce(q, k, have_delete=tomb)  # matrix-core screening + exact re-ranking
-    redone = idx.bruteforce_last_redone()
+    redone, fused = idx.bruteforce_last_redone(), idx.bruteforce_last_fused()
+    idx.bruteforce_exact_only(2)                            # the screening's candidates from the distance matrix
+    ids3, dists3, _ = idx.bruteforce(q, k, have_delete=tomb)
+    assert idx.bruteforce_last_fused() == 0 and idx.bruteforce_last_redone() == redone
+    assert np.array_equal(ids3, ids) and dists3.tobytes() == dists.tobytes()
     idx.bruteforce_exact_only(True)                         # every pair in the reference's order
     ids2, dists2, _ = idx.bruteforce(q, k, have_delete=tomb)
-    assert idx.bruteforce_last_redone() == 0
+    assert idx.bruteforce_last_redone() == 0 and idx.bruteforce_last_fused() == 0
     idx.close()
+    assert fused == (1 if n >= 8192 else 0)  # 64 tiles of 128 points are what the sample needs
     print("queries that the screening could not vouch for: %d of %d" % (redone, Q), flush=True)
     oi, od = orc.bruteforce(base, q, k, m, deleted=mask, order=SEQ)
     assert np.array_equal(ids, oi)
@@ -93,8 +98,9 @@ def test_bruteforce_exact_against_oracle(orc, n, dim, Q, k, metric, tomb):
 def test_randomised_knn_problems_equal_the_oracle(orc):
     """Seeded random sizes, k, metrics, tombstones and laws of the data (ties on a lattice, repeated vectors, large
     and small magnitudes, a common offset that makes the screening's error bound bite): the screened path and the
-    exact-only path both return the oracle's ids and distance bits."""
-    redone = 0
+    exact-only path both return the oracle's ids and distance bits; so does the screening with its candidates
+    selected from the distance matrix instead of inside the kernel."""
+    redone = fused = unfused = 0
     for c in range(80):
         rng = np.random.RandomState(7000 + c)
         n = int(rng.choice([50, 129, 300, 1000, 4097, 10000, 30000]))
@@ -127,13 +133,20 @@ def test_randomised_knn_problems_equal_the_oracle(orc):
         idx = capi.Index(base, None, None, metric)
         if tomb:
             idx.set_deleted(mask)
-        for exact_only in (False, True):
-            idx.bruteforce_exact_only(exact_only)
+        for mode in (0, 2, 1):
+            idx.bruteforce_exact_only(mode)
             ids, dists, _ = idx.bruteforce(q, k, have_delete=tomb)
-            redone += 0 if exact_only else idx.bruteforce_last_redone()
-            assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+            redone += idx.bruteforce_last_redone() if mode == 0 else 0
+            if mode == 0 and n >= 8192 and k + 32 <= 1024:
+                fused += idx.bruteforce_last_fused()
+                unfused += 1 - idx.bruteforce_last_fused()
+            else:
+                assert idx.bruteforce_last_fused() == 0
+            assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes(), "mode %d" % mode
         idx.close()
+    print("selection inside the kernel: %d cases, handed to the distance matrix: %d" % (fused, unfused), flush=True)
     assert redone > 0  # some of these queries went through the exact passes after the screening
+    assert fused > 0
 
 
 def test_bruteforce_ties_are_ordered_by_id(orc):
@@ -199,6 +212,12 @@ def test_bruteforce_ground_truth_at_full_size(orc):
     q = synth.shifted_queries(Q, dim, 2002, 2003, 2004)
     idx = capi.Index(base, ring(n), np.array([0], np.int32))
     ids, dists, t = idx.bruteforce(q, k)
+    assert idx.bruteforce_last_fused() == 1 and idx.bruteforce_last_redone() == 0
+    idx.bruteforce_exact_only(2)
+    ids_m, dists_m, t_m = idx.bruteforce(q, k)
+    idx.bruteforce_exact_only(0)
+    assert np.array_equal(ids_m, ids) and dists_m.tobytes() == dists.tobytes()
+    print("candidates selected inside the kernel: %.3f s; from the distance matrix: %.3f s" % (t, t_m), flush=True)
     pairs = float(Q) * n * dim
     print("brute force 10k x 1M x 200: %.3f s, %.2f T pair-dims/s (%.1f TFLOP/s at 3 flop per pair-dim)" %
           (t, pairs / t / 1e12, 3 * pairs / t / 1e12), flush=True)
