@@ -45,6 +45,10 @@ struct SearchArgs {
     // nullptr; tcap2 = entries of the list of rows it leaves for the exact pass (tcap, or 0 without screening)
     const unsigned char* vec16;
     size_t stride16;
+    // the same screening on a copy in eight-bit codes (rows stride8 bytes apart: codes, then scale, squared norm of
+    // the coded row and a bound of its distance to the row), or nullptr; taken when both are given
+    const unsigned char* vec8;
+    size_t stride8;
     int32_t tcap2;
     int32_t scap;              // BIG form: keys of the LDS sample of the beam that the merge searches first
     int32_t prefetch_rows;     // request a chunk's graph rows one chunk ahead (launches with one workgroup per CU)
@@ -123,6 +127,10 @@ hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& 
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening);
 // the half-precision copy of the vectors that the screening phase reads: bytes per row, and its construction
 size_t half_row_stride(int dim);
+// the copy in eight-bit codes (dim <= 512: a row's chunks of sixteen codes are read by sixteen lanes, two each at most)
+size_t byte_row_stride(int dim);
+hipError_t launch_byte_rows(const float* vec, int64_t n, int dim, unsigned char* out, hipStream_t stream);
+constexpr int kMaxByteRowDim = 512;
 hipError_t launch_half_rows(const float* vec, int64_t n, int dim, unsigned char* out, hipStream_t stream);
 // 64-bit words of global scratch one workgroup of a BIG launch needs for a beam of capacity L
 size_t search_beam_stride(int L);

@@ -184,6 +184,7 @@ void coral_index_destroy(coral_index* idx) {
     (void)hipFree(idx->d_spill);
     (void)hipFree(idx->d_beam);
     (void)hipFree(idx->d_vec16);
+    (void)hipFree(idx->d_vec8);
     (void)hipFree(idx->d_counters);
     (void)hipFree(idx->d_scalars);
     (void)hipFree(idx->d_hit);
@@ -274,13 +275,17 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     int id_bits = 1;
     while (id_bits < 31 && ((int64_t)1 << id_bits) < idx->n) ++id_bits;
     const size_t lds_max = (size_t)kMaxLdsBytes;
-    // ---- screening in half precision (rounds policy, L2, rows of 132 .. 2048 floats): see beam_search.hip
+    // ---- screening on a smaller copy of the vectors (rounds policy, L2, rows of 132 .. 2048 floats): eight-bit codes
+    // (tuning 2; the library's choice up to 512 floats) or half precision (tuning 1); see beam_search.hip
     // (best-first: the wavefront-per-query kernel with the beam in LDS screens too, see coral_search_prepare)
     const bool screen_possible = !best_first && idx->metric == CORAL_L2 && idx->dim / 4 > 32;
+    if (t.screening > 2 || t.screening < -1) return fail(CORAL_ERR_ARG, "screening must be -1, 0, 1 or 2 (got %d)", t.screening);
     if (t.screening > 0 && !(idx->metric == CORAL_L2 && idx->dim / 4 > 32))
         return fail(CORAL_ERR_ARG, "screening needs the L2 metric and more than 128 dimensions");
+    if (t.screening == 2 && idx->dim > coral::kMaxByteRowDim)
+        return fail(CORAL_ERR_ARG, "screening on eight-bit codes takes rows of up to %d floats", coral::kMaxByteRowDim);
     const bool screen = screen_possible && (t.screening > 0 || (t.screening == 0 && !no_screen));
-    p.screen = screen;
+    p.screen = !screen ? 0 : t.screening > 0 ? t.screening : (idx->dim <= coral::kMaxByteRowDim ? 2 : 1);
     // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
     // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
     // -1, or the library's choice): one LDS atomic per test and nothing ever overflows, at n / 8 bytes -- 125 KB for
@@ -411,12 +416,27 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
             (void)hipFree(p);
         return e;
     };
-    if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, false, false, &plan)) return rc;
+    auto ensure_vec8 = [&]() -> hipError_t {
+        if (idx->d_vec8) return hipSuccess;
+        const size_t bytes = coral::byte_row_stride(idx->dim) * (size_t)idx->n;
+        unsigned char* p = nullptr;
+        hipError_t e = hipMalloc(&p, bytes);
+        if (e != hipSuccess) return e;
+        e = hipMemsetAsync(p, 0, bytes, idx->stream);
+        if (e == hipSuccess) e = coral::launch_byte_rows(idx->d_vec, idx->n, idx->dim, p, idx->stream);
+        if (e == hipSuccess)
+            idx->d_vec8 = p;
+        else
+            (void)hipFree(p);
+        return e;
+    };
+    const int bump = idx->bump_L == L ? idx->bump_log2 : 0;
+    if (int rc = plan_search(idx, Q, L, t, bump, false, false, &plan)) return rc;
     if (plan.screen) {
-        const hipError_t e = ensure_vec16();
+        const hipError_t e = plan.screen == 2 ? ensure_vec8() : ensure_vec16();
         if (e == hipErrorOutOfMemory && t.screening == 0) {
             (void)hipGetLastError();
-            if (int rc = plan_search(idx, Q, L, t, idx->bump_L == L ? idx->bump_log2 : 0, false, true, &plan)) return rc;
+            if (int rc = plan_search(idx, Q, L, t, bump, false, true, &plan)) return rc;
         } else {
             HIP_TRY(e);
         }
@@ -601,7 +621,8 @@ static coral::SearchArgs search_args(const coral_index* idx, const coral_search_
     a.id_bits = p.id_bits, a.rem_bits = p.rem_bits, a.dmax = p.dmax, a.ocap = p.ocap;
     a.beam_stride = p.beam_stride, a.direct_bitmap = p.direct, a.table_words = p.table_words;
     a.prefetch_rows = p.prefetch;
-    a.vec16 = p.screen ? idx->d_vec16 : nullptr, a.stride16 = coral::half_row_stride(idx->dim);
+    a.vec16 = p.screen == 1 ? idx->d_vec16 : nullptr, a.stride16 = coral::half_row_stride(idx->dim);
+    a.vec8 = p.screen == 2 ? idx->d_vec8 : nullptr, a.stride8 = coral::byte_row_stride(idx->dim);
     a.tcap2 = p.screen ? p.tcap : 0;
     a.scap = p.big ? coral::kBeamSampleKeys : 0;
     return a;

@@ -24,7 +24,7 @@ struct coral_search_plan {
     bool big = false;         // beams in global memory (the kernel's BIG form)
     int direct = 0;           // the visited set is a bitmap of all ids in LDS
     int prefetch = 0;         // a chunk's graph rows are requested one chunk ahead
-    bool screen = false;      // rows are screened in half precision before their fp32 row is read
+    int screen = 0;           // rows are screened before their fp32 row is read: 1 in half precision, 2 in eight-bit codes
     int slots_log2 = 0, table_words = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
     int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0;
     size_t lds_bytes = 0;
@@ -50,6 +50,7 @@ struct coral_index {
     uint32_t* d_spill = nullptr;
     size_t spill_alloc_words = 0;
     unsigned char* d_vec16 = nullptr;  // half-precision copy of the vectors for the screening phase (made on first use)
+    unsigned char* d_vec8 = nullptr;   // copy in eight-bit codes for the screening phase (made on first use)
     uint64_t* d_beam = nullptr;  // beam blocks of a BIG launch, plan.workgroups x plan.beam_stride words
     size_t beam_alloc_words = 0;
     int32_t* d_counters = nullptr;

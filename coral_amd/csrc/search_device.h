@@ -30,6 +30,11 @@ __device__ __forceinline__ float dpp_mov(float x) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
 }
 
+template <int CTRL>
+__device__ __forceinline__ int dpp_mov_i(int x) {
+    return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, true);
+}
+
 // number of set bits of m below the calling lane
 __device__ __forceinline__ int prefix_popc(uint64_t m) {
     const uint32_t lane = threadIdx.x & 63;
