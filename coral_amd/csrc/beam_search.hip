@@ -195,7 +195,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
 
         for (int i = tid; i < a.table_words; i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
-        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0, s_cursor = 0;
+        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0, s_cursor = 0, s_ntodo2 = 0;
         __syncthreads();
 
         float4 qreg[CPL];
@@ -676,6 +676,21 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             __syncthreads();
         };
 
+        // ---- the rows the screening left open, todo2[0..s_ntodo2): exact distances (entered by every thread after a
+        // barrier; the candidates they add must fit the buffer)
+        const bool screening = (a.vec16 != nullptr || a.vec8 != nullptr) && a.policy == 0;
+        auto flush_exact = [&]() {
+            const int n2 = s_ntodo2;
+            if (n2 == 0) return;
+            if (s_ncand + n2 > CCAP) merge();  // merge() starts and ends with a barrier
+            PHASE_MARK(5);
+            distance_phase(todo2, n2);
+            __syncthreads();
+            if (tid == 0) s_ntodo2 = 0;
+            __syncthreads();
+            PHASE_MARK(4);
+        };
+
         PHASE_MARK(0);
         // ---- seeds: every start id is visited and measured, none counts as a hop
         const int M = a.M;
@@ -794,7 +809,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 const int T = s_ntodo;
                 nd += T;
                 PHASE_MARK(3);
-                if (s_ncand + T > CCAP) merge();  // merge() starts and ends with a barrier
+                if (!screening && s_ncand + T > CCAP) merge();  // merge() starts and ends with a barrier
                 PHASE_MARK(5);
                 if (tid == 0) s_nvis += T;
                 if (ahead) {
@@ -804,22 +819,23 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     if (pe < ech && e1 + pe < nexp) vpre = a.nbrs[(size_t)epre * R + pj];
                     if (pe < ech && e2 + pe < nexp) epre = elist[e2 + pe];
                 }
-                if ((a.vec16 != nullptr || a.vec8 != nullptr) && a.policy == 0) {
-                    if (tid == 0) s_ntodo2 = 0;
-                    __syncthreads();
+                if (screening) {
+                    // what the screening leaves for the exact pass collects over the chunks of a round (the round's
+                    // threshold does not move) and is measured when the list could overflow, and at the round's end
+                    if (s_ntodo2 + T > a.tcap2) flush_exact();
                     if (a.vec8 != nullptr)
                         screening_phase8(T);
                     else
                         screening_phase(T);
                     __syncthreads();
                     PHASE_MARK(7);
-                    distance_phase(todo2, s_ntodo2);
                 } else {
                     distance_phase(todo, T);
                 }
                 __syncthreads();
                 PHASE_MARK(4);
             }
+            if (screening) flush_exact();
             ++rounds;
             const int cntf = s_cntf;
             if (a.policy == 0) {
