@@ -69,28 +69,35 @@ struct BestFirstArgs {
     // buckets of four; rem_bits = the bits of the mixed id (id_bits wide) that a cell stores, at most 14; what
     // finds its two buckets full goes to the state in HBM
     int32_t table_log2, id_bits, rem_bits;
-    // screening: the half-precision copy of the vectors (see SearchArgs), or nullptr
+    // screening: the half-precision copy of the vectors, or the copy in eight-bit codes (see SearchArgs); one of them
+    // or neither.  coded_bytes: LDS a wavefront keeps for its query in integer codes (with vec8; else 0)
     const unsigned char* vec16;
     size_t stride16;
+    const unsigned char* vec8;
+    size_t stride8;
+    int32_t coded_bytes;
 };
 
 // LDS bytes of one wavefront: a beam of L keys, 32 candidate keys, two lists of 32 ids, L byte counters, a Bloom filter of
 // 2^bloom_log2 bits over the visited ids in HBM (bloom_log2 = 0: none) and a table of 2^table_log2 16-bit cells
 // (table_log2 = 0: none)
-__host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2, int table_log2 = 0) {
+__host__ __device__ inline size_t best_first_wave_lds_bytes(int L, int bloom_log2, int table_log2 = 0, int coded_bytes = 0) {
     const size_t bloom = bloom_log2 ? ((size_t)1 << bloom_log2) / 8 : 0;
     const size_t table = table_log2 ? (size_t)2 << table_log2 : 0;
-    return ((size_t)((L + 3) & ~3) * 9 + 32 * 8 + 2 * 32 * 4 + bloom + table + 15) & ~(size_t)15;
+    return ((size_t)((L + 3) & ~3) * 9 + 32 * 8 + 2 * 32 * 4 + bloom + table + (size_t)coded_bytes + 15) & ~(size_t)15;
 }
+// LDS of a wavefront's query in integer codes for the screening on eight-bit rows: two bytes per dimension
+__host__ __device__ inline int coded_query_bytes(int dim) { return 2 * ((dim + 15) & ~15); }
 // the filter size for a beam of L: 128 bits per beam entry rounded up to a power of two, halved while that would leave
 // a CU fewer than sixteen wavefronts; none below 4096 bits
-__host__ inline int best_first_bloom_log2(int L) {
+__host__ inline int best_first_bloom_log2(int L, int coded_bytes = 0) {
     int lg = 12;
     while (((size_t)1 << lg) < (size_t)128 * L && lg < 17) ++lg;
-    while (lg >= 12 && best_first_wave_lds_bytes(L, lg) > (size_t)10 * 1024) --lg;
+    while (lg >= 12 && best_first_wave_lds_bytes(L, lg, 0, coded_bytes) > (size_t)10 * 1024) --lg;
     return lg >= 12 ? lg : 0;
 }
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, bool screen, int bloom_log2,
+// screen: 0 none, 1 rows are first measured in half precision, 2 in eight-bit codes (rows of up to 512 floats)
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int screen, int bloom_log2,
                               int table_log2, int* max_wg_per_cu);
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream);
 // *flag (a device word, zero before) becomes nonzero if a row of nbrs [n][R] holds the same id twice

@@ -59,8 +59,9 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
 
 // PACKED: the visited state of a slot is one 32-bit word per 24 nodes (8 bits of epoch, 24 flags) instead of one
 // byte per node: a sixth of the memory, the same one line per test.
-// SCREEN: rows are measured in the half-precision copy of the vectors first (b.vec16; rows of more than 128 floats).
-template <int G, int CPL, int RIF, bool PACKED, bool SCREEN>
+// SCREEN: rows are first measured in a smaller copy of the vectors (rows of more than 128 floats): 1 the half-precision
+// copy (b.vec16), 2 the copy in eight-bit codes (b.vec8; rows of up to 512 floats).
+template <int G, int CPL, int RIF, bool PACKED, int SCREEN>
 __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
     if (slot >= b.slots) return;  // the whole wavefront; no workgroup barrier is used below
     const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2, M = a.M;
     const int Lp = (L + 3) & ~3;
-    unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L, b.bloom_log2, b.table_log2);
+    unsigned char* mine_lds = smem + (size_t)wave * best_first_wave_lds_bytes(L, b.bloom_log2, b.table_log2, b.coded_bytes);
     uint64_t* beam = reinterpret_cast<uint64_t*>(mine_lds);      // L keys, sorted
     uint64_t* cand = beam + Lp;                                   // kBatch keys
     uint32_t* todo = reinterpret_cast<uint32_t*>(cand + kBatch);  // kBatch ids
@@ -82,6 +83,8 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
     // is looked up as before.  Two multiplicative hashes.
     const int bl = b.bloom_log2;
     const int bloom_words = bl ? (1 << bl) >> 5 : 0;
+    signed char* qh8 = reinterpret_cast<signed char*>(bloom + bloom_words);  // the query in integer codes (SCREEN == 2)
+    signed char* ql8 = qh8 + ((dim + 15) & ~15);
     auto bloom_bits = [&](uint32_t id, uint32_t& h1, uint32_t& h2) {
         h1 = (id * 0x9E3779B1u) >> (32 - bl);
         h2 = (id * 0x85EBCA77u + 0x3C6EF372u) >> (32 - bl);
@@ -200,6 +203,40 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             }
         }
 
+        // The query in integer codes for the screening on eight-bit rows (see beam_search.hip): q~_i = sq (128 h_i +
+        // l_i), bytes h_i and l_i in LDS; |q~|^2, sq and |q - q~| (rounded up) in registers.
+        float c_qq = 0.0f, c_sq = 0.0f, c_eq = 0.0f;
+        if constexpr (SCREEN == 2) {
+            const float* qv = a.queries + (size_t)qid * dim;
+            float amax = 0.0f;
+            bool bad = false;
+            for (int i = lane; i < dim; i += 64) {
+                const float v = fabsf(qv[i]);
+                bad |= !(v <= 3.0e38f);
+                amax = fmaxf(amax, v);
+            }
+            for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            bad = __ballot(bad) != 0ull || (amax != 0.0f && !(amax >= 1.0e-18f && amax <= 1.0e17f));
+            const float sq = bad ? 0.0f : amax / 16256.0f;
+            double se = 0.0, sx = 0.0;
+            for (int i = lane; i < ((dim + 15) & ~15); i += 64) {
+                const float v = i < dim ? qv[i] : 0.0f;
+                int code = 0;
+                if (sq > 0.0f) {
+                    code = (int)rintf(v / sq);
+                    code = code > 16256 ? 16256 : (code < -16256 ? -16256 : code);
+                }
+                const int h = (code + 64) >> 7, l = code - 128 * h;
+                qh8[i] = (signed char)h, ql8[i] = (signed char)l;
+                const double qt = (double)sq * (double)code, dv = (double)v - qt;
+                se += dv * dv, sx += qt * qt;
+            }
+            for (int off = 32; off > 0; off >>= 1) se += __shfl_xor(se, off, 64), sx += __shfl_xor(sx, off, 64);
+            c_qq = (float)sx, c_sq = sq;
+            c_eq = bad ? __int_as_float(0x7f800000) : (float)(sqrt(se) * 1.000001) * (1.0f + 2.0e-7f);
+            wave_sync();
+        }
+
         int nb = 0, cursor = 0;
         uint64_t live = kKeyMax;
         int hops = M, nd = M, ne = 0, rounds = 0;
@@ -210,7 +247,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             // Screening (see beam_search.hip): each row is first measured in the half-precision copy of the vectors;
             // a row whose exact distance is certainly beyond the beam's worst entry is dropped without reading its
             // fp32 row -- most of what a search measures once its beam is full.
-            if (SCREEN && G == 64 && nb == L) {
+            if (SCREEN == 1 && G == 64 && nb == L) {
                 constexpr int UH = U > kScreenRows ? kScreenRows : U;
                 constexpr int RPIH = 2 * UH;
                 const int glh = lane & 31, grph = lane >> 5;
@@ -298,6 +335,88 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 wave_sync();
                 list = todo2;
                 T = n2;
+            }
+            if constexpr (SCREEN == 2 && G == 64 && CPL <= 2) {
+              if (nb == L) {
+                // the same on eight-bit codes: sixteen lanes per row, all 32 rows of a step in one round of requests
+                constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
+                const int gl8 = lane & 15, grp8 = lane >> 4;
+                const int nck = (dim + 15) >> 4;
+                const float s_live = key_s(live);
+                int qh[CPL8][4], ql[CPL8][4];
+#pragma unroll
+                for (int t = 0; t < CPL8; ++t)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int c = gl8 + 16 * t;
+                        qh[t][j] = c < nck ? reinterpret_cast<const int*>(qh8)[4 * c + j] : 0;
+                        ql[t][j] = c < nck ? reinterpret_cast<const int*>(ql8)[4 * c + j] : 0;
+                    }
+                int n2 = 0;
+                for (int base = 0; base < T; base += RPI8) {
+                    int vid[U8];
+                    const int r0 = base + grp8 * U8;
+#pragma unroll
+                    for (int u = 0; u < U8; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
+                    uint4 hb[U8][CPL8];
+#pragma unroll
+                    for (int u = 0; u < U8; ++u) {
+                        const uint4* row = reinterpret_cast<const uint4*>(
+                            b.vec8 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * b.stride8);
+#pragma unroll
+                        for (int t = 0; t < CPL8; ++t) {
+                            const int c = gl8 + 16 * t;
+                            hb[u][t] = (vid[u] >= 0 && c < nck) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
+                        }
+                    }
+                    int myid = vid[0];
+#pragma unroll
+                    for (int u = 1; u < U8; ++u)
+                        if (gl8 == u) myid = vid[u];
+                    const bool valid = gl8 < U8 && myid >= 0;
+                    float4 fig = make_float4(0, 0, 0, 0);
+                    if (valid)
+                        fig = *reinterpret_cast<const float4*>(b.vec8 + (uint64_t)(uint32_t)myid * b.stride8 + (size_t)nck * 16);
+                    int acc[U8];
+#pragma unroll
+                    for (int u = 0; u < U8; ++u) {
+                        int dh = 0, dl = 0;
+#pragma unroll
+                        for (int t = 0; t < CPL8; ++t) {
+                            const int w[4] = {(int)hb[u][t].x, (int)hb[u][t].y, (int)hb[u][t].z, (int)hb[u][t].w};
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                dh = __builtin_amdgcn_sdot4(w[j], qh[t][j], dh, false);
+                                dl = __builtin_amdgcn_sdot4(w[j], ql[t][j], dl, false);
+                            }
+                        }
+                        acc[u] = 128 * dh + dl;
+                    }
+#pragma unroll
+                    for (int u = 0; u < U8; ++u) {
+                        acc[u] = acc[u] + dpp_mov_i<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
+                        acc[u] = acc[u] + dpp_mov_i<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
+                        acc[u] = acc[u] + dpp_mov_i<0x141>(acc[u]);  // row_half_mirror
+                        acc[u] = acc[u] + dpp_mov_i<0x140>(acc[u]);  // row_mirror
+                    }
+                    int mine = acc[0];
+#pragma unroll
+                    for (int u = 1; u < U8; ++u)
+                        if (gl8 == u) mine = acc[u];
+                    const float both = c_qq + fig.y;
+                    const float d8 = both - (2.0f * c_sq * fig.x) * (float)mine;
+                    const float delta = 16.0f * 5.9604645e-8f * both, e = fig.z + c_eq;
+                    const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
+                    const float lo = lo_root * lo_root * (1.0f - 1.0e-4f);
+                    const bool exact = valid && !(lo > s_live);
+                    const uint64_t m = __ballot(exact);
+                    if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;
+                    n2 += __popcll(m);
+                }
+                wave_sync();
+                list = todo2;
+                T = n2;
+              }
             }
             int nc = 0;
             for (int base = 0; base < T; base += RPI) {
@@ -554,18 +673,19 @@ using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 // RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
 // dependent memory waits of a step against 8 and needs 128 registers; 32 (a whole step at once, 212 registers) is
 // for launches whose LDS holds a CU to eight wavefronts anyway (+2..3 %)
-template <int RIF, bool PACKED, bool SCREEN>
+template <int RIF, bool PACKED, int SCREEN>
 bf_kernel_fn pick_bf_kernel_rif(int chunks) {
-    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED, false>;
-    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, false>;
+    constexpr int WIDE = SCREEN == 2 ? 1 : SCREEN;  // rows of more than 512 floats have no copy in eight-bit codes
+    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED, 0>;
+    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, 0>;
     if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED, SCREEN>;
     if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED, SCREEN>;
-    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED, SCREEN>;
-    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED, SCREEN>;
+    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED, WIDE>;
+    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED, WIDE>;
     return nullptr;
 }
 
-template <bool SCREEN>
+template <int SCREEN>
 bf_kernel_fn pick_bf_kernel_screen(int dim, int rif, bool packed) {
     // 32: for launches that hold eight wavefronts per CU or fewer (256 registers per lane); rows of 17..64 chunks
     if (rif >= 32 && dim / 4 > 16 && dim / 4 <= 64)
@@ -575,17 +695,20 @@ bf_kernel_fn pick_bf_kernel_screen(int dim, int rif, bool packed) {
     return rif >= 16 ? pick_bf_kernel_rif<16, false, SCREEN>(dim / 4) : pick_bf_kernel_rif<8, false, SCREEN>(dim / 4);
 }
 
-bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed, bool screen) {
-    return screen ? pick_bf_kernel_screen<true>(dim, rif, packed) : pick_bf_kernel_screen<false>(dim, rif, packed);
+bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed, int screen) {
+    return screen == 2   ? pick_bf_kernel_screen<2>(dim, rif, packed)
+           : screen == 1 ? pick_bf_kernel_screen<1>(dim, rif, packed)
+                         : pick_bf_kernel_screen<0>(dim, rif, packed);
 }
 
 }  // namespace
 
-hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, bool screen, int bloom_log2,
+hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int screen, int bloom_log2,
                               int table_log2, int* max_wg_per_cu) {
+    if (screen == 2 && dim > kMaxByteRowDim) return hipErrorInvalidValue;
     bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed, screen);
     if (!fn) return hipErrorInvalidValue;
-    const size_t lds = best_first_wave_lds_bytes(L, bloom_log2, table_log2) * kWavesPerWg;
+    const size_t lds = best_first_wave_lds_bytes(L, bloom_log2, table_log2, screen == 2 ? coded_query_bytes(dim) : 0) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -597,11 +720,13 @@ hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, b
 }
 
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream) {
-    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0, b.vec16 != nullptr);
+    const int screen = b.vec8 != nullptr ? 2 : b.vec16 != nullptr ? 1 : 0;
+    if (screen == 2 && (a.dim > kMaxByteRowDim || b.coded_bytes != coded_query_bytes(a.dim))) return hipErrorInvalidValue;
+    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0, screen);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64),
-                       best_first_wave_lds_bytes(a.L, b.bloom_log2, b.table_log2) * kWavesPerWg, stream, a, b);
+                       best_first_wave_lds_bytes(a.L, b.bloom_log2, b.table_log2, b.coded_bytes) * kWavesPerWg, stream, a, b);
     return hipGetLastError();
 }
 

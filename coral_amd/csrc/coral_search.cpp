@@ -488,16 +488,19 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // Best-first, one wavefront per query: the visited state lives in HBM, n bytes per wavefront (n / 6 in the packed
     // form), up to a third of what is free and 64 GiB.  wg_per_cu: what the chosen kernel's occupancy allows;
     // reprepare(packed): sets that kernel up in the packed form and returns its occupancy.
-    idx->bf_ready = false, idx->bf_long = false, idx->bf_screen = false;
+    idx->bf_ready = false, idx->bf_long = false, idx->bf_screen = 0;
     // Best-first with the beam in LDS screens rows in half precision too, where a CU holds sixteen wavefronts (beams
     // without the LDS table: L > 409): +12 % at L = 512 and 1024.  With the table (eight wavefronts per CU) the extra
     // wait per step costs more than the bytes it spares (L = 256 / 320: -27 %), so those launches go without unless
     // the caller asks for it by name.
     if (wave_form && idx->metric == CORAL_L2 && idx->dim / 4 > 32 &&
         (t.screening > 0 || (t.screening == 0 && table_log2 == 0))) {
-        const hipError_t e = ensure_vec16();
+        // eight-bit codes where they apply; launches with the LDS table (whose size was chosen to fill LDS) and rows of
+        // more than 512 floats screen in half precision
+        const int form = t.screening == 1 || idx->dim > coral::kMaxByteRowDim || table_log2 != 0 ? 1 : 2;
+        const hipError_t e = form == 2 ? ensure_vec8() : ensure_vec16();
         if (e == hipSuccess) {
-            idx->bf_screen = true;
+            idx->bf_screen = form;
         } else if (e == hipErrorOutOfMemory && t.screening == 0) {
             (void)hipGetLastError();
         } else {
@@ -558,7 +561,8 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
             rif = 32;
         idx->bf_rows_in_flight = rif;
         // with a table the filter would only cover what outgrew it, and its LDS is worth more as cells
-        const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L);
+        const int coded = idx->bf_screen == 2 ? coral::coded_query_bytes(idx->dim) : 0;
+        const int bloom_log2 = table_log2 ? 0 : coral::best_first_bloom_log2(L, coded);
         idx->bf_bloom_log2 = bloom_log2;
         HIP_TRY(coral::best_first_prepare(idx->dim, L, rif, false, idx->bf_screen, bloom_log2, table_log2, &bf_wg_per_cu));
         auto reprepare = [&](int* occ) {
@@ -689,7 +693,9 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         b.visited = idx->d_bf_visited, b.epochs = idx->d_bf_epochs, b.stride = idx->bf_stride;
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_in_flight = idx->bf_rows_in_flight;
-        b.vec16 = idx->bf_screen ? idx->d_vec16 : nullptr, b.stride16 = coral::half_row_stride(idx->dim);
+        b.vec16 = idx->bf_screen == 1 ? idx->d_vec16 : nullptr, b.stride16 = coral::half_row_stride(idx->dim);
+        b.vec8 = idx->bf_screen == 2 ? idx->d_vec8 : nullptr, b.stride8 = coral::byte_row_stride(idx->dim);
+        b.coded_bytes = idx->bf_screen == 2 ? coral::coded_query_bytes(idx->dim) : 0;
         HIP_TRY(coral::launch_best_first(a, b, stream));
     } else {
         const int wgs = std::min(plan.workgroups, (int)Q);

@@ -83,7 +83,7 @@ struct coral_index {
     int bf_slots = 0, bf_alloc_slots = 0, bf_rows_in_flight = 8, bf_packed = 0, bf_bloom_log2 = 0;
     int bf_table_log2 = 0, bf_table_rem_bits = 0;
     // ... or, for long beams, with an insert buffer in LDS and the long sorted run of every slot in global memory
-    bool bf_screen = false;  // the kernel with the beam in LDS screens rows in half precision (d_vec16)
+    int bf_screen = 0;  // the kernel with the beam in LDS screens rows: 1 in half precision (d_vec16), 2 in eight-bit codes (d_vec8)
     bool bf_long = false;
     uint64_t* d_bf_beams = nullptr;
     size_t bf_beam_alloc_words = 0, bf_beam_stride = 0;
