@@ -121,14 +121,21 @@ struct BestFirstLongArgs {
     int32_t bcap;        // keys of the sorted insert buffer in LDS, a multiple of 64
     int32_t scap;        // keys of the LDS sample of the long run
     int32_t sshift;      // the sample holds every 2^sshift-th key: ((L - 1) >> sshift) + 1 <= scap
+    // screening: the copy of the vectors in eight-bit codes (see SearchArgs), or nullptr; coded_bytes: LDS a wavefront
+    // keeps for its query in integer codes and the list the screening leaves (with vec8; else 0)
+    const unsigned char* vec8;
+    size_t stride8;
+    int32_t coded_bytes;
 };
 // LDS bytes of one wavefront: the insert buffer, a copy of the long run's last bcap + 32 keys, two samples, 32 candidate
 // keys, 32 ids, bcap byte counters
-__host__ __device__ inline size_t best_first_long_lds_bytes(int bcap, int scap) {
-    return ((size_t)bcap * 8 + (size_t)(bcap + 32) * 8 + (size_t)scap * 16 + 32 * 8 + 32 * 4 + (size_t)bcap + 15) &
-           ~(size_t)15;
+__host__ __device__ inline size_t best_first_long_lds_bytes(int bcap, int scap, int coded_bytes = 0) {
+    return ((size_t)bcap * 8 + (size_t)(bcap + 32) * 8 + (size_t)scap * 16 + 32 * 8 + 32 * 4 + (size_t)bcap +
+            (size_t)coded_bytes + 15) & ~(size_t)15;
 }
-hipError_t best_first_long_prepare(int dim, bool packed, int bcap, int scap, int* max_wg_per_cu);
+// with screening on eight-bit codes: the coded query and a second list of 32 ids
+__host__ __device__ inline int best_first_long_coded_bytes(int dim) { return coded_query_bytes(dim) + 32 * 4; }
+hipError_t best_first_long_prepare(int dim, bool packed, bool screen, int bcap, int scap, int* max_wg_per_cu);
 hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& b, hipStream_t stream);
 
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening);

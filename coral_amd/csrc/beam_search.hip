@@ -204,42 +204,14 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             const int c = gl + G * t;
             qreg[t] = c < chunks ? reinterpret_cast<const float4*>(qs)[c] : make_float4(0, 0, 0, 0);
         }
-        // The query in integer codes for the screening on eight-bit rows: q~_i = sq (128 h_i + l_i) with bytes h_i in
-        // [-127, 127] and l_i in [-64, 63], sq = max |q_i| / 16256, so that sum q~_i k_i is two integer dot products;
-        // |q~|^2 and |q - q~| (rounded up) from sums in double precision.  A query with a component that is not
-        // finite, or whose largest lies outside [1e-18, 1e17], gets an infinite error: every row goes to the exact pass.
-        // (Written by wave 0 alone; first read after the barriers of the seeds' merge.)
+        // The query in integer codes for the screening on eight-bit rows (search_device.h).  Written by wave 0 alone;
+        // first read after the barriers of the seeds' merge.
         signed char* qh8 = reinterpret_cast<signed char*>(qs + ((dim + 3) & ~3));
         signed char* ql8 = qh8 + ((dim + 15) & ~15);
         if (a.vec8 != nullptr && wave == 0) {
-            float amax = 0.0f;
-            bool bad = false;
-            for (int i = lane; i < dim; i += 64) {
-                const float v = fabsf(qs[i]);
-                bad |= !(v <= 3.0e38f);
-                amax = fmaxf(amax, v);
-            }
-            for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-            bad = __ballot(bad) != 0ull || (amax != 0.0f && !(amax >= 1.0e-18f && amax <= 1.0e17f));
-            const float sq = bad ? 0.0f : amax / 16256.0f;
-            double se = 0.0, sx = 0.0;
-            for (int i = lane; i < ((dim + 15) & ~15); i += 64) {
-                const float v = i < dim ? qs[i] : 0.0f;
-                int code = 0;
-                if (sq > 0.0f) {
-                    code = (int)rintf(v / sq);
-                    code = code > 16256 ? 16256 : (code < -16256 ? -16256 : code);
-                }
-                const int h = (code + 64) >> 7, l = code - 128 * h;
-                qh8[i] = (signed char)h, ql8[i] = (signed char)l;
-                const double qt = (double)sq * (double)code, dv = (double)v - qt;
-                se += dv * dv, sx += qt * qt;
-            }
-            for (int off = 32; off > 0; off >>= 1) se += __shfl_xor(se, off, 64), sx += __shfl_xor(sx, off, 64);
-            if (lane == 0) {
-                s_qq = (float)sx, s_qscale = sq;
-                s_qerr = bad ? __int_as_float(0x7f800000) : (float)(sqrt(se) * 1.000001) * (1.0f + 2.0e-7f);
-            }
+            float qq, sq, eq;
+            code_query(qs, dim, lane, qh8, ql8, qq, sq, eq);
+            if (lane == 0) s_qq = qq, s_qscale = sq, s_qerr = eq;
         }
 
         WgState st;
@@ -356,109 +328,45 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             }
         };
 
-        // ---- screening phase on eight-bit codes (launches with a.vec8): the same three classes from a quarter of
-        // the bytes.  Row x is stored as codes k_i in [-127, 127] with x~_i = s k_i, s = max |x_i| / 127, followed by
-        // s, |x~|^2 and e >= |x - x~| (rounded up; infinite for rows that take no part); the query is coded likewise
-        // (above), with error eq.  D = |q~ - x~|^2 = |q~|^2 + |x~|^2 - 2 sq s sum (128 h_i + l_i) k_i needs integer dot
-        // products only (v_dot4_i32_i8, exact), and the exact distance d satisfies
-        // (sqrt(D) - e - eq)^2 <= d <= (sqrt(D) + e + eq)^2.  The computed D is within delta = 16 * 2^-24 (|q~|^2 + |x~|^2)
-        // of its true value (the conversion of the integer sum, the product of the scales, the two stored norms and
-        // the two final additions: each relative 2^-24 of a quantity no larger than |q~|^2 + |x~|^2; taken twice);
-        // both ends are widened by 1e-4 for the fp32 rounding of the exact distance itself, as in the half-precision
-        // phase.  Sixteen lanes per row (a 256-byte row at dim 200: two cache lines), eight rows in flight per group,
-        // four groups per wavefront.
+        // ---- screening phase on eight-bit codes (launches with a.vec8; bounds: search_device.h): the same three
+        // classes from a quarter of the bytes.  Sixteen lanes per row (a 256-byte row at dim 200: two cache lines),
+        // eight rows in flight per group, four groups per wavefront.
         auto screening_phase8 = [&](int T) {
-          if constexpr (G == 64 && CPL <= 2) {  // dim <= 512: a row's code chunks are CPL per lane of its sixteen
-            constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
-            const int gl8 = lane & 15, grp8 = lane >> 4;
-            const int nck = (dim + 15) >> 4;  // chunks of sixteen codes; the row's three figures are chunk nck
-            int qh[CPL8][4], ql[CPL8][4];
+            if constexpr (G == 64 && CPL <= 2) {  // dim <= 512: a row's code chunks are CPL per lane of its sixteen
+                constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
+                const int gl8 = lane & 15, grp8 = lane >> 4;
+                const int nck = (dim + 15) >> 4;  // chunks of sixteen codes; the row's three figures are chunk nck
+                CodedQuery<CPL8> cq;
+                load_coded_query<CPL8>(qh8, ql8, nck, gl8, cq);
+                const float qq = s_qq, sq = s_qscale, eq = s_qerr;
+                const float s_live = st.live == kKeyMax ? 3.402823466e+38f : key_s(st.live);
+                int cnt = 0;
+                for (int base = wave * RPI8; base < T; base += NW * RPI8) {
+                    int vid[U8];
+                    const int r0 = base + grp8 * U8;
 #pragma unroll
-            for (int t = 0; t < CPL8; ++t)
+                    for (int u = 0; u < U8; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int c = gl8 + 16 * t;
-                    qh[t][j] = c < nck ? reinterpret_cast<const int*>(qh8)[4 * c + j] : 0;
-                    ql[t][j] = c < nck ? reinterpret_cast<const int*>(ql8)[4 * c + j] : 0;
-                }
-            const float qq = s_qq, sq2 = 2.0f * s_qscale, eq = s_qerr;
-            const float kdelta = 16.0f * 5.9604645e-8f;
-            const float s_live = st.live == kKeyMax ? 3.402823466e+38f : key_s(st.live);
-            int cnt = 0;
-            for (int base = wave * RPI8; base < T; base += NW * RPI8) {
-                int vid[U8];
-                const int r0 = base + grp8 * U8;
-#pragma unroll
-                for (int u = 0; u < U8; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
-#pragma unroll
-                for (int u = 0; u < U8; ++u)
-                    if (r0 + u >= T) vid[u] = -1;
-                uint4 hb[U8][CPL8];
-#pragma unroll
-                for (int u = 0; u < U8; ++u) {
-                    const uint4* row = reinterpret_cast<const uint4*>(
-                        a.vec8 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * a.stride8);
-#pragma unroll
-                    for (int t = 0; t < CPL8; ++t) {
-                        const int c = gl8 + 16 * t;
-                        hb[u][t] = (vid[u] >= 0 && c < nck) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
+                    for (int u = 0; u < U8; ++u)
+                        if (r0 + u >= T) vid[u] = -1;
+                    int myid;
+                    bool valid;
+                    float lo, hi;
+                    coded_rows_bounds<CPL8, U8>(a.vec8, a.stride8, nck, gl8, vid, cq, qq, sq, eq, myid, valid, lo, hi);
+                    const bool gone = valid && lo > thr;
+                    const bool counted = valid && !gone && hi < thr && lo > s_live;
+                    const bool exact = valid && !gone && !counted;
+                    cnt += __popcll(__ballot(counted));
+                    const uint64_t m = __ballot(exact);
+                    if (m) {
+                        int pos = 0;
+                        if (lane == 0) pos = atomicAdd(&s_ntodo2, __popcll(m));
+                        pos = __shfl(pos, 0, 64);
+                        if (exact) todo2[pos + prefix_popc(m)] = (uint32_t)myid;
                     }
                 }
-                // the row this lane will file, and its three figures
-                int myid = vid[0];
-#pragma unroll
-                for (int u = 1; u < U8; ++u)
-                    if (gl8 == u) myid = vid[u];
-                const bool valid = gl8 < U8 && myid >= 0;
-                float4 fig = make_float4(0, 0, 0, 0);
-                if (valid)
-                    fig = *reinterpret_cast<const float4*>(a.vec8 + (uint64_t)(uint32_t)myid * a.stride8 + (size_t)nck * 16);
-                int acc[U8];
-#pragma unroll
-                for (int u = 0; u < U8; ++u) {
-                    int dh = 0, dl = 0;
-#pragma unroll
-                    for (int t = 0; t < CPL8; ++t) {
-                        const int w[4] = {(int)hb[u][t].x, (int)hb[u][t].y, (int)hb[u][t].z, (int)hb[u][t].w};
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            dh = __builtin_amdgcn_sdot4(w[j], qh[t][j], dh, false);
-                            dl = __builtin_amdgcn_sdot4(w[j], ql[t][j], dl, false);
-                        }
-                    }
-                    acc[u] = 128 * dh + dl;  // below 2^31 for 512 dimensions: 512 * 127 * 16256
-                }
-#pragma unroll
-                for (int u = 0; u < U8; ++u) {
-                    acc[u] = acc[u] + dpp_mov_i<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
-                    acc[u] = acc[u] + dpp_mov_i<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
-                    acc[u] = acc[u] + dpp_mov_i<0x141>(acc[u]);  // row_half_mirror
-                    acc[u] = acc[u] + dpp_mov_i<0x140>(acc[u]);  // row_mirror
-                }
-                int mine = acc[0];
-#pragma unroll
-                for (int u = 1; u < U8; ++u)
-                    if (gl8 == u) mine = acc[u];
-                const float both = qq + fig.y;
-                const float d8 = both - (sq2 * fig.x) * (float)mine, delta = kdelta * both, e = fig.z + eq;
-                const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
-                const float hi_root = sqrtf(fmaxf(d8 + delta, 0.0f)) + e;
-                const float lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
-                // (a row that takes no part has e = inf: lo = 0, hi = inf; a NaN anywhere fails both comparisons)
-                const bool gone = valid && lo > thr;
-                const bool counted = valid && !gone && hi < thr && lo > s_live;
-                const bool exact = valid && !gone && !counted;
-                cnt += __popcll(__ballot(counted));
-                const uint64_t m = __ballot(exact);
-                if (m) {
-                    int pos = 0;
-                    if (lane == 0) pos = atomicAdd(&s_ntodo2, __popcll(m));
-                    pos = __shfl(pos, 0, 64);
-                    if (exact) todo2[pos + prefix_popc(m)] = (uint32_t)myid;
-                }
+                if (lane == 0 && cnt) atomicAdd(&s_cntf, cnt);
             }
-            if (lane == 0 && cnt) atomicAdd(&s_cntf, cnt);
-          }
         };
 
         // ---- distance phase: list[0..T) -> cand[], counting passes of the frozen threshold

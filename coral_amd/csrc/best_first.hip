@@ -203,37 +203,11 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             }
         }
 
-        // The query in integer codes for the screening on eight-bit rows (see beam_search.hip): q~_i = sq (128 h_i +
-        // l_i), bytes h_i and l_i in LDS; |q~|^2, sq and |q - q~| (rounded up) in registers.
+        // The query in integer codes for the screening on eight-bit rows (search_device.h): bytes in LDS; |q~|^2, the
+        // scale and |q - q~| in registers.
         float c_qq = 0.0f, c_sq = 0.0f, c_eq = 0.0f;
         if constexpr (SCREEN == 2) {
-            const float* qv = a.queries + (size_t)qid * dim;
-            float amax = 0.0f;
-            bool bad = false;
-            for (int i = lane; i < dim; i += 64) {
-                const float v = fabsf(qv[i]);
-                bad |= !(v <= 3.0e38f);
-                amax = fmaxf(amax, v);
-            }
-            for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-            bad = __ballot(bad) != 0ull || (amax != 0.0f && !(amax >= 1.0e-18f && amax <= 1.0e17f));
-            const float sq = bad ? 0.0f : amax / 16256.0f;
-            double se = 0.0, sx = 0.0;
-            for (int i = lane; i < ((dim + 15) & ~15); i += 64) {
-                const float v = i < dim ? qv[i] : 0.0f;
-                int code = 0;
-                if (sq > 0.0f) {
-                    code = (int)rintf(v / sq);
-                    code = code > 16256 ? 16256 : (code < -16256 ? -16256 : code);
-                }
-                const int h = (code + 64) >> 7, l = code - 128 * h;
-                qh8[i] = (signed char)h, ql8[i] = (signed char)l;
-                const double qt = (double)sq * (double)code, dv = (double)v - qt;
-                se += dv * dv, sx += qt * qt;
-            }
-            for (int off = 32; off > 0; off >>= 1) se += __shfl_xor(se, off, 64), sx += __shfl_xor(sx, off, 64);
-            c_qq = (float)sx, c_sq = sq;
-            c_eq = bad ? __int_as_float(0x7f800000) : (float)(sqrt(se) * 1.000001) * (1.0f + 2.0e-7f);
+            code_query(a.queries + (size_t)qid * dim, dim, lane, qh8, ql8, c_qq, c_sq, c_eq);
             wave_sync();
         }
 
@@ -337,86 +311,33 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 T = n2;
             }
             if constexpr (SCREEN == 2 && G == 64 && CPL <= 2) {
-              if (nb == L) {
-                // the same on eight-bit codes: sixteen lanes per row, all 32 rows of a step in one round of requests
-                constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
-                const int gl8 = lane & 15, grp8 = lane >> 4;
-                const int nck = (dim + 15) >> 4;
-                const float s_live = key_s(live);
-                int qh[CPL8][4], ql[CPL8][4];
+                if (nb == L) {
+                    // the same on eight-bit codes: sixteen lanes per row, all 32 rows of a step in one round of requests
+                    constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
+                    const int gl8 = lane & 15, grp8 = lane >> 4;
+                    const int nck = (dim + 15) >> 4;
+                    const float s_live = key_s(live);
+                    CodedQuery<CPL8> cq;
+                    load_coded_query<CPL8>(qh8, ql8, nck, gl8, cq);
+                    int n2 = 0;
+                    for (int base = 0; base < T; base += RPI8) {
+                        int vid[U8];
+                        const int r0 = base + grp8 * U8;
 #pragma unroll
-                for (int t = 0; t < CPL8; ++t)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int c = gl8 + 16 * t;
-                        qh[t][j] = c < nck ? reinterpret_cast<const int*>(qh8)[4 * c + j] : 0;
-                        ql[t][j] = c < nck ? reinterpret_cast<const int*>(ql8)[4 * c + j] : 0;
+                        for (int u = 0; u < U8; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
+                        int myid;
+                        bool valid;
+                        float lo, hi;
+                        coded_rows_bounds<CPL8, U8>(b.vec8, b.stride8, nck, gl8, vid, cq, c_qq, c_sq, c_eq, myid, valid, lo, hi);
+                        const bool exact = valid && !(lo > s_live);
+                        const uint64_t m = __ballot(exact);
+                        if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;
+                        n2 += __popcll(m);
                     }
-                int n2 = 0;
-                for (int base = 0; base < T; base += RPI8) {
-                    int vid[U8];
-                    const int r0 = base + grp8 * U8;
-#pragma unroll
-                    for (int u = 0; u < U8; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
-                    uint4 hb[U8][CPL8];
-#pragma unroll
-                    for (int u = 0; u < U8; ++u) {
-                        const uint4* row = reinterpret_cast<const uint4*>(
-                            b.vec8 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * b.stride8);
-#pragma unroll
-                        for (int t = 0; t < CPL8; ++t) {
-                            const int c = gl8 + 16 * t;
-                            hb[u][t] = (vid[u] >= 0 && c < nck) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
-                        }
-                    }
-                    int myid = vid[0];
-#pragma unroll
-                    for (int u = 1; u < U8; ++u)
-                        if (gl8 == u) myid = vid[u];
-                    const bool valid = gl8 < U8 && myid >= 0;
-                    float4 fig = make_float4(0, 0, 0, 0);
-                    if (valid)
-                        fig = *reinterpret_cast<const float4*>(b.vec8 + (uint64_t)(uint32_t)myid * b.stride8 + (size_t)nck * 16);
-                    int acc[U8];
-#pragma unroll
-                    for (int u = 0; u < U8; ++u) {
-                        int dh = 0, dl = 0;
-#pragma unroll
-                        for (int t = 0; t < CPL8; ++t) {
-                            const int w[4] = {(int)hb[u][t].x, (int)hb[u][t].y, (int)hb[u][t].z, (int)hb[u][t].w};
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                dh = __builtin_amdgcn_sdot4(w[j], qh[t][j], dh, false);
-                                dl = __builtin_amdgcn_sdot4(w[j], ql[t][j], dl, false);
-                            }
-                        }
-                        acc[u] = 128 * dh + dl;
-                    }
-#pragma unroll
-                    for (int u = 0; u < U8; ++u) {
-                        acc[u] = acc[u] + dpp_mov_i<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
-                        acc[u] = acc[u] + dpp_mov_i<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
-                        acc[u] = acc[u] + dpp_mov_i<0x141>(acc[u]);  // row_half_mirror
-                        acc[u] = acc[u] + dpp_mov_i<0x140>(acc[u]);  // row_mirror
-                    }
-                    int mine = acc[0];
-#pragma unroll
-                    for (int u = 1; u < U8; ++u)
-                        if (gl8 == u) mine = acc[u];
-                    const float both = c_qq + fig.y;
-                    const float d8 = both - (2.0f * c_sq * fig.x) * (float)mine;
-                    const float delta = 16.0f * 5.9604645e-8f * both, e = fig.z + c_eq;
-                    const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
-                    const float lo = lo_root * lo_root * (1.0f - 1.0e-4f);
-                    const bool exact = valid && !(lo > s_live);
-                    const uint64_t m = __ballot(exact);
-                    if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;
-                    n2 += __popcll(m);
+                    wave_sync();
+                    list = todo2;
+                    T = n2;
                 }
-                wave_sync();
-                list = todo2;
-                T = n2;
-              }
             }
             int nc = 0;
             for (int base = 0; base < T; base += RPI) {

@@ -64,7 +64,9 @@ __device__ __forceinline__ void memory_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int G, int CPL, int RIF, bool PACKED>
+// SCREEN: once the queue is full, rows are first measured in the copy in eight-bit codes (b.vec8; rows of 132 .. 512
+// floats) and only those that may enter the queue are read in fp32 (search_device.h).
+template <int G, int CPL, int RIF, bool PACKED, bool SCREEN>
 __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_first_long_kernel(const SearchArgs a,
                                                                                                    const BestFirstLongArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
     const int L = a.L, R = a.R, dim = a.dim, chunks = dim >> 2, M = a.M;
     const int Lp = (L + 3) & ~3;
     const int bcap = b.bcap, tcap = b.bcap + kBatch, scap = b.scap, ss = b.sshift;
-    unsigned char* mine_lds = smem + (size_t)wave * best_first_long_lds_bytes(bcap, scap);
+    unsigned char* mine_lds = smem + (size_t)wave * best_first_long_lds_bytes(bcap, scap, b.coded_bytes);
     uint64_t* buf = reinterpret_cast<uint64_t*>(mine_lds);  // bcap keys, sorted: the insert buffer
     uint64_t* tail = buf + bcap;                             // tcap keys: the last keys of g as of the last merge
     uint64_t* samp0 = tail + tcap;                           // scap keys: every 2^ss-th key of g (two copies: the
@@ -82,6 +84,9 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
     uint64_t* cand = samp1 + scap;                           // kBatch keys
     uint32_t* todo = reinterpret_cast<uint32_t*>(cand + kBatch);  // kBatch ids
     uint32_t* marks = todo + kBatch;                         // bcap byte counters, zero between merges
+    uint32_t* todo2 = marks + (bcap >> 2);                   // (SCREEN) kBatch ids: what the screening leaves to measure
+    signed char* qh8 = reinterpret_cast<signed char*>(todo2 + kBatch);  // (SCREEN) the query in integer codes
+    signed char* ql8 = qh8 + ((dim + 15) & ~15);
     for (int i = lane; i < (bcap >> 2); i += 64) marks[i] = 0u;
 
     uint64_t* gbuf0 = b.beams + (size_t)slot * b.beam_stride;
@@ -131,6 +136,12 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                 const int c = gl + G * t;
                 qreg[t] = c < chunks ? q4[c] : make_float4(0, 0, 0, 0);
             }
+        }
+
+        float c_qq = 0.0f, c_sq = 0.0f, c_eq = 0.0f;
+        if constexpr (SCREEN) {
+            code_query(a.queries + (size_t)qid * dim, dim, lane, qh8, ql8, c_qq, c_sq, c_eq);
+            wave_sync();
         }
 
         // ---- the queue: g[0..ng) in global memory, buf[0..nbuf) in LDS, ng + nbuf <= L
@@ -206,12 +217,42 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
 
         // todo[0..T) -> distances -> the queue
         auto measure_and_merge = [&](int T) {
+            const uint32_t* list = todo;
+            if constexpr (SCREEN && G == 64 && CPL <= 2) {
+                if (live != kKeyMax) {
+                    // a row whose exact distance is certainly beyond the queue's worst entry is dropped on its codes
+                    constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
+                    const int gl8 = lane & 15, grp8 = lane >> 4;
+                    const int nck = (dim + 15) >> 4;
+                    const float s_live = key_s(live);
+                    CodedQuery<CPL8> cq;
+                    load_coded_query<CPL8>(qh8, ql8, nck, gl8, cq);
+                    int n2 = 0;
+                    for (int base = 0; base < T; base += RPI8) {
+                        int vid[U8];
+                        const int r0 = base + grp8 * U8;
+#pragma unroll
+                        for (int u = 0; u < U8; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
+                        int myid;
+                        bool valid;
+                        float lo, hi;
+                        coded_rows_bounds<CPL8, U8>(b.vec8, b.stride8, nck, gl8, vid, cq, c_qq, c_sq, c_eq, myid, valid, lo, hi);
+                        const bool exact = valid && !(lo > s_live);
+                        const uint64_t m = __ballot(exact);
+                        if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;
+                        n2 += __popcll(m);
+                    }
+                    wave_sync();
+                    list = todo2;
+                    T = n2;
+                }
+            }
             int nc = 0;
             for (int base = 0; base < T; base += RPI) {
                 int vid[U];
                 const int r0 = base + grp * U;
 #pragma unroll
-                for (int u = 0; u < U; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
+                for (int u = 0; u < U; ++u) vid[u] = r0 + u < T ? (int)list[r0 + u] : -1;
                 float4 v[U][CPL];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -460,31 +501,37 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
 
 using bfl_kernel_fn = void (*)(const SearchArgs, const BestFirstLongArgs);
 
-template <int RIF, bool PACKED>
+template <int RIF, bool PACKED, bool SCREEN>
 bfl_kernel_fn pick_rif(int chunks) {
-    if (chunks <= 16) return best_first_long_kernel<16, 1, RIF, PACKED>;
-    if (chunks <= 32) return best_first_long_kernel<32, 1, RIF, PACKED>;
-    if (chunks <= 64) return best_first_long_kernel<64, 1, RIF, PACKED>;
-    if (chunks <= 128) return best_first_long_kernel<64, 2, RIF, PACKED>;
-    if (chunks <= 256) return best_first_long_kernel<64, 4, RIF, PACKED>;
-    if (chunks <= 512) return best_first_long_kernel<64, 8, RIF, PACKED>;
+    if (chunks <= 16) return best_first_long_kernel<16, 1, RIF, PACKED, false>;
+    if (chunks <= 32) return best_first_long_kernel<32, 1, RIF, PACKED, false>;
+    if (chunks <= 64) return best_first_long_kernel<64, 1, RIF, PACKED, SCREEN>;
+    if (chunks <= 128) return best_first_long_kernel<64, 2, RIF, PACKED, SCREEN>;
+    if (chunks <= 256) return best_first_long_kernel<64, 4, RIF, PACKED, false>;
+    if (chunks <= 512) return best_first_long_kernel<64, 8, RIF, PACKED, false>;
     return nullptr;
 }
 
-bfl_kernel_fn pick(int dim, bool packed) {
+template <bool SCREEN>
+bfl_kernel_fn pick_screen(int dim, bool packed) {
     const int chunks = dim / 4;
     // 16 rows requested per wavefront before any is added up where that fits 128 registers, else 8
     const bool wide = chunks > 16 && chunks <= 256;
-    if (packed) return wide ? pick_rif<16, true>(chunks) : pick_rif<8, true>(chunks);
-    return wide ? pick_rif<16, false>(chunks) : pick_rif<8, false>(chunks);
+    if (packed) return wide ? pick_rif<16, true, SCREEN>(chunks) : pick_rif<8, true, SCREEN>(chunks);
+    return wide ? pick_rif<16, false, SCREEN>(chunks) : pick_rif<8, false, SCREEN>(chunks);
+}
+
+bfl_kernel_fn pick(int dim, bool packed, bool screen) {
+    return screen ? pick_screen<true>(dim, packed) : pick_screen<false>(dim, packed);
 }
 
 }  // namespace
 
-hipError_t best_first_long_prepare(int dim, bool packed, int bcap, int scap, int* max_wg_per_cu) {
-    bfl_kernel_fn fn = pick(dim, packed);
+hipError_t best_first_long_prepare(int dim, bool packed, bool screen, int bcap, int scap, int* max_wg_per_cu) {
+    if (screen && (dim > kMaxByteRowDim || dim / 4 <= 32)) return hipErrorInvalidValue;
+    bfl_kernel_fn fn = pick(dim, packed, screen);
     if (!fn) return hipErrorInvalidValue;
-    const size_t lds = best_first_long_lds_bytes(bcap, scap) * kWavesPerWg;
+    const size_t lds = best_first_long_lds_bytes(bcap, scap, screen ? best_first_long_coded_bytes(dim) : 0) * kWavesPerWg;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -496,11 +543,14 @@ hipError_t best_first_long_prepare(int dim, bool packed, int bcap, int scap, int
 }
 
 hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& b, hipStream_t stream) {
-    bfl_kernel_fn fn = pick(a.dim, b.packed != 0);
+    const bool screen = b.vec8 != nullptr;
+    if (screen && (a.dim > kMaxByteRowDim || a.dim / 4 <= 32 || b.coded_bytes != best_first_long_coded_bytes(a.dim)))
+        return hipErrorInvalidValue;
+    bfl_kernel_fn fn = pick(a.dim, b.packed != 0, screen);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
-    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), best_first_long_lds_bytes(b.bcap, b.scap) * kWavesPerWg,
-                       stream, a, b);
+    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64),
+                       best_first_long_lds_bytes(b.bcap, b.scap, b.coded_bytes) * kWavesPerWg, stream, a, b);
     return hipGetLastError();
 }
 

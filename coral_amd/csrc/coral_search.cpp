@@ -493,6 +493,20 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // without the LDS table: L > 409): +12 % at L = 512 and 1024.  With the table (eight wavefronts per CU) the extra
     // wait per step costs more than the bytes it spares (L = 256 / 320: -27 %), so those launches go without unless
     // the caller asks for it by name.
+    if (long_form && idx->metric == CORAL_L2 && idx->dim / 4 > 32 && idx->dim <= coral::kMaxByteRowDim &&
+        (t.screening == 2 || (t.screening == 0 && L <= 8192))) {
+        // the kernel of long beams screens on eight-bit codes only, and by itself only up to L = 8192: the longer
+        // the queue, the larger the share of rows that enter it and need their fp32 row after all (measured at a
+        // million nodes: +8 % at L = 1536, +2 % at 4096, nothing at 8192, -5 % at 19 456)
+        const hipError_t e = ensure_vec8();
+        if (e == hipSuccess) {
+            idx->bf_screen = 2;
+        } else if (e == hipErrorOutOfMemory && t.screening == 0) {
+            (void)hipGetLastError();
+        } else {
+            HIP_TRY(e);
+        }
+    }
     if (wave_form && idx->metric == CORAL_L2 && idx->dim / 4 > 32 &&
         (t.screening > 0 || (t.screening == 0 && table_log2 == 0))) {
         // eight-bit codes where they apply; launches with the LDS table (whose size was chosen to fill LDS) and rows of
@@ -575,11 +589,13 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         const int scap = 128;
         int sshift = 0;
         while ((((int64_t)L - 1) >> sshift) + 1 > scap) ++sshift;
-        if (coral::best_first_long_lds_bytes(bcap, scap) * 4 > (size_t)kMaxLdsBytes)
+        const bool screen = idx->bf_screen == 2;
+        if (coral::best_first_long_lds_bytes(bcap, scap, screen ? coral::best_first_long_coded_bytes(idx->dim) : 0) * 4 >
+            (size_t)kMaxLdsBytes)
             return fail(CORAL_ERR_ARG, "best_first_buffer = %d does not fit LDS", bcap);
         int bf_wg_per_cu = 0;
-        HIP_TRY(coral::best_first_long_prepare(idx->dim, false, bcap, scap, &bf_wg_per_cu));
-        auto reprepare = [&](int* occ) { return coral::best_first_long_prepare(idx->dim, true, bcap, scap, occ); };
+        HIP_TRY(coral::best_first_long_prepare(idx->dim, false, screen, bcap, scap, &bf_wg_per_cu));
+        auto reprepare = [&](int* occ) { return coral::best_first_long_prepare(idx->dim, true, screen, bcap, scap, occ); };
         const size_t Lp = (size_t)((L + 3) & ~3);
         const size_t beam_stride = (2 * Lp + 15) & ~(size_t)15;  // two runs of Lp keys, a multiple of 128 bytes
         if (int rc = visited_slots(bf_wg_per_cu, reprepare, (int64_t)beam_stride * 8)) return rc;
@@ -682,6 +698,8 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         b.slots = std::min(idx->bf_slots, (int)Q);
         b.rows_unique = idx->rows_unique == 1, b.packed = idx->bf_packed;
         b.bcap = idx->bf_bcap, b.scap = idx->bf_scap, b.sshift = idx->bf_sshift;
+        b.vec8 = idx->bf_screen == 2 ? idx->d_vec8 : nullptr, b.stride8 = coral::byte_row_stride(idx->dim);
+        b.coded_bytes = idx->bf_screen == 2 ? coral::best_first_long_coded_bytes(idx->dim) : 0;
         HIP_TRY(coral::launch_best_first_long(a, b, stream));
     } else if (wave_kernel) {
         coral::BestFirstArgs b;

@@ -35,6 +35,124 @@ __device__ __forceinline__ int dpp_mov_i(int x) {
     return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, true);
 }
 
+// ---- Screening on rows in eight-bit codes (the copy byte_rows_kernel makes).  Row x is stored as codes k_i in
+// [-127, 127] with x~_i = s k_i, s = max |x_i| / 127, followed by s, |x~|^2 and e >= |x - x~| (rounded up; infinite for
+// rows that take no part).  The query is coded as q~_i = sq (128 h_i + l_i), bytes h_i in [-127, 127] and l_i in
+// [-64, 63], sq = max |q_i| / 16256, with eq >= |q - q~|.  D = |q~ - x~|^2 = |q~|^2 + |x~|^2 - 2 sq s sum (128 h_i + l_i) k_i
+// needs integer dot products only (v_dot4_i32_i8, exact), and the exact distance d = |q - x|^2 satisfies
+// (sqrt(D) - e - eq)^2 <= d <= (sqrt(D) + e + eq)^2.  The computed D is within delta = 16 * 2^-24 (|q~|^2 + |x~|^2) of its
+// true value (the conversion of the integer sum, the product of the scales, the two stored norms and the two final
+// additions: each relative 2^-24 of a quantity no larger than |q~|^2 + |x~|^2; taken twice); both ends are widened by
+// 1e-4 for the fp32 rounding of the exact distance that the bounds are compared with.
+
+// The query in integer codes, by one whole wavefront: bytes h_i to qh8, l_i to ql8 (zero up to a multiple of 16
+// dimensions); qq = |q~|^2, sq, eq (sums in double precision, eq rounded up).  A query with a component that is not
+// finite, or whose largest lies outside [1e-18, 1e17], gets eq = inf: every row then goes to the exact pass.
+__device__ __forceinline__ void code_query(const float* q, int dim, int lane, signed char* qh8, signed char* ql8,
+                                           float& qq, float& sq, float& eq) {
+    float amax = 0.0f;
+    bool bad = false;
+    for (int i = lane; i < dim; i += 64) {
+        const float v = fabsf(q[i]);
+        bad |= !(v <= 3.0e38f);
+        amax = fmaxf(amax, v);
+    }
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    bad = __ballot(bad) != 0ull || (amax != 0.0f && !(amax >= 1.0e-18f && amax <= 1.0e17f));
+    sq = bad ? 0.0f : amax / 16256.0f;
+    double se = 0.0, sx = 0.0;
+    for (int i = lane; i < ((dim + 15) & ~15); i += 64) {
+        const float v = i < dim ? q[i] : 0.0f;
+        int code = 0;
+        if (sq > 0.0f) {
+            code = (int)rintf(v / sq);
+            code = code > 16256 ? 16256 : (code < -16256 ? -16256 : code);
+        }
+        const int h = (code + 64) >> 7, l = code - 128 * h;
+        qh8[i] = (signed char)h, ql8[i] = (signed char)l;
+        const double qt = (double)sq * (double)code, dv = (double)v - qt;
+        se += dv * dv, sx += qt * qt;
+    }
+    for (int off = 32; off > 0; off >>= 1) se += __shfl_xor(se, off, 64), sx += __shfl_xor(sx, off, 64);
+    qq = (float)sx;
+    eq = bad ? __int_as_float(0x7f800000) : (float)(sqrt(se) * 1.000001) * (1.0f + 2.0e-7f);
+}
+
+// the coded query of the lane: sixteen lanes share a row, lane gl8 of them takes the 16-byte chunks gl8 + 16 t
+template <int CPL8>
+struct CodedQuery {
+    int h[CPL8][4], l[CPL8][4];
+};
+template <int CPL8>
+__device__ __forceinline__ void load_coded_query(const signed char* qh8, const signed char* ql8, int nck, int gl8,
+                                                 CodedQuery<CPL8>& q) {
+#pragma unroll
+    for (int t = 0; t < CPL8; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = gl8 + 16 * t;
+            q.h[t][j] = c < nck ? reinterpret_cast<const int*>(qh8)[4 * c + j] : 0;
+            q.l[t][j] = c < nck ? reinterpret_cast<const int*>(ql8)[4 * c + j] : 0;
+        }
+}
+
+// Rows vid[0..U8) (-1: none) of one group of sixteen lanes, all requested before any is added up.  Lane gl8 < U8 of the
+// group files row vid[gl8]: myid, valid, and the bounds lo <= d <= hi of its exact distance (lo = 0 and hi = inf for a
+// row that takes no part; a NaN anywhere fails every comparison a caller makes with them).
+template <int CPL8, int U8>
+__device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, size_t stride8, int nck, int gl8,
+                                                  const int (&vid)[U8], const CodedQuery<CPL8>& q, float qq, float sq,
+                                                  float eq, int& myid, bool& valid, float& lo, float& hi) {
+    uint4 hb[U8][CPL8];
+#pragma unroll
+    for (int u = 0; u < U8; ++u) {
+        const uint4* row = reinterpret_cast<const uint4*>(vec8 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * stride8);
+#pragma unroll
+        for (int t = 0; t < CPL8; ++t) {
+            const int c = gl8 + 16 * t;
+            hb[u][t] = (vid[u] >= 0 && c < nck) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+    myid = vid[0];
+#pragma unroll
+    for (int u = 1; u < U8; ++u)
+        if (gl8 == u) myid = vid[u];
+    valid = gl8 < U8 && myid >= 0;
+    float4 fig = make_float4(0, 0, 0, 0);  // s, |x~|^2, e
+    if (valid) fig = *reinterpret_cast<const float4*>(vec8 + (uint64_t)(uint32_t)myid * stride8 + (size_t)nck * 16);
+    int acc[U8];
+#pragma unroll
+    for (int u = 0; u < U8; ++u) {
+        int dh = 0, dl = 0;
+#pragma unroll
+        for (int t = 0; t < CPL8; ++t) {
+            const int w[4] = {(int)hb[u][t].x, (int)hb[u][t].y, (int)hb[u][t].z, (int)hb[u][t].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                dh = __builtin_amdgcn_sdot4(w[j], q.h[t][j], dh, false);
+                dl = __builtin_amdgcn_sdot4(w[j], q.l[t][j], dl, false);
+            }
+        }
+        acc[u] = 128 * dh + dl;  // below 2^31 for 512 dimensions: 512 * 127 * 16256
+    }
+#pragma unroll
+    for (int u = 0; u < U8; ++u) {
+        acc[u] = acc[u] + dpp_mov_i<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
+        acc[u] = acc[u] + dpp_mov_i<0x4E>(acc[u]);   // quad_perm [2,3,0,1]
+        acc[u] = acc[u] + dpp_mov_i<0x141>(acc[u]);  // row_half_mirror
+        acc[u] = acc[u] + dpp_mov_i<0x140>(acc[u]);  // row_mirror
+    }
+    int mine = acc[0];
+#pragma unroll
+    for (int u = 1; u < U8; ++u)
+        if (gl8 == u) mine = acc[u];
+    const float both = qq + fig.y;
+    const float d8 = both - (2.0f * sq * fig.x) * (float)mine, delta = 16.0f * 5.9604645e-8f * both, e = fig.z + eq;
+    const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
+    const float hi_root = sqrtf(fmaxf(d8 + delta, 0.0f)) + e;
+    lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
+}
+
 // number of set bits of m below the calling lane
 __device__ __forceinline__ int prefix_popc(uint64_t m) {
     const uint32_t lane = threadIdx.x & 63;

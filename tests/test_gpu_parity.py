@@ -225,7 +225,9 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
     for form in (dict(screening=-1), dict(screening=1), dict(screening=1, best_first_table_log2=-1),
                  dict(screening=1, best_first_packed=True), dict(screening=2), dict(screening=2, best_first_table_log2=-1),
-                 dict(screening=2, best_first_packed=True, best_first_table_log2=-1), dict(best_first_table_log2=-1)):
+                 dict(screening=2, best_first_packed=True, best_first_table_log2=-1), dict(best_first_table_log2=-1),
+                 dict(best_first_long=1), dict(best_first_long=1, screening=-1),
+                 dict(best_first_long=1, best_first_buffer=64, best_first_packed=True, screening=2)):
         idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, **form)
         ids, dists, _ = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)
         assert np.array_equal(ids, oi), form
