@@ -36,14 +36,16 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* __restric
     if (acc == 0x9E3779B9u) *sink = acc;  // keeps the loads alive; the buffer holds no such pattern
 }
 
-// one group of 64 lanes per row (a wavefront), 16 bytes per lane and step; rows chosen by a hash of the row counter
+// A group of LPG lanes per row (16, 32 or 64: the smallest that covers the row with 16 bytes per lane, as the search
+// kernels read their rows), eight rows in flight per group; rows chosen by a hash of the row counter
+template <int LPG>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint4* __restrict__ p, size_t rows_in_buffer,
                                                           int row16, size_t rows_to_read, uint32_t seed, uint32_t* sink) {
-    const int lane = threadIdx.x & 63;
-    const size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    const int lig = threadIdx.x % LPG;
+    const size_t grp = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) / LPG;
+    const size_t ngrp = ((size_t)gridDim.x * blockDim.x) / LPG;
     uint32_t acc = 0;
-    for (size_t r = wave * 8; r < rows_to_read; r += nwaves * 8) {
+    for (size_t r = grp * 8; r < rows_to_read; r += ngrp * 8) {
         uint4 v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -52,7 +54,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint4* __restric
             h *= 0xBF58476D1CE4E5B9ull;
             h ^= h >> 32;
             const size_t row = (size_t)(h % rows_in_buffer);
-            v[u] = lane < row16 ? p[row * row16 + lane] : make_uint4(0, 0, 0, 0);
+            v[u] = lig < row16 ? p[row * row16 + lig] : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
@@ -102,8 +104,14 @@ extern "C" int coral_membench(int32_t device, size_t bytes, int32_t row_bytes, i
                 MB_TRY(hipEventRecord(e0, 0));
                 if (which == 0)
                     hipLaunchKernelGGL(stream_read_kernel, dim3(grid), dim3(256), 0, 0, (const u32x4*)buf, n16, sink);
+                else if (row16 <= 16)
+                    hipLaunchKernelGGL(gather_rows_kernel<16>, dim3(grid), dim3(256), 0, 0, (const uint4*)buf, rows_in_buffer,
+                                       row16, rows_to_read, (uint32_t)r * 7919u, sink);
+                else if (row16 <= 32)
+                    hipLaunchKernelGGL(gather_rows_kernel<32>, dim3(grid), dim3(256), 0, 0, (const uint4*)buf, rows_in_buffer,
+                                       row16, rows_to_read, (uint32_t)r * 7919u, sink);
                 else
-                    hipLaunchKernelGGL(gather_rows_kernel, dim3(grid), dim3(256), 0, 0, (const uint4*)buf, rows_in_buffer,
+                    hipLaunchKernelGGL(gather_rows_kernel<64>, dim3(grid), dim3(256), 0, 0, (const uint4*)buf, rows_in_buffer,
                                        row16, rows_to_read, (uint32_t)r * 7919u, sink);
                 MB_TRY(hipGetLastError());
                 MB_TRY(hipEventRecord(e1, 0));
