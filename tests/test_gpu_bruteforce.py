@@ -193,6 +193,37 @@ def test_bruteforce_rows_with_thousands_of_ties_and_large_k(orc):
     idx.close(), idx2.close()
 
 
+def test_bruteforce_candidate_lists_that_overflow_go_through_the_matrix(orc):
+    """The selection inside the matrix-core kernel keeps what does not exceed a bound taken from a sample of the base.
+    Where that is more than a list holds -- most of the base at one and the same distance, or a sample that is
+    tombstoned away so that no bound exists -- the call falls back to the distance matrix, with the same result."""
+    n, dim, k = 20000, 16, 10
+    rng = np.random.RandomState(5)
+    q = synth.gaussian_matrix(8, 7, dim)
+    # (a) all but 50 rows are the same vector: every one of them ties at the bound
+    base = np.ones((n, dim), np.float32)
+    base[rng.choice(n, 50, replace=False)] = synth.gaussian_matrix(9, 50, dim)
+    idx = capi.Index(base, None, None)
+    ids, dists, _ = idx.bruteforce(q, k)
+    assert idx.bruteforce_last_fused() == 0
+    oi, od = orc.bruteforce(base, q, k, order=SEQ)
+    assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+    idx.close()
+    # (b) everything but the last 300 ids is tombstoned: the sample holds fewer live points than candidates are kept
+    base = synth.gaussian_matrix(10, n, dim)
+    mask = np.zeros((n + 31) // 32, np.uint32)
+    dead = np.arange(n - 300)
+    np.bitwise_or.at(mask, dead >> 5, (np.uint32(1) << (dead & 31).astype(np.uint32)))
+    idx = capi.Index(base, None, None)
+    idx.set_deleted(mask)
+    ids, dists, _ = idx.bruteforce(q, k, have_delete=True)
+    assert idx.bruteforce_last_fused() == 0
+    oi, od = orc.bruteforce(base, q, k, deleted=mask, order=SEQ)
+    assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
+    assert (ids >= n - 300).all()
+    idx.close()
+
+
 def test_bruteforce_segments(orc):
     # more base points than one pass holds (4M): per-segment winners are merged
     n, dim, Q, k = 5 * 1000 * 1000, 8, 40, 50
