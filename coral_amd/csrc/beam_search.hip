@@ -352,7 +352,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     int myid;
                     bool valid;
                     float lo, hi;
-                    coded_rows_bounds<CPL8, U8>(a.vec8, a.stride8, nck, gl8, vid, cq, qq, sq, eq, myid, valid, lo, hi);
+                    coded_rows_bounds<CPL8, U8>(a.vec8, a.stride8, nck, gl8, vid, cq, qq, sq, eq, a.metric, myid, valid, lo, hi);
                     const bool gone = valid && lo > thr;
                     const bool counted = valid && !gone && hi < thr && lo > s_live;
                     const bool exact = valid && !gone && !counted;

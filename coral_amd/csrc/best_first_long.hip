@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                         int myid;
                         bool valid;
                         float lo, hi;
-                        coded_rows_bounds<CPL8, U8>(b.vec8, b.stride8, nck, gl8, vid, cq, c_qq, c_sq, c_eq, myid, valid, lo, hi);
+                        coded_rows_bounds<CPL8, U8>(b.vec8, b.stride8, nck, gl8, vid, cq, c_qq, c_sq, c_eq, a.metric, myid, valid, lo, hi);
                         const bool exact = valid && !(lo > s_live);
                         const uint64_t m = __ballot(exact);
                         if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;

@@ -278,14 +278,16 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     // ---- screening on a smaller copy of the vectors (rounds policy, L2, rows of 132 .. 2048 floats): eight-bit codes
     // (tuning 2; the library's choice up to 512 floats) or half precision (tuning 1); see beam_search.hip
     // (best-first: the wavefront-per-query kernel with the beam in LDS screens too, see coral_search_prepare)
-    const bool screen_possible = !best_first && idx->metric == CORAL_L2 && idx->dim / 4 > 32;
+    const bool codes_possible = idx->dim <= coral::kMaxByteRowDim;  // the inner product is screened on codes only
+    const bool screen_possible = !best_first && idx->dim / 4 > 32 && (idx->metric == CORAL_L2 || codes_possible);
     if (t.screening > 2 || t.screening < -1) return fail(CORAL_ERR_ARG, "screening must be -1, 0, 1 or 2 (got %d)", t.screening);
-    if (t.screening > 0 && !(idx->metric == CORAL_L2 && idx->dim / 4 > 32))
-        return fail(CORAL_ERR_ARG, "screening needs the L2 metric and more than 128 dimensions");
-    if (t.screening == 2 && idx->dim > coral::kMaxByteRowDim)
+    if (t.screening > 0 && idx->dim / 4 <= 32) return fail(CORAL_ERR_ARG, "screening needs more than 128 dimensions");
+    if (t.screening == 1 && idx->metric != CORAL_L2)
+        return fail(CORAL_ERR_ARG, "screening in half precision needs the L2 metric");
+    if (t.screening == 2 && !codes_possible)
         return fail(CORAL_ERR_ARG, "screening on eight-bit codes takes rows of up to %d floats", coral::kMaxByteRowDim);
     const bool screen = screen_possible && (t.screening > 0 || (t.screening == 0 && !no_screen));
-    p.screen = !screen ? 0 : t.screening > 0 ? t.screening : (idx->dim <= coral::kMaxByteRowDim ? 2 : 1);
+    p.screen = !screen ? 0 : t.screening > 0 ? t.screening : (codes_possible ? 2 : 1);
     // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
     // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
     // -1, or the library's choice): one LDS atomic per test and nothing ever overflows, at n / 8 bytes -- 125 KB for
@@ -493,7 +495,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // without the LDS table: L > 409): +12 % at L = 512 and 1024.  With the table (eight wavefronts per CU) the extra
     // wait per step costs more than the bytes it spares (L = 256 / 320: -27 %), so those launches go without unless
     // the caller asks for it by name.
-    if (long_form && idx->metric == CORAL_L2 && idx->dim / 4 > 32 && idx->dim <= coral::kMaxByteRowDim &&
+    if (long_form && idx->dim / 4 > 32 && idx->dim <= coral::kMaxByteRowDim &&
         (t.screening == 2 || (t.screening == 0 && L <= 8192))) {
         // the kernel of long beams screens on eight-bit codes only, and by itself only up to L = 8192: the longer
         // the queue, the larger the share of rows that enter it and need their fp32 row after all (measured at a
@@ -507,11 +509,11 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
             HIP_TRY(e);
         }
     }
-    if (wave_form && idx->metric == CORAL_L2 && idx->dim / 4 > 32 &&
+    // eight-bit codes where they apply; launches with the LDS table (whose size was chosen to fill LDS) and rows of
+    // more than 512 floats screen in half precision, which only the L2 metric has
+    const int form = t.screening == 1 || idx->dim > coral::kMaxByteRowDim || table_log2 != 0 ? 1 : 2;
+    if (wave_form && idx->dim / 4 > 32 && (form == 2 || idx->metric == CORAL_L2) &&
         (t.screening > 0 || (t.screening == 0 && table_log2 == 0))) {
-        // eight-bit codes where they apply; launches with the LDS table (whose size was chosen to fill LDS) and rows of
-        // more than 512 floats screen in half precision
-        const int form = t.screening == 1 || idx->dim > coral::kMaxByteRowDim || table_log2 != 0 ? 1 : 2;
         const hipError_t e = form == 2 ? ensure_vec8() : ensure_vec16();
         if (e == hipSuccess) {
             idx->bf_screen = form;

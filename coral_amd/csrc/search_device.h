@@ -99,10 +99,14 @@ __device__ __forceinline__ void load_coded_query(const signed char* qh8, const s
 // Rows vid[0..U8) (-1: none) of one group of sixteen lanes, all requested before any is added up.  Lane gl8 < U8 of the
 // group files row vid[gl8]: myid, valid, and the bounds lo <= d <= hi of its exact distance (lo = 0 and hi = inf for a
 // row that takes no part; a NaN anywhere fails every comparison a caller makes with them).
+//
+// Inner product (metric 1; the signed distance is -q.x): q.x = q~.x~ + q~.(x - x~) + (q - q~).x, so
+// |q.x - q~.x~| <= |q~| e + eq (|x~| + e); the bound is widened by 2e-4 (|q~| + eq)(|x~| + e) for the fp32 rounding of
+// the exact inner product and of the computed q~.x~ (each at most dim 2^-24 |q| |x|, dim <= 512).
 template <int CPL8, int U8>
 __device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, size_t stride8, int nck, int gl8,
                                                   const int (&vid)[U8], const CodedQuery<CPL8>& q, float qq, float sq,
-                                                  float eq, int& myid, bool& valid, float& lo, float& hi) {
+                                                  float eq, int metric, int& myid, bool& valid, float& lo, float& hi) {
     uint4 hb[U8][CPL8];
 #pragma unroll
     for (int u = 0; u < U8; ++u) {
@@ -146,11 +150,18 @@ __device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, siz
 #pragma unroll
     for (int u = 1; u < U8; ++u)
         if (gl8 == u) mine = acc[u];
-    const float both = qq + fig.y;
-    const float d8 = both - (2.0f * sq * fig.x) * (float)mine, delta = 16.0f * 5.9604645e-8f * both, e = fig.z + eq;
-    const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
-    const float hi_root = sqrtf(fmaxf(d8 + delta, 0.0f)) + e;
-    lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
+    if (metric == 0) {
+        const float both = qq + fig.y;
+        const float d8 = both - (2.0f * sq * fig.x) * (float)mine, delta = 16.0f * 5.9604645e-8f * both, e = fig.z + eq;
+        const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
+        const float hi_root = sqrtf(fmaxf(d8 + delta, 0.0f)) + e;
+        lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
+    } else {
+        const float p = (sq * fig.x) * (float)mine;  // q~.x~
+        const float nq = sqrtf(qq) * (1.0f + 1.0e-6f), nx = sqrtf(fig.y) * (1.0f + 1.0e-6f), e = fig.z;
+        const float bound = (nq * e + eq * (nx + e) + 2.0e-4f * (nq + eq) * (nx + e)) * (1.0f + 1.0e-5f);
+        lo = (0.0f - p) - bound, hi = (0.0f - p) + bound;  // e = inf or eq = inf: lo = -inf, hi = inf (or NaN)
+    }
 }
 
 // number of set bits of m below the calling lane

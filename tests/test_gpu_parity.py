@@ -92,9 +92,11 @@ def test_exact_against_same_order_oracle(orc, case):
              dict(best_first_packed=True, best_first_table_log2=8), dict(best_first_table_log2=9),
              dict(best_first_long=1), dict(best_first_long=1, best_first_buffer=64, best_first_packed=True),
              dict(best_first_long=1, best_first_buffer=192)) if policy == 1 else (dict(),)
-    if policy == 0 and metric == "l2" and dim > 128:
+    if policy == 0 and dim > 128:
         # the rounds policy without, and with either form of, its screening of the rows on a smaller copy
-        forms = (dict(screening=-1), dict(screening=1), dict(screening=1, beam_in_hbm=True))
+        forms = (dict(screening=-1),)
+        if metric == "l2":
+            forms += (dict(screening=1), dict(screening=1, beam_in_hbm=True))
         if dim <= 512:  # what the copy in eight-bit codes takes
             forms += (dict(screening=2), dict(screening=2, beam_in_hbm=True))
     for form in forms:
@@ -176,7 +178,8 @@ def test_beams_in_global_memory_equal_the_oracle(orc, case):
 
 
 @pytest.mark.parametrize("kind", ["lattice", "large", "beyond_half", "tiny", "dim_not_a_multiple_of_8", "dim_200",
-                                  "dim_264", "mixed_magnitudes", "outliers", "tiny_queries", "huge_rows"])
+                                  "dim_264", "mixed_magnitudes", "outliers", "tiny_queries", "huge_rows", "ip_unit",
+                                  "ip_raw", "ip_lattice", "ip_mixed_magnitudes"])
 def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     """The rounds kernel measures every row in a smaller copy of the vectors first -- half precision, or eight-bit
     codes with a scale per row -- and reads the fp32 row only where bounds on the exact distance leave the row's fate
@@ -186,12 +189,15 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     pass), components of 1e-6 (halves underflow to zero and subnormals), dimensions whose last 16-byte chunk is part
     padding (140: halves; 200 and 264: codes, the latter with two chunks per lane), rows of very different magnitudes
     in one base (a scale per row), rows with one component a hundred times the others (codes lose the rest), queries
-    of 1e-20 (no scale: every row goes to the exact pass), rows of 1e18 (they take no part in the coded copy).  Ids,
-    distance bits and counters equal the oracle's, with the screening and without."""
+    of 1e-20 (no scale: every row goes to the exact pass), rows of 1e18 (they take no part in the coded copy); and the
+    inner-product metric, which is screened on codes only: unit vectors, raw Gaussian rows, a lattice, rows of very
+    different norms.  Ids, distance bits and counters equal the oracle's, with the screening and without."""
     n, dim, R, Q, L, k = 4000, 136, 24, 100, 200, 50
-    dim = {"dim_not_a_multiple_of_8": 140, "dim_200": 200, "dim_264": 264}.get(kind, dim)
+    dim = {"dim_not_a_multiple_of_8": 140, "dim_200": 200, "dim_264": 264, "ip_raw": 200}.get(kind, dim)
+    ip = kind.startswith("ip_")
+    m, mname = (capi.IP, "ip") if ip else (capi.L2, "l2")
     rng = np.random.RandomState(77)
-    if kind == "lattice":
+    if kind in ("lattice", "ip_lattice"):
         base = rng.randint(0, 4, (n, dim)).astype(np.float32)
         q = (rng.randint(0, 8, (Q, dim)) * 0.5).astype(np.float32)
     else:
@@ -200,34 +206,42 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
         q = (make_queries(Q, dim, 89) * np.float32(scale)).astype(np.float32)
         if kind == "beyond_half":
             base[::7] *= np.float32(1e-3)  # a share of the rows fits the format, the rest does not
-        if kind == "mixed_magnitudes":
+        if kind in ("mixed_magnitudes", "ip_mixed_magnitudes"):
             base *= (10.0 ** rng.randint(-3, 4, (n, 1))).astype(np.float32)
+        if kind == "ip_unit":
+            base, q = synth.normalize_rows(base), synth.normalize_rows(q)
         if kind == "outliers":
             base[np.arange(n), rng.randint(0, dim, n)] *= np.float32(100.0)
         if kind == "tiny_queries":
             q[::2] *= np.float32(1e-20)
         if kind == "huge_rows":
             base[::5] *= np.float32(1e18)
-    nbrs = ragged(gpu_graph(base, R), 5, keep_min=3)
+    nbrs = ragged(gpu_graph(base, R, mname), 5, keep_min=3)
     starts = rng.choice(n, 8, replace=False).astype(np.int32)
     prob = orc.Problem(base, nbrs, starts)
-    oi, od, os_, _ = orc.search_B(prob, q, k, L, start_order=WAVE64, nbr_order=WAVE64)
-    idx = capi.Index(base, nbrs, starts)
+    oi, od, os_, _ = orc.search_B(prob, q, k, L, metric=m, start_order=WAVE64, nbr_order=WAVE64)
+    idx = capi.Index(base, nbrs, starts, m)
     for form in (dict(screening=-1), dict(screening=1), dict(screening=1, beam_in_hbm=True),
                  dict(screening=1, visited_slots_log2=12, threads=256), dict(screening=2),
                  dict(screening=2, beam_in_hbm=True), dict(screening=2, visited_slots_log2=12, threads=256), dict()):
+        if ip and form.get("screening") == 1:  # half precision screens the L2 metric only
+            with pytest.raises(capi.CoralError):
+                idx.prepare(Q, L, **form)
+            continue
         idx.prepare(Q, L, **form)
         ids, dists, _ = idx.search(q, k, L)
         assert np.array_equal(ids, oi), form
         assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), form
         assert np.array_equal(idx.query_counters(Q), os_), form
     # best-first on the wavefront-per-query kernel screens against the beam's worst entry
-    oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
+    oi, od, os_, _ = orc.search_A(prob, q, k, L, metric=m, order=WAVE64)
     for form in (dict(screening=-1), dict(screening=1), dict(screening=1, best_first_table_log2=-1),
                  dict(screening=1, best_first_packed=True), dict(screening=2), dict(screening=2, best_first_table_log2=-1),
                  dict(screening=2, best_first_packed=True, best_first_table_log2=-1), dict(best_first_table_log2=-1),
                  dict(best_first_long=1), dict(best_first_long=1, screening=-1),
                  dict(best_first_long=1, best_first_buffer=64, best_first_packed=True, screening=2)):
+        if ip and form.get("screening") == 1:
+            continue
         idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, **form)
         ids, dists, _ = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)
         assert np.array_equal(ids, oi), form
@@ -235,7 +249,7 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
         assert np.array_equal(idx.query_counters(Q), os_), form
     idx.close()
     # where it does not apply it is refused when asked for by name, and left out otherwise
-    small = capi.Index(base[:, :64].copy(), nbrs, starts)
+    small = capi.Index(base[:, :64].copy(), nbrs, starts, m)
     for named in (1, 2):
         with pytest.raises(capi.CoralError):
             small.prepare(Q, L, screening=named)
@@ -314,9 +328,11 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         if rng.rand() < 0.2:
             slots = -1  # the visited set as a bitmap of all ids in LDS
         ahead = int(rng.choice([0, 1, -1]))  # graph rows requested a chunk ahead: the library's choice, yes, no
-        screen = int(rng.choice([0, 1, 2, -1])) if (policy == 0 and metric == "l2" and dim > 128) else 0
+        screen = int(rng.choice([0, 1, 2, -1])) if (policy == 0 and dim > 128) else 0
         if screen == 2 and dim > 512:
             screen = 1
+        if screen == 1 and metric != "l2":
+            screen = 2 if dim <= 512 else -1
         print("case", dict(c=c, n=n, dim=dim, R=R, metric=metric, policy=policy, L=L, k=k, M=M, Q=Q, slots=slots,
                            threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl, big=big, ahead=ahead,
                            screen=screen),
