@@ -332,7 +332,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         // classes from a quarter of the bytes.  Sixteen lanes per row (a 256-byte row at dim 200: two cache lines),
         // eight rows in flight per group, four groups per wavefront.
         auto screening_phase8 = [&](int T) {
-            if constexpr (G == 64 && CPL <= 2) {  // dim <= 512: a row's code chunks are CPL per lane of its sixteen
+            if constexpr (G >= 32 && CPL <= 2) {  // 64 < dim <= 512: a row's code chunks are CPL per lane of its sixteen
                 constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
                 const int gl8 = lane & 15, grp8 = lane >> 4;
                 const int nck = (dim + 15) >> 4;  // chunks of sixteen codes; the row's three figures are chunk nck

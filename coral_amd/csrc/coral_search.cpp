@@ -279,9 +279,13 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     // (tuning 2; the library's choice up to 512 floats) or half precision (tuning 1); see beam_search.hip
     // (best-first: the wavefront-per-query kernel with the beam in LDS screens too, see coral_search_prepare)
     const bool codes_possible = idx->dim <= coral::kMaxByteRowDim;  // the inner product is screened on codes only
-    const bool screen_possible = !best_first && idx->dim / 4 > 32 && (idx->metric == CORAL_L2 || codes_possible);
+    // (the rounds kernel takes codes for rows of more than 64 floats; half precision, and the best-first kernels,
+    // need more than 128)
+    const bool wide = idx->dim / 4 > 32, codes_wide = idx->dim / 4 > 16 && !best_first;
+    const bool screen_possible = !best_first && ((wide && idx->metric == CORAL_L2) || ((wide || codes_wide) && codes_possible));
     if (t.screening > 2 || t.screening < -1) return fail(CORAL_ERR_ARG, "screening must be -1, 0, 1 or 2 (got %d)", t.screening);
-    if (t.screening > 0 && idx->dim / 4 <= 32) return fail(CORAL_ERR_ARG, "screening needs more than 128 dimensions");
+    if (t.screening > 0 && !wide && !(t.screening == 2 && codes_wide))
+        return fail(CORAL_ERR_ARG, "screening needs more than 128 dimensions (on eight-bit codes, rounds policy: more than 64)");
     if (t.screening == 1 && idx->metric != CORAL_L2)
         return fail(CORAL_ERR_ARG, "screening in half precision needs the L2 metric");
     if (t.screening == 2 && !codes_possible)

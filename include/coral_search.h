@@ -123,7 +123,7 @@ typedef struct {
                                    runs of L keys per query slot): 1 = that form whatever L is, -1 = never (beams
                                    beyond CORAL_MAX_LDS_BEAM then run on the workgroup-per-query kernel), 0 = by L */
     int32_t best_first_buffer;  /* keys of that insert buffer, a multiple of 64 in 64..4096; 0 = 512 */
-    int32_t screening;          /* rounds policy, more than 128 dimensions: every row is first measured in a
+    int32_t screening;          /* rows of more than 128 floats (rounds policy on codes: more than 64): every row is first measured in a
                                    smaller copy of the vectors (made on first use) and its fp32 row is read only if
                                    rigorous bounds on the exact distance leave open whether it is a candidate or a
                                    beam entry; results and counters are the same bit for bit.  2 = a copy in

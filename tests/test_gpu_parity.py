@@ -179,7 +179,7 @@ def test_beams_in_global_memory_equal_the_oracle(orc, case):
 
 @pytest.mark.parametrize("kind", ["lattice", "large", "beyond_half", "tiny", "dim_not_a_multiple_of_8", "dim_200",
                                   "dim_264", "mixed_magnitudes", "outliers", "tiny_queries", "huge_rows", "ip_unit",
-                                  "ip_raw", "ip_lattice", "ip_mixed_magnitudes"])
+                                  "ip_raw", "ip_lattice", "ip_mixed_magnitudes", "dim_128", "dim_72", "ip_dim_100"])
 def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     """The rounds kernel measures every row in a smaller copy of the vectors first -- half precision, or eight-bit
     codes with a scale per row -- and reads the fp32 row only where bounds on the exact distance leave the row's fate
@@ -193,7 +193,9 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     inner-product metric, which is screened on codes only: unit vectors, raw Gaussian rows, a lattice, rows of very
     different norms.  Ids, distance bits and counters equal the oracle's, with the screening and without."""
     n, dim, R, Q, L, k = 4000, 136, 24, 100, 200, 50
-    dim = {"dim_not_a_multiple_of_8": 140, "dim_200": 200, "dim_264": 264, "ip_raw": 200}.get(kind, dim)
+    dim = {"dim_not_a_multiple_of_8": 140, "dim_200": 200, "dim_264": 264, "ip_raw": 200, "dim_128": 128, "dim_72": 72,
+           "ip_dim_100": 100}.get(kind, dim)
+    narrow = dim <= 128  # the rounds kernel screens such rows on codes; half precision and best-first do not
     ip = kind.startswith("ip_")
     m, mname = (capi.IP, "ip") if ip else (capi.L2, "l2")
     rng = np.random.RandomState(77)
@@ -224,7 +226,7 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     for form in (dict(screening=-1), dict(screening=1), dict(screening=1, beam_in_hbm=True),
                  dict(screening=1, visited_slots_log2=12, threads=256), dict(screening=2),
                  dict(screening=2, beam_in_hbm=True), dict(screening=2, visited_slots_log2=12, threads=256), dict()):
-        if ip and form.get("screening") == 1:  # half precision screens the L2 metric only
+        if (ip or narrow) and form.get("screening") == 1:  # half precision: L2 and more than 128 floats only
             with pytest.raises(capi.CoralError):
                 idx.prepare(Q, L, **form)
             continue
@@ -240,7 +242,7 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
                  dict(screening=2, best_first_packed=True, best_first_table_log2=-1), dict(best_first_table_log2=-1),
                  dict(best_first_long=1), dict(best_first_long=1, screening=-1),
                  dict(best_first_long=1, best_first_buffer=64, best_first_packed=True, screening=2)):
-        if ip and form.get("screening") == 1:
+        if (ip and form.get("screening") == 1) or (narrow and form.get("screening", 0) > 0):
             continue
         idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, **form)
         ids, dists, _ = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)
