@@ -123,15 +123,16 @@ typedef struct {
                                    runs of L keys per query slot): 1 = that form whatever L is, -1 = never (beams
                                    beyond CORAL_MAX_LDS_BEAM then run on the workgroup-per-query kernel), 0 = by L */
     int32_t best_first_buffer;  /* keys of that insert buffer, a multiple of 64 in 64..4096; 0 = 512 */
-    int32_t screening;          /* rows of more than 128 floats (rounds policy on codes: more than 64): every row is first measured in a
-                                   smaller copy of the vectors (made on first use) and its fp32 row is read only if
-                                   rigorous bounds on the exact distance leave open whether it is a candidate or a
-                                   beam entry; results and counters are the same bit for bit.  2 = a copy in
-                                   eight-bit codes (256 bytes per row at dim 200; rows of up to 512 floats),
-                                   1 = a half-precision copy (512 bytes per row at dim 200; L2 only), -1 = off, 0 = the
-                                   eight-bit copy where it applies, else the half-precision one, where the memory
-                                   for it is there.  (Best-first beams of 410 .. 1280 entries screen in half
-                                   precision under 0, 1 and 2.) */
+    int32_t screening;          /* rows of more than 128 floats (rounds policy on codes: more than 64): every row is
+                                   first measured in a smaller copy of the vectors (made on first use) and its fp32
+                                   row is read only if rigorous bounds on the exact distance leave open whether it
+                                   is a candidate or a beam entry; results and counters are the same bit for bit.
+                                   2 = a copy in eight-bit codes (256 bytes per row at dim 200; rows of up to 512
+                                   floats), 1 = a half-precision copy (512 bytes per row at dim 200; L2 only),
+                                   -1 = off, 0 = the eight-bit copy where it applies, else the half-precision one,
+                                   where the memory for it is there.  Best-first: beams of 410 .. 1280 entries screen
+                                   on codes (in half precision under 1, or for rows beyond 512 floats), longer ones
+                                   on codes up to L = 8192 (under 2: whatever L). */
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);
