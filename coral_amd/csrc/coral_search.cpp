@@ -290,7 +290,9 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         return fail(CORAL_ERR_ARG, "screening in half precision needs the L2 metric");
     if (t.screening == 2 && !codes_possible)
         return fail(CORAL_ERR_ARG, "screening on eight-bit codes takes rows of up to %d floats", coral::kMaxByteRowDim);
-    const bool screen = screen_possible && (t.screening > 0 || (t.screening == 0 && !no_screen));
+    // (by itself the library screens rows of more than 128 floats only: at 128 floats and the short beam of the
+    // configuration that has such rows, the codes cost 9 %)
+    const bool screen = screen_possible && (t.screening > 0 || (t.screening == 0 && !no_screen && wide));
     p.screen = !screen ? 0 : t.screening > 0 ? t.screening : (codes_possible ? 2 : 1);
     // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
     // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
