@@ -136,6 +136,19 @@ def test_config2_headline_workload(orc):
     assert np.array_equal(ids3, ids[perm])
     ids4, dists4, _ = idx.search(q[:777], k, 256)
     assert np.array_equal(ids4, ids[:777]) and dists4.tobytes() == dists[:777].tobytes()
+    # the screening of rows on a smaller copy changes no byte of the whole batch's answer and no counter: without it,
+    # in half precision and on eight-bit codes (the library's choice above), at the configuration's beam and at the
+    # headline's; best-first likewise
+    for policy, L in ((capi.POLICY_ROUNDS, 512), (capi.POLICY_ROUNDS, 13312), (capi.POLICY_BEST_FIRST, 512)):
+        ids, dists = kept[(policy, L)]
+        idx.prepare(Q, L, policy=policy)
+        idx.search(q, k, L, policy=policy)
+        cnt = idx.query_counters(Q)
+        for screening in (-1, 1):
+            idx.prepare(Q, L, policy=policy, screening=screening)
+            ids5, dists5, _ = idx.search(q, k, L, policy=policy)
+            assert np.array_equal(ids5, ids) and dists5.tobytes() == dists.tobytes(), (policy, L, screening)
+            assert np.array_equal(idx.query_counters(Q), cnt), (policy, L, screening)
     idx.close()
 
 
