@@ -802,9 +802,14 @@ int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* 
     coral_tuning t;
     std::memset(&t, 0, sizeof t);
     t.policy = policy;  // both policies run on the workgroup-per-query kernel here
-    t.screening = -1;   // (the half-precision copy of the vectors is made by coral_search_prepare)
+    // rows are screened on a smaller copy of the vectors only if an earlier coral_search_prepare has made one:
+    // nothing is allocated here
+    const bool rounds = policy == CORAL_POLICY_ROUNDS;
+    t.screening = rounds && idx->d_vec8 && idx->dim / 4 > 16                            ? 2
+                  : rounds && idx->d_vec16 && idx->dim / 4 > 32 && idx->metric == CORAL_L2 ? 1
+                                                                                           : -1;
     coral_search_plan plan;
-    if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, /*no_screen*/ true, &plan)) return rc;
+    if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, /*no_screen*/ t.screening < 0, &plan)) return rc;
     // the block: 256 bytes of scalars, the per-query counters, then one overflow bitmap per workgroup
     int* scal = reinterpret_cast<int*>(base);
     int32_t* counters = reinterpret_cast<int32_t*>(base + 256);

@@ -189,7 +189,8 @@ CORAL_API int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t
  * 32.3 MiB block of device memory inside the library's code object (each GPU that loads the library holds its
  * copy until the process ends).  The call makes no allocation of any kind, records only kernels on `stream`
  * (NULL = the index's own) and returns without waiting for them; both policies run on the workgroup-per-query
- * kernel, with the results of coral_search_gpu bit for bit.  Limits (CORAL_ERR_ARG beyond them): Q <= 16384,
+ * kernel, with the results of coral_search_gpu bit for bit.  Rows are screened on a smaller copy of the vectors
+ * (rounds policy) only where an earlier coral_search_prepare on this index has made that copy.  Limits (CORAL_ERR_ARG beyond them): Q <= 16384,
  * n <= 4194304, L <= CORAL_MAX_LDS_BEAM.  Every call on a GPU shares that GPU's block: calls that overlap on one
  * GPU (two streams, two indexes, two threads) race; order them. */
 CORAL_API int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* d_ids, float* d_dists,

@@ -41,7 +41,9 @@ def test_no_alloc_entry_point_equals_the_allocating_one():
     idx.set_deleted(mask)
     q_all = make_queries(700, dim, 901)
     # two calls in a row per setting, the second with a smaller input (fewer queries, shorter beam, smaller k):
-    # what the first left in the block must not show in the second
+    # what the first left in the block must not show in the second.  (The very first call finds no coded copy of the
+    # vectors on the index and reads every row in full; the prepare of the comparison leaves one, and every later
+    # rounds call screens on it.)
     for policy in (capi.POLICY_ROUNDS, capi.POLICY_BEST_FIRST):
         for have_delete in (False, True):
             for Q, k, L in ((700, 100, 256), (130, 10, 64)):
