@@ -42,7 +42,7 @@ struct SearchArgs {
     // 16-bit cells; no id ever goes to the bitmap in global memory then
     int32_t direct_bitmap;
     // screening: a half-precision copy of the vectors (rows stride16 bytes apart, the row's norm behind its halves), or
-    // nullptr; tcap2 = entries of the list of rows it leaves for the exact pass (tcap, or 0 without screening)
+    // nullptr; tcap2 = entries of the list of rows it leaves for the exact pass (search_exact_list_cap(tcap), or 0 without screening)
     const unsigned char* vec16;
     size_t stride16;
     // the same screening on a copy in eight-bit codes (rows stride8 bytes apart: codes, then scale, squared norm of
@@ -138,6 +138,8 @@ __host__ __device__ inline int best_first_long_coded_bytes(int dim) { return cod
 hipError_t best_first_long_prepare(int dim, bool packed, bool screen, int bcap, int scap, int* max_wg_per_cu);
 hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& b, hipStream_t stream);
 
+// entries of the list of rows a screening leaves for the exact pass, beside a todo list of tcap
+constexpr int search_exact_list_cap(int tcap) { return tcap < 1024 ? tcap : 1024; }
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening);
 // the half-precision copy of the vectors that the screening phase reads: bytes per row, and its construction
 size_t half_row_stride(int dim);

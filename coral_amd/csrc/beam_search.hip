@@ -167,7 +167,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     }
     float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ntodo2, s_ncand, s_nexp, s_cntf, s_nvis, s_cursor, s_nover;
+    __shared__ int s_qid, s_ntodo, s_ntodo2, s_ncand, s_nexp, s_cntf, s_cursor, s_nover;
     __shared__ int s_wcnt[16];
     __shared__ float s_qq, s_qscale, s_qerr;  // of the query in integer codes: |q~|^2, its scale, |q - q~| rounded up
 
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
 
         for (int i = tid; i < a.table_words; i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
-        if (tid == 0) s_ncand = 0, s_nvis = 0, s_cntf = 0, s_nover = 0, s_cursor = 0, s_ntodo2 = 0;
+        if (tid == 0) s_ncand = 0, s_cntf = 0, s_nover = 0, s_cursor = 0, s_ntodo2 = 0;
         __syncthreads();
 
         float4 qreg[CPL];
@@ -218,6 +218,11 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         st.nb = 0, st.cur = 0, st.live = kKeyMax;
         float thr = 3.402823466e+38f;  // signed form of the farthest sentinel
         int hops = 0, nd = 0, ne = 0, rounds = 0;
+        // Counts that decide what the whole workgroup does next (merge first? measure the open rows first?) are
+        // kept in registers, the same in every thread: each is read from LDS only behind a barrier that no thread's
+        // next addition to it can overtake.  A thread that read the LDS count where it decides could see the
+        // additions of wavefronts already a step ahead, and the workgroup would part ways.
+        int ncand_u = 0, ntodo2_u = 0, nvis = 0;
         bool spill = false;
 
         // ---- screening phase (launches with a half-precision copy of the vectors): todo[0..T) -> todo2[0..s_ntodo2)
@@ -232,7 +237,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         // cannot enter the beam.  Only the rest -- possible beam entries and rows within 0.1 % of the threshold --
         // have their fp32 row read, by the distance phase below; results and counters are what they are without
         // the screening, bit for bit.
-        auto screening_phase = [&](int T) {
+        auto screening_phase = [&](const uint32_t* list, int T) {
             if constexpr (G == 64) {
                 constexpr int RPIH = 2 * U;  // two groups of 32 lanes per wave, U rows in flight per group
                 const int glh = lane & 31, grph = lane >> 5;
@@ -250,7 +255,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     int vid[U];
                     const int r0 = base + grph * U;
 #pragma unroll
-                    for (int u = 0; u < U; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
+                    for (int u = 0; u < U; ++u) vid[u] = (int)list[r0 + u];  // inside the lists' LDS
 #pragma unroll
                     for (int u = 0; u < U; ++u)
                         if (r0 + u >= T) vid[u] = -1;
@@ -331,7 +336,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         // ---- screening phase on eight-bit codes (launches with a.vec8; bounds: search_device.h): the same three
         // classes from a quarter of the bytes.  Sixteen lanes per row (a 256-byte row at dim 200: two cache lines),
         // eight rows in flight per group, four groups per wavefront.
-        auto screening_phase8 = [&](int T) {
+        auto screening_phase8 = [&](const uint32_t* list, int T) {
             if constexpr (G >= 32 && CPL <= 2) {  // 64 < dim <= 512: a row's code chunks are CPL per lane of its sixteen
                 constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
                 const int gl8 = lane & 15, grp8 = lane >> 4;
@@ -340,19 +345,22 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 load_coded_query<CPL8>(qh8, ql8, nck, gl8, cq);
                 const float qq = s_qq, sq = s_qscale, eq = s_qerr;
                 const float s_live = st.live == kKeyMax ? 3.402823466e+38f : key_s(st.live);
+                const uint32_t st8 = (uint32_t)a.stride8;
                 int cnt = 0;
                 for (int base = wave * RPI8; base < T; base += NW * RPI8) {
                     int vid[U8];
                     const int r0 = base + grp8 * U8;
 #pragma unroll
-                    for (int u = 0; u < U8; ++u) vid[u] = (int)todo[r0 + u];  // inside the list's capacity
+                    for (int u = 0; u < U8; ++u) vid[u] = (int)list[r0 + u];  // inside the lists' LDS
 #pragma unroll
                     for (int u = 0; u < U8; ++u)
                         if (r0 + u >= T) vid[u] = -1;
-                    int myid;
-                    bool valid;
+                    const int mi = r0 + gl8;
+                    int myid = (int)list[mi];  // the row this lane files (inside the lists' LDS)
+                    if (gl8 >= U8 || mi >= T) myid = -1;
+                    const bool valid = myid >= 0;
                     float lo, hi;
-                    coded_rows_bounds<CPL8, U8>(a.vec8, a.stride8, nck, gl8, vid, cq, qq, sq, eq, a.metric, myid, valid, lo, hi);
+                    coded_rows_bounds<CPL8, U8>(a.vec8, st8, nck, gl8, vid, myid, cq, qq, sq, eq, a.metric, lo, hi);
                     const bool gone = valid && lo > thr;
                     const bool counted = valid && !gone && hi < thr && lo > s_live;
                     const bool exact = valid && !gone && !counted;
@@ -480,6 +488,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 st.cur ^= 1;
                 st.live = st.nb == L ? dst[L - 1] : kKeyMax;
                 if (tid == 0) s_ncand = 0;
+                ncand_u = 0;
                 __syncthreads();
                 return;
             }
@@ -581,6 +590,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             st.cur ^= 1;
             st.live = st.nb == L ? dst[L - 1] : kKeyMax;
             if (tid == 0) s_ncand = 0;
+            ncand_u = 0;
             __syncthreads();
         };
 
@@ -588,15 +598,39 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         // barrier; the candidates they add must fit the buffer)
         const bool screening = (a.vec16 != nullptr || a.vec8 != nullptr) && a.policy == 0;
         auto flush_exact = [&]() {
-            const int n2 = s_ntodo2;
+            const int n2 = ntodo2_u;
             if (n2 == 0) return;
-            if (s_ncand + n2 > CCAP) merge();  // merge() starts and ends with a barrier
+            if (ncand_u + n2 > CCAP) merge();  // merge() starts and ends with a barrier
             PHASE_MARK(5);
             distance_phase(todo2, n2);
             __syncthreads();
             if (tid == 0) s_ntodo2 = 0;
+            ncand_u = s_ncand, ntodo2_u = 0;  // (the next additions to either lie behind the barrier below)
             __syncthreads();
             PHASE_MARK(4);
+        };
+
+        // ---- the screening of todo[0..T): in pieces that the list for the exact pass has room for whatever the
+        // screening leaves (entered by every thread after a barrier, ends with one)
+        auto screen_list = [&](int T) {
+            for (int off = 0; off < T;) {
+                // (what is left goes in one piece where the emptied list could take it whole: a small second piece
+                // is one more exposed wait)
+                int n = min(T - off, a.tcap2 - ntodo2_u);
+                if (n < (T - off <= a.tcap2 ? T - off : a.tcap2 / 2)) {
+                    flush_exact();
+                    n = min(T - off, a.tcap2);
+                }
+                if (a.vec8 != nullptr)
+                    screening_phase8(todo + off, n);
+                else
+                    screening_phase(todo + off, n);
+                __syncthreads();
+                ntodo2_u = s_ntodo2;
+                PHASE_MARK(7);
+                off += n;
+                if (off < T) __syncthreads();  // every thread has the count before the next piece adds to it
+            }
         };
 
         PHASE_MARK(0);
@@ -611,8 +645,8 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         distance_phase(todo, M);
         merge();
         PHASE_MARK(1);
-        if (tid == 0) s_nvis = M, s_cntf = 0;
-        nd = M;
+        if (tid == 0) s_cntf = 0;
+        nd = M, nvis = M;
         if (a.policy == 1) hops = M;
 
         // ---- rounds
@@ -679,7 +713,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             // ids are requested one chunk ahead -- and the entry whose row they come from two chunks ahead -- so
             // that both waits pass while the chunk before is being measured.  With two workgroups per CU the other
             // workgroup covers those waits and the look-ahead only costs (measured); with one it pays.
-            const int ech = TCAP / R;
+            const int ech = (screening ? min(TCAP, NT) : TCAP) / R;
             ne += nexp;
             const bool ahead = a.prefetch_rows != 0 && ech * R <= NT;
             const int pe = tid / R, pj = tid - pe * R;  // this thread's entry of a chunk and neighbour slot
@@ -689,9 +723,14 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 if (pe < min(ech, nexp)) vpre = a.nbrs[(size_t)elist[pe] * R + pj];
                 if (pe < ech && ech + pe < nexp) epre = elist[ech + pe];
             }
+            // With a screening, the ids of several chunks collect in the todo list (while the next chunk's could
+            // all still join it) and are screened together: a screening of a few hundred rows is one exposed
+            // memory wait, of a thousand and more the same wait and some work under it.  (Screening only
+            // whole passes of the workgroup, the rest waiting in the list for the next ids, gains nothing: measured.)
+            int tprev = 0;  // ids in the todo list from the chunks before, not yet screened
             for (int e0 = 0; e0 < nexp; e0 += ech) {
-                if (!spill && s_nvis > a.vis_limit) spill = true;
-                if (tid == 0) s_ntodo = 0;
+                if (!spill && nvis > a.vis_limit) spill = true;
+                if (tid == 0 && tprev == 0) s_ntodo = 0;
                 __syncthreads();
                 const int total = min(ech, nexp - e0) * R;
                 for (int f0 = 0; f0 < total; f0 += NT) {
@@ -714,12 +753,12 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     }
                 }
                 __syncthreads();
-                const int T = s_ntodo;
+                const int tall = s_ntodo, T = tall - tprev;
                 nd += T;
                 PHASE_MARK(3);
-                if (!screening && s_ncand + T > CCAP) merge();  // merge() starts and ends with a barrier
+                if (!screening && ncand_u + T > CCAP) merge();  // merge() starts and ends with a barrier
                 PHASE_MARK(5);
-                if (tid == 0) s_nvis += T;
+                nvis += T;
                 if (ahead) {
                     // the next chunk's ids (their entries arrived a chunk ago) and the entries of the chunk after
                     vpre = -1;
@@ -730,17 +769,17 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 if (screening) {
                     // what the screening leaves for the exact pass collects over the chunks of a round (the round's
                     // threshold does not move) and is measured when the list could overflow, and at the round's end
-                    if (s_ntodo2 + T > a.tcap2) flush_exact();
-                    if (a.vec8 != nullptr)
-                        screening_phase8(T);
-                    else
-                        screening_phase(T);
-                    __syncthreads();
-                    PHASE_MARK(7);
+                    if (e0 + ech >= nexp || tall + ech * R > TCAP) {
+                        screen_list(tall);
+                        tprev = 0;
+                    } else {
+                        tprev = tall;
+                    }
                 } else {
                     distance_phase(todo, T);
+                    __syncthreads();
+                    ncand_u = s_ncand;  // (the next chunk's additions lie behind the barrier at its start)
                 }
-                __syncthreads();
                 PHASE_MARK(4);
             }
             if (screening) flush_exact();
@@ -878,7 +917,7 @@ static kernel_fn pick_kernel(int dim, bool big) {
 
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening) {
     const size_t Lp = (size_t)((L + 3) & ~3);
-    if (screening) tcap *= 2;  // the list of rows the screening leaves for the exact pass
+    if (screening) tcap += search_exact_list_cap(tcap);  // the list of rows the screening leaves for the exact pass
     const size_t beams = big ? (size_t)kBeamSampleKeys * 8 : Lp * 8 * 2 + Lp * 4;  // (big: the merge's sample) two key buffers and the expand list
     const size_t coded_query = screening ? 2 * (size_t)((dim + 15) & ~15) : 0;  // two bytes per dimension
     return beams + (size_t)ccap * 8 + (size_t)table_words * 4 + (size_t)tcap * 4 + (size_t)ocap * 4 +

@@ -325,10 +325,11 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                         const int r0 = base + grp8 * U8;
 #pragma unroll
                         for (int u = 0; u < U8; ++u) vid[u] = r0 + u < T ? (int)todo[r0 + u] : -1;
-                        int myid;
-                        bool valid;
+                        const int mi = r0 + gl8;
+                        const int myid = (gl8 < U8 && mi < T) ? (int)todo[mi] : -1;  // the row this lane files
+                        const bool valid = myid >= 0;
                         float lo, hi;
-                        coded_rows_bounds<CPL8, U8>(b.vec8, b.stride8, nck, gl8, vid, cq, c_qq, c_sq, c_eq, a.metric, myid, valid, lo, hi);
+                        coded_rows_bounds<CPL8, U8>(b.vec8, (uint32_t)b.stride8, nck, gl8, vid, myid, cq, c_qq, c_sq, c_eq, a.metric, lo, hi);
                         const bool exact = valid && !(lo > s_live);
                         const uint64_t m = __ballot(exact);
                         if (exact) todo2[n2 + prefix_popc(m)] = (uint32_t)myid;

@@ -366,8 +366,10 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
                     lds_for(min_cap, min_cap));
     int tcap = min_cap;
     const int wg_fit = (int)(lds_max / lds_for(min_cap, min_cap));
-    for (int cap : {1024, 512}) {
+    for (int cap : {2048, 1024, 512}) {
         if (cap <= tcap || best_first) break;
+        // (twice the ids of one pass of 1024 threads: a screening collects the ids of several chunks, see beam_search.hip)
+        if (cap == 2048 && !(screen && wg_fit == 1)) continue;
         if (lds_for(cap, cap) <= lds_max && (int)(lds_max / lds_for(cap, cap)) >= std::min(wg_fit, 2)) {
             tcap = cap;
             break;
@@ -651,7 +653,7 @@ static coral::SearchArgs search_args(const coral_index* idx, const coral_search_
     a.prefetch_rows = p.prefetch;
     a.vec16 = p.screen == 1 ? idx->d_vec16 : nullptr, a.stride16 = coral::half_row_stride(idx->dim);
     a.vec8 = p.screen == 2 ? idx->d_vec8 : nullptr, a.stride8 = coral::byte_row_stride(idx->dim);
-    a.tcap2 = p.screen ? p.tcap : 0;
+    a.tcap2 = p.screen ? coral::search_exact_list_cap(p.tcap) : 0;
     a.scap = p.big ? coral::kBeamSampleKeys : 0;
     return a;
 }

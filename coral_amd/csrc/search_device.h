@@ -96,41 +96,49 @@ __device__ __forceinline__ void load_coded_query(const signed char* qh8, const s
         }
 }
 
-// Rows vid[0..U8) (-1: none) of one group of sixteen lanes, all requested before any is added up.  Lane gl8 < U8 of the
-// group files row vid[gl8]: myid, valid, and the bounds lo <= d <= hi of its exact distance (lo = 0 and hi = inf for a
-// row that takes no part; a NaN anywhere fails every comparison a caller makes with them).
+// Rows vid[0..U8) (-1: none) of one group of sixteen lanes, in three steps so that a caller with more rows to come can
+// request the next ones before it finishes these: request (all loads back to back), dots (the integer sums, which
+// wait for the loads and leave their registers free), finish (the lane that files a row gets the bounds
+// lo <= d <= hi of its exact distance).  Lane gl8 < U8 of the group files row vid[gl8]; the caller hands it that id as
+// myid (-1: the lane files none; lo and hi are then worthless).  A row that takes no part has lo = 0 and hi = inf; a
+// NaN anywhere fails every comparison a caller makes with the bounds.
 //
 // Inner product (metric 1; the signed distance is -q.x): q.x = q~.x~ + q~.(x - x~) + (q - q~).x, so
 // |q.x - q~.x~| <= |q~| e + eq (|x~| + e); the bound is widened by 2e-4 (|q~| + eq)(|x~| + e) for the fp32 rounding of
 // the exact inner product and of the computed q~.x~ (each at most dim 2^-24 |q| |x|, dim <= 512).
 template <int CPL8, int U8>
-__device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, size_t stride8, int nck, int gl8,
-                                                  const int (&vid)[U8], const CodedQuery<CPL8>& q, float qq, float sq,
-                                                  float eq, int metric, int& myid, bool& valid, float& lo, float& hi) {
+struct CodedRows {
     uint4 hb[U8][CPL8];
+    float4 fig;  // s, |x~|^2, e of the row this lane files
+};
+
+// Every lane requests a chunk of every row, with no condition: a lane whose chunk lies past the codes takes the row's
+// figures instead (its query codes are zero, so whatever it reads adds nothing), a row that is none takes row 0 (and
+// is dropped by its lane).  One 32 x 32 -> 64 bit multiply-add per address.
+template <int CPL8, int U8>
+__device__ __forceinline__ void coded_rows_request(const unsigned char* vec8, uint32_t st8, int nck, int gl8,
+                                                   const int (&vid)[U8], int myid, CodedRows<CPL8, U8>& r) {
 #pragma unroll
     for (int u = 0; u < U8; ++u) {
-        const uint4* row = reinterpret_cast<const uint4*>(vec8 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * stride8);
+        const uint4* row = reinterpret_cast<const uint4*>(vec8 + (uint64_t)(uint32_t)(vid[u] < 0 ? 0 : vid[u]) * st8);
 #pragma unroll
         for (int t = 0; t < CPL8; ++t) {
             const int c = gl8 + 16 * t;
-            hb[u][t] = (vid[u] >= 0 && c < nck) ? row[c] : make_uint4(0u, 0u, 0u, 0u);
+            r.hb[u][t] = row[c < nck ? c : nck];
         }
     }
-    myid = vid[0];
-#pragma unroll
-    for (int u = 1; u < U8; ++u)
-        if (gl8 == u) myid = vid[u];
-    valid = gl8 < U8 && myid >= 0;
-    float4 fig = make_float4(0, 0, 0, 0);  // s, |x~|^2, e
-    if (valid) fig = *reinterpret_cast<const float4*>(vec8 + (uint64_t)(uint32_t)myid * stride8 + (size_t)nck * 16);
-    int acc[U8];
+    r.fig = make_float4(0, 0, 0, 0);
+    if (myid >= 0) r.fig = *reinterpret_cast<const float4*>(vec8 + (uint64_t)(uint32_t)myid * st8 + (uint32_t)nck * 16u);
+}
+
+template <int CPL8, int U8>
+__device__ __forceinline__ void coded_rows_dots(const CodedRows<CPL8, U8>& r, const CodedQuery<CPL8>& q, int (&acc)[U8]) {
 #pragma unroll
     for (int u = 0; u < U8; ++u) {
         int dh = 0, dl = 0;
 #pragma unroll
         for (int t = 0; t < CPL8; ++t) {
-            const int w[4] = {(int)hb[u][t].x, (int)hb[u][t].y, (int)hb[u][t].z, (int)hb[u][t].w};
+            const int w[4] = {(int)r.hb[u][t].x, (int)r.hb[u][t].y, (int)r.hb[u][t].z, (int)r.hb[u][t].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 dh = __builtin_amdgcn_sdot4(w[j], q.h[t][j], dh, false);
@@ -139,6 +147,11 @@ __device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, siz
         }
         acc[u] = 128 * dh + dl;  // below 2^31 for 512 dimensions: 512 * 127 * 16256
     }
+}
+
+template <int U8>
+__device__ __forceinline__ void coded_rows_finish(int (&acc)[U8], int gl8, const float4& fig, float qq, float sq, float eq,
+                                                  int metric, float& lo, float& hi) {
 #pragma unroll
     for (int u = 0; u < U8; ++u) {
         acc[u] = acc[u] + dpp_mov_i<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
@@ -153,15 +166,31 @@ __device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, siz
     if (metric == 0) {
         const float both = qq + fig.y;
         const float d8 = both - (2.0f * sq * fig.x) * (float)mine, delta = 16.0f * 5.9604645e-8f * both, e = fig.z + eq;
-        const float lo_root = fmaxf(sqrtf(fmaxf(d8 - delta, 0.0f)) - e, 0.0f);
-        const float hi_root = sqrtf(fmaxf(d8 + delta, 0.0f)) + e;
+        // (the hardware's square root, good to one unit in the last place and only trusted on normal numbers: below
+        // 1e-36 the lower end takes 0 and the upper end the root of 1e-36; the 1e-4 covers the last place)
+        const float under = d8 - delta, over = fmaxf(d8 + delta, 1.0e-36f);
+        const float lo_root = fmaxf((under < 1.0e-36f ? 0.0f : __builtin_amdgcn_sqrtf(under)) - e, 0.0f);
+        const float hi_root = __builtin_amdgcn_sqrtf(over) + e;
         lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
     } else {
         const float p = (sq * fig.x) * (float)mine;  // q~.x~
-        const float nq = sqrtf(qq) * (1.0f + 1.0e-6f), nx = sqrtf(fig.y) * (1.0f + 1.0e-6f), e = fig.z;
+        const float nq = sqrtf(qq) * (1.0f + 1.0e-6f), e = fig.z;
+        const float nx = __builtin_amdgcn_sqrtf(fmaxf(fig.y, 1.0e-36f)) * (1.0f + 1.0e-6f);
         const float bound = (nq * e + eq * (nx + e) + 2.0e-4f * (nq + eq) * (nx + e)) * (1.0f + 1.0e-5f);
         lo = (0.0f - p) - bound, hi = (0.0f - p) + bound;  // e = inf or eq = inf: lo = -inf, hi = inf (or NaN)
     }
+}
+
+// the three steps in one go
+template <int CPL8, int U8>
+__device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, uint32_t st8, int nck, int gl8,
+                                                  const int (&vid)[U8], int myid, const CodedQuery<CPL8>& q, float qq,
+                                                  float sq, float eq, int metric, float& lo, float& hi) {
+    CodedRows<CPL8, U8> r;
+    coded_rows_request<CPL8, U8>(vec8, st8, nck, gl8, vid, myid, r);
+    int acc[U8];
+    coded_rows_dots<CPL8, U8>(r, q, acc);
+    coded_rows_finish<U8>(acc, gl8, r.fig, qq, sq, eq, metric, lo, hi);
 }
 
 // number of set bits of m below the calling lane
