@@ -534,43 +534,103 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             uint64_t* dst = st.cur ? beam0 : beam1;
             const int nb = st.nb;
             if constexpr (BIG) {
-                // The beam is in global memory: every access is a trip to L2.  Beam keys are fetched four per
-                // thread before the first is placed, and keys outside the candidates' range need no search; a
-                // candidate's search through the beam starts in an LDS sample of every 2^ss-th beam key, so that
-                // only its last few steps (inside one or two cache lines) go to memory.
-                int ss = 0;
-                while (((nb - 1) >> ss) + 1 > a.scap) ++ss;
-                const int ns = nb > 0 ? ((nb - 1) >> ss) + 1 : 0;
-                for (int j = tid; j < ns; j += NT) samp[j] = src[(size_t)j << ss];
+                // The beam is in global memory: every access is a trip to L2 or beyond.  Beam keys are fetched eight
+                // per thread before the first is placed, and keys outside the candidates' range need no search.
+                // A candidate's place is its index plus the number of beam keys below it.  That number is not
+                // searched for in the beam (a chain of dependent reads from memory): every beam key has just found
+                // its own count b of candidates below it, and the keys below candidate j are exactly those with
+                // b <= j.  So the keys are counted per value of b (16-bit counts, two to a word, in the LDS that
+                // holds the sample otherwise; one addition per run of equal values among a wavefront's 64
+                // consecutive keys) and a prefix sum over the counts gives every candidate its place.  Beams of
+                // 65536 keys and more, or more candidates than there are counts, take the search: through an LDS
+                // sample of every 2^ss-th beam key, then the last few steps in memory.
+                const bool counted = nc <= 4 * a.scap && nb < 65536;
+                uint32_t* cnt = reinterpret_cast<uint32_t*>(samp);
+                const int ncw = (nc + 1) >> 1;
+                int ss = 0, ns = 0;
+                if (counted) {
+                    for (int w = tid; w < ncw; w += NT) cnt[w] = 0u;
+                    __syncthreads();
+                } else {
+                    while (((nb - 1) >> ss) + 1 > a.scap) ++ss;
+                    ns = nb > 0 ? ((nb - 1) >> ss) + 1 : 0;
+                    for (int j = tid; j < ns; j += NT) samp[j] = src[(size_t)j << ss];
+                }
                 const uint64_t c_lo = cand[0], c_hi = cand[nc - 1];
-                for (int i0 = tid; i0 < nb; i0 += 4 * NT) {
-                    uint64_t key[4];
+                for (int i0 = tid; i0 < nb; i0 += 8 * NT) {
+                    uint64_t key[8];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) key[u] = i0 + u * NT < nb ? src[i0 + u * NT] : kKeyMax;
+                    for (int u = 0; u < 8; ++u) key[u] = i0 + u * NT < nb ? src[i0 + u * NT] : kKeyMax;
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < 8; ++u) {
                         const int i = i0 + u * NT;
+                        int below = nc;  // (a lane past the beam's end counts nothing)
                         if (i < nb) {
-                            const int below = key[u] < c_lo ? 0 : key[u] > c_hi ? nc : lower_bound_u64(cand, nc, key[u]);
+                            below = key[u] < c_lo ? 0 : key[u] > c_hi ? nc : lower_bound_u64(cand, nc, key[u]);
                             if (i + below < L) dst[i + below] = key[u];
+                        }
+                        if (counted) {
+                            // the wavefront's keys ascend with the lane, and so do their counts: the lanes with
+                            // below < nc are the first few, and equal counts sit side by side
+                            const int prev = __shfl_up(below, 1, 64);
+                            const bool in = below < nc;
+                            const bool head = in && (lane == 0 || prev != below);
+                            const uint64_t hm = __ballot(head);
+                            const int nin = __popcll(__ballot(in));
+                            if (head) {
+                                const uint64_t after = hm & ~((2ull << lane) - 1ull);  // heads in the lanes above
+                                const int end = after ? min(__ffsll((long long)after) - 1, nin) : nin;
+                                atomicAdd(&cnt[below >> 1], (uint32_t)(end - lane) << (16 * (below & 1)));
+                            }
                         }
                     }
                 }
-                __syncthreads();  // the sample is complete
-                for (int j = tid; j < nc; j += NT) {
-                    const uint64_t key = cand[j];
-                    const int js = lower_bound_u64(samp, ns, key);
-                    int lo = js == 0 ? 0 : ((js - 1) << ss) + 1, hi = js == ns ? nb : (js << ss);
-                    while (lo < hi) {
-                        const int mid = (lo + hi) >> 1;
-                        if (src[mid] < key)
-                            lo = mid + 1;
-                        else
-                            hi = mid;
+                __syncthreads();  // the counts (or the sample) are complete
+                if (counted) {
+                    int base = 0;  // beam keys below the candidates of the passes before
+                    for (int w0 = 0; w0 < ncw; w0 += NT) {
+                        const int w = w0 + tid;
+                        const uint32_t c2 = w < ncw ? cnt[w] : 0u;
+                        const int c_even = (int)(c2 & 0xffffu), c_odd = (int)(c2 >> 16);
+                        const int incl = wave_inclusive_sum(c_even + c_odd);
+                        if (lane == 63) s_wcnt[wave] = incl;
+                        __syncthreads();
+                        int before = base, total = 0;
+                        for (int x = 0; x < NW; ++x) {
+                            const int c = s_wcnt[x];
+                            before += x < wave ? c : 0;
+                            total += c;
+                        }
+                        const int excl = before + incl - (c_even + c_odd);
+                        const int j = 2 * w;
+                        if (j < nc) {
+                            const int pos = j + excl + c_even;
+                            if (pos < L) dst[pos] = cand[j];
+                            if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
+                        }
+                        if (j + 1 < nc) {
+                            const int pos = j + 1 + excl + c_even + c_odd;
+                            if (pos < L) dst[pos] = cand[j + 1];
+                        }
+                        base += total;
+                        __syncthreads();  // the wavefronts' totals are read before the next pass posts its own
                     }
-                    const int pos = j + lo;
-                    if (pos < L) dst[pos] = key;
-                    if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
+                } else {
+                    for (int j = tid; j < nc; j += NT) {
+                        const uint64_t key = cand[j];
+                        const int js = lower_bound_u64(samp, ns, key);
+                        int lo = js == 0 ? 0 : ((js - 1) << ss) + 1, hi = js == ns ? nb : (js << ss);
+                        while (lo < hi) {
+                            const int mid = (lo + hi) >> 1;
+                            if (src[mid] < key)
+                                lo = mid + 1;
+                            else
+                                hi = mid;
+                        }
+                        const int pos = j + lo;
+                        if (pos < L) dst[pos] = key;
+                        if (j == 0 && pos < s_cursor) s_cursor = pos;  // entries before the cursor are all expanded
+                    }
                 }
             } else {
                 for (int i = tid; i < nb; i += NT) {

@@ -45,18 +45,6 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// inclusive prefix sum over the 64 lanes: four steps inside the rows of 16 lanes, then the totals of the rows
-// before (row_bcast15 into rows 1 and 3, row_bcast31 into rows 2 and 3); lanes without a source add 0
-__device__ __forceinline__ int wave_inclusive_sum(int v) {
-    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
-    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
-    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
-    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
-    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast15
-    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast31
-    return v;
-}
-
 // PACKED: the visited state of a slot is one 32-bit word per 24 nodes (8 bits of epoch, 24 flags) instead of one
 // byte per node: a sixth of the memory, the same one line per test.
 // SCREEN: rows are first measured in a smaller copy of the vectors (rows of more than 128 floats): 1 the half-precision

@@ -39,17 +39,6 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// inclusive prefix sum over the 64 lanes (see best_first.hip)
-__device__ __forceinline__ int wave_inclusive_sum(int v) {
-    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
-    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
-    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
-    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
-    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast15
-    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast31
-    return v;
-}
-
 // The long run is written by some lanes and read by others of the same wavefront: both go past the CU's cache
 // (agent-scope atomics), ordered by the fences of the steps that separate them.
 __device__ __forceinline__ uint64_t gload(const uint64_t* p) {

@@ -193,6 +193,18 @@ __device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, uin
     coded_rows_finish<U8>(acc, gl8, r.fig, qq, sq, eq, metric, lo, hi);
 }
 
+// inclusive prefix sum over the 64 lanes: four steps inside the rows of 16 lanes, then the totals of the rows
+// before (row_bcast15 into rows 1 and 3, row_bcast31 into rows 2 and 3); lanes without a source add 0
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast15
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast31
+    return v;
+}
+
 // number of set bits of m below the calling lane
 __device__ __forceinline__ int prefix_popc(uint64_t m) {
     const uint32_t lane = threadIdx.x & 63;
