@@ -368,8 +368,11 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     const int wg_fit = (int)(lds_max / lds_for(min_cap, min_cap));
     for (int cap : {2048, 1024, 512}) {
         if (cap <= tcap || best_first) break;
-        // (twice the ids of one pass of 1024 threads: a screening collects the ids of several chunks, see beam_search.hip)
-        if (cap == 2048 && !(screen && wg_fit == 1)) continue;
+        // (twice the ids of one pass of 1024 threads: a screening collects the ids of several chunks, see
+        // beam_search.hip; for beams in global memory only -- with a beam in LDS the candidate buffer would double
+        // with the list, the beam's worst entry be refreshed half as often, and a 512-float inner-product search at
+        // L = 256 lost 5 %)
+        if (cap == 2048 && !(screen && wg_fit == 1 && p.big)) continue;
         if (lds_for(cap, cap) <= lds_max && (int)(lds_max / lds_for(cap, cap)) >= std::min(wg_fit, 2)) {
             tcap = cap;
             break;
