@@ -70,7 +70,11 @@ __global__ __launch_bounds__(256) void bfs_expand_kernel(const int32_t* __restri
             if (valid) s_buf[base + __popcll(m & ((1ull << lane) - 1ull))] = v;
         }
         __syncthreads();
-        if (s_cnt > kBfsStage - 256) flush();  // a step adds at most 256
+        // every thread reads the count before any thread's next step can add to it: a thread that read it later
+        // could see more than the others and flush alone
+        const int staged = s_cnt;
+        __syncthreads();
+        if (staged > kBfsStage - 256) flush();  // a step adds at most 256
     }
     flush();
 }
