@@ -92,6 +92,7 @@ class Bench:
         self.d_q = torch.from_numpy(self.queries).cuda()
         self.d_ids = torch.empty((self.Q, self.k), dtype=torch.int32, device="cuda")
         self.d_gt = torch.from_numpy(self.gt).cuda()
+        self.workgroups = 0  # of the search launch; 0: the library's choice (what a CU holds x the CUs)
 
     def close(self):
         self.idx.close()
@@ -101,7 +102,7 @@ class Bench:
         torch, idx = self.torch, self.idx
         Q = Q or self.Q
         k, dim = self.k, self.dim
-        idx.prepare(Q, L, policy=policy)
+        idx.prepare(Q, L, policy=policy, workgroups=self.workgroups)
         for _ in range(warmup):
             idx.search_device(self.d_q.data_ptr(), self.d_ids.data_ptr(), None, Q, k, policy=policy)
         torch.cuda.synchronize()
@@ -343,6 +344,9 @@ def main():
                     help="no further leg beside the headline is started once the run is this old")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for memory counters)")
+    ap.add_argument("--workgroups", type=int, default=0,
+                    help="with --L: workgroups of the search launch (0: the library's choice), to see how the rate "
+                         "scales with the CUs in use")
     ap.add_argument("--n", type=int, default=1000000, help=argparse.SUPPRESS)
     ap.add_argument("--queries", type=int, default=10000, help=argparse.SUPPRESS)
     args = ap.parse_args()
@@ -393,6 +397,7 @@ def main():
     probes = []
     if args.L:
         L_head = args.L
+        b.workgroups = args.workgroups
     else:
         L_head, probes = b.operating_point(policy)
         log("operating point: L=%s after probes %s" % (L_head, [(p[0], round(p[1], 4)) for p in probes]))
@@ -415,7 +420,7 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "L": head["L"], "k": k, "policy": args.policy,
                    "recall@100": head["recall"], "recall_met": recall_met,
-                   "qps_at_config_L": head["qps"],
+                   "qps_at_config_L": head["qps"], "workgroups": args.workgroups if args.L else 0,
                    "note": "L is the smallest multiple of %d whose recall@100 over the whole batch is >= %.2f on this "
                            "workload (isotropic 200-d Gaussian base: a degree-32 graph needs a beam this long); the "
                            "configuration's own L = 256 and 512 are under 'also'" % (L_STEP, RECALL_TARGET),
