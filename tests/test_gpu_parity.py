@@ -132,6 +132,28 @@ BIG_CASES = [
 ]
 
 
+def test_merge_forms_of_a_full_long_beam(orc):
+    """The merge of a beam in global memory places the candidates from counts while the beam holds fewer than 65536
+    keys and a merge brings at most 2048 candidates, and by a search through the beam otherwise: a search that fills the
+    longest beam the library takes passes through both, with and without the screening on codes (whose todo list
+    collects the ids of several chunks), and with a candidate buffer of 4096."""
+    n, dim, R, L, k, M, Q = 80000, 72, 32, capi.MAX_BEAM, 100, 16, 5
+    base, nbrs, starts = problem(n, dim, R, seed=4242, n_start=M)
+    q = make_queries(Q, dim, 4243)
+    prob = orc.Problem(base, nbrs, starts)
+    oi, od, os_, _ = orc.search_B(prob, q, k, L, start_order=WAVE64, nbr_order=WAVE64)
+    assert (os_[:, 2] > L).all()  # every query measures more rows than the beam holds: the beam fills
+    idx = capi.Index(base, nbrs, starts)
+    for form in (dict(screening=2), dict(screening=-1), dict(screening=-1, cand_cap=4096), dict(screening=2, cand_cap=4096)):
+        print("merge form", form, flush=True)
+        idx.prepare(Q, L, beam_in_hbm=True, **form)
+        ids, dists, st = idx.search(q, k, L)
+        assert np.array_equal(ids, oi), form
+        assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), form
+        assert np.array_equal(idx.query_counters(Q), os_), form
+    idx.close()
+
+
 @pytest.mark.parametrize("case", BIG_CASES, ids=lambda c: "n%d_d%d_R%d_%s_p%d_L%d_k%d_M%d_rg%s_s%d_w%d_del%d" % c)
 def test_beams_in_global_memory_equal_the_oracle(orc, case):
     """Beams beyond CORAL_MAX_LDS_BEAM (the reference sets no limit on L, src/search.cu:400-408; its driver grows L
