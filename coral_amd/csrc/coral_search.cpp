@@ -395,6 +395,15 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     int wg_per_cu = 0;
     HIP_TRY(coral::search_kernel_prepare(idx->dim, p.big, p.lds_bytes, threads, &wg_per_cu));
     if (wg_per_cu <= 0) return fail(CORAL_ERR_DEVICE, "kernel does not fit the device");
+    // A small batch that the chip cannot take at once in workgroups of 512 threads, but can in workgroups of 256 (twice
+    // as many per CU where LDS allows), runs in one go instead of two: 1000 queries on a 100 000-node graph at L = 64
+    // take 276 us instead of 312.
+    if (t.threads == 0 && threads == 512 && !best_first && Q > (int64_t)wg_per_cu * idx->num_cu) {
+        int wg256 = 0;
+        if (coral::search_kernel_prepare(idx->dim, p.big, p.lds_bytes, 256, &wg256) == hipSuccess && wg256 > wg_per_cu &&
+            Q <= (int64_t)wg256 * idx->num_cu)
+            threads = 256, wg_per_cu = wg256;
+    }
     int workgroups = t.workgroups > 0 ? t.workgroups : wg_per_cu * idx->num_cu;
     p.workgroups = std::min(workgroups, (int)Q);
     p.tcap = tcap, p.ccap = ccap, p.threads = threads, p.id_bits = id_bits, p.ocap = ocap;
