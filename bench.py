@@ -29,8 +29,10 @@ HBM_PEAK_GBPS = 8000.0
 RECALL_TARGET = 0.90
 L_STEP = 512
 # files whose text decides what the search kernels do; profiles/search_kernels_traffic.txt names their digest
+# (the kernels, and the host code that plans their launches: workgroup size, list capacities, visited form, screening form)
 KERNEL_SOURCES = ("coral_amd/csrc/beam_search.hip", "coral_amd/csrc/beam_search.h", "coral_amd/csrc/best_first.hip",
-                  "coral_amd/csrc/best_first_long.hip", "coral_amd/csrc/search_device.h")
+                  "coral_amd/csrc/best_first_long.hip", "coral_amd/csrc/search_device.h",
+                  "coral_amd/csrc/coral_search.cpp", "coral_amd/csrc/index_internal.h")
 T0 = time.time()
 
 
@@ -39,8 +41,25 @@ def log(msg):
 
 
 def algorithmic_bytes(expansions, dist_evals, Q, dim, k, R=32):
-    """Graph rows (R int32 each) + vector rows + the queries read + ids and distances written."""
+    """What the reference's own kernel would read for the same traversal: graph rows (R int32 each), one fp32 vector
+    row per distance evaluation, the queries, ids and distances written."""
     return expansions * R * 4 + dist_evals * dim * 4 + Q * (dim * 4 + k * 8)
+
+
+def scheme_bytes(st, plan, Q, dim, k, R=32):
+    """What this library's kernels must read for the traversal, from the kernels' own counts of the rows they
+    requested: a graph row per expansion, a row of the smaller copy (eight-bit codes or half precision) per screened
+    evaluation, an fp32 row per evaluation the screening left open (all of them without screening), the queries,
+    the ids and the per-query counters written.  No credit for scratch (beam passes, visited state): those are
+    `scratch_bytes`."""
+    return (st.expansions * R * 4 + st.screened_rows * plan.screen_row_bytes + st.exact_rows * dim * 4 +
+            Q * (dim * 4 + k * 4 + 32))
+
+
+def scratch_bytes(st):
+    """Bytes of the launch's own state in global memory: passes over beams that do not live in LDS (32-bit words
+    counted by the kernel) and visited-state requests, each priced at one 32-byte sector."""
+    return st.beam_words * 4 + st.visited_requests * 32
 
 
 def kernel_sources_digest():
@@ -114,14 +133,25 @@ class Bench:
         torch.cuda.synchronize()
         wall = time.perf_counter() - t
         hits = idx.verify(self.d_ids.data_ptr(), self.d_gt.data_ptr(), Q, k)
-        bytes_per_launch = algorithmic_bytes(st.expansions, st.dist_evals, Q, dim, k)
+        plan = idx.plan_info()
+        alg_bytes = algorithmic_bytes(st.expansions, st.dist_evals, Q, dim, k)
+        bytes_per_launch = scheme_bytes(st, plan, Q, dim, k)
+        scratch = scratch_bytes(st)
         avg_kernel = kernel_s / steps
         return {"L": L, "queries": Q, "qps": steps * Q / wall, "ms_per_step": 1e3 * wall / steps,
                 "recall": hits / float(Q * k), "kernel_ms": 1e3 * avg_kernel,
+                # the bytes the kernels asked for (counted on the device), over the kernel time
                 "gbps": bytes_per_launch / avg_kernel / 1e9, "frac": bytes_per_launch / avg_kernel / 1e9 / HBM_PEAK_GBPS,
-                "bytes_per_launch": bytes_per_launch,
+                "bytes_per_launch": bytes_per_launch, "scratch_bytes_per_launch": scratch,
+                "frac_with_scratch": (bytes_per_launch + scratch) / avg_kernel / 1e9 / HBM_PEAK_GBPS,
+                # the reference's bytes for the same traversal (an fp32 row per evaluation), over the same time
+                "algorithmic_gbps": alg_bytes / avg_kernel / 1e9,
+                "algorithmic_frac": alg_bytes / avg_kernel / 1e9 / HBM_PEAK_GBPS,
+                "algorithmic_bytes_per_launch": alg_bytes,
                 "expansions_per_query": st.expansions / Q, "dist_evals_per_query": st.dist_evals / Q,
-                "hops_per_query": st.hops / Q, "rounds_per_query": st.rounds / Q, "spills": st.spills}
+                "screened_rows_per_query": st.screened_rows / Q, "exact_rows_per_query": st.exact_rows / Q,
+                "hops_per_query": st.hops / Q, "rounds_per_query": st.rounds / Q, "spills": st.spills,
+                "plan": plan.as_dict()}
 
     def operating_point(self, policy, Q=None, first=512):
         """The smallest multiple of L_STEP at which recall@k of the first Q queries reaches RECALL_TARGET: doubling
@@ -152,8 +182,8 @@ class Bench:
         return hi, probes
 
 
-def slim(r, keys=("L", "queries", "qps", "recall", "kernel_ms", "gbps", "frac", "dist_evals_per_query",
-                  "expansions_per_query", "spills")):
+def slim(r, keys=("L", "queries", "qps", "recall", "kernel_ms", "gbps", "frac", "algorithmic_frac",
+                  "dist_evals_per_query", "exact_rows_per_query", "expansions_per_query", "spills")):
     return {k2: r[k2] for k2 in keys if k2 in r}
 
 
@@ -421,6 +451,11 @@ def main():
         "config": {"workload": w["name"], "L": head["L"], "k": k, "policy": args.policy,
                    "recall@100": head["recall"], "recall_met": recall_met,
                    "qps_at_config_L": head["qps"], "workgroups": args.workgroups if args.L else 0,
+                   "screening": head["plan"]["screening"], "visited": head["plan"]["visited_form"],
+                   "launch": head["plan"],
+                   "graph_is": "built by the library from the auxiliary queries with top_hit_num = 0 (the code's default, "
+                               "src/index_gpu.cpp:78): no second enhancement pass; the graph of the shipped "
+                               "config.json (top_hit_num = 5000000) is the leg 'shipped_config_graph'",
                    "note": "L is the smallest multiple of %d whose recall@100 over the whole batch is >= %.2f on this "
                            "workload (isotropic 200-d Gaussian base: a degree-32 graph needs a beam this long); the "
                            "configuration's own L = 256 and 512 are under 'also'" % (L_STEP, RECALL_TARGET),
@@ -429,12 +464,29 @@ def main():
         "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": head["frac"], "traffic": traffic["bytes"] if traffic else None,
                      "traffic_record": traffic,
-                     "achieved_is": "algorithmic bytes per launch / average kernel duration (HIP events)",
+                     "achieved_is": "bytes the kernel asked for per launch / average kernel duration (HIP events on "
+                                    "the launch's stream): per query E graph rows x 128 B + S screened rows x "
+                                    "screen_row_bytes + X fp32 rows x dim x 4 B + the query + the ids and counters "
+                                    "written, with E, S, X counted by the kernel itself",
                      "kernel": head_kernel, "kernel_ms": head["kernel_ms"],
-                     "algorithmic_bytes_per_launch": head["bytes_per_launch"],
+                     "bytes_per_launch": head["bytes_per_launch"],
+                     "screen_row_bytes": head["plan"]["screen_row_bytes"],
                      "expansions_per_query": head["expansions_per_query"],
-                     "dist_evals_per_query": head["dist_evals_per_query"]},
+                     "dist_evals_per_query": head["dist_evals_per_query"],
+                     "screened_rows_per_query": head["screened_rows_per_query"],
+                     "exact_rows_per_query": head["exact_rows_per_query"],
+                     "scratch_bytes_per_launch": head["scratch_bytes_per_launch"],
+                     "frac_with_scratch": head["frac_with_scratch"],
+                     "scratch_is": "passes over the beam in global memory (words counted by the kernel) + visited-"
+                                   "state requests x 32 B; mostly served by L2, no part of 'achieved'",
+                     "algorithmic": {"achieved": head["algorithmic_gbps"], "frac": head["algorithmic_frac"],
+                                     "bytes_per_launch": head["algorithmic_bytes_per_launch"],
+                                     "is": "the reference kernel's bytes for the same traversal: an fp32 row per "
+                                           "distance evaluation, a 128-byte graph row per expansion; the screening "
+                                           "reads fewer, so this can exceed the peak"}},
     }
+    if traffic:
+        out["roofline"]["traffic_over_bytes"] = traffic["bytes"] / head["bytes_per_launch"]
     if also:
         out["also"] = also
 
@@ -447,11 +499,9 @@ def main():
         out["roofline"]["gather_peak_is"] = "coral_membench: %d-byte rows from random places of 8 GiB, GB/s" % (dim * 4)
         out["roofline"]["frac_of_practical_peak"] = head["gbps"] / mem[0]
         out["roofline"]["note"] = (
-            "achieved counts the bytes the algorithm asks for (an 800-byte row per distance evaluation, a 128-byte "
-            "row per expansion); the kernel settles most rows on a 256-byte copy in eight-bit codes and reads the "
-            "800-byte row only where rigorous bounds cannot decide, so it moves fewer bytes than it is priced at "
-            "(traffic) and achieved can exceed gather_peak and the HBM peak; part of the rows is served by L2 and "
-            "the 256 MB memory-side cache")
+            "achieved counts the rows the kernel requested (most evaluations are settled on the 256-byte coded row; "
+            "the 800-byte fp32 row is read only where rigorous bounds cannot decide); rows served by L2 or the "
+            "256 MB memory-side cache never reach HBM, so traffic can be below it")
         for rb in (256, 512):  # the rows of the screening: eight-bit codes, half precision (dim 200)
             m2 = optional(capi.membench, 8 << 30, rb, 3)
             if m2 and not isinstance(m2, dict):

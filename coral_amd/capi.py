@@ -33,10 +33,30 @@ class IndexDesc(C.Structure):
 
 class Stats(C.Structure):
     _fields_ = [("time_s", C.c_double), ("kernel_s", C.c_double), ("hops", C.c_int64), ("expansions", C.c_int64),
-                ("dist_evals", C.c_int64), ("rounds", C.c_int64), ("spills", C.c_int64)]
+                ("dist_evals", C.c_int64), ("rounds", C.c_int64), ("spills", C.c_int64),
+                ("screened_rows", C.c_int64), ("exact_rows", C.c_int64), ("beam_words", C.c_int64),
+                ("visited_requests", C.c_int64)]
 
     def as_dict(self):
         return {f: getattr(self, f) for f, _ in self._fields_}
+
+
+class PlanInfo(C.Structure):
+    _fields_ = [("kernel", C.c_int32), ("threads", C.c_int32), ("workgroups", C.c_int32), ("lds_bytes", C.c_int32),
+                ("screening", C.c_int32), ("screen_row_bytes", C.c_int32), ("visited_form", C.c_int32),
+                ("visited_slots_log2", C.c_int32), ("beam_in_hbm", C.c_int32), ("todo_cap", C.c_int32),
+                ("cand_cap", C.c_int32), ("query_slots", C.c_int32), ("reserved", C.c_int32 * 4)]
+
+    KERNELS = ("beam_search_kernel", "best_first_wave_kernel", "best_first_long_kernel")
+    SCREENING = ("none", "fp16", "int8")
+    VISITED = ("lds_table16+hbm_bitmap", "lds_bitmap", "hbm_bytes", "hbm_packed_words", "lds_table16+hbm_state")
+
+    def as_dict(self):
+        d = {f: getattr(self, f) for f, _ in self._fields_ if f != "reserved"}
+        d["kernel"] = self.KERNELS[self.kernel]
+        d["screening"] = self.SCREENING[self.screening]
+        d["visited_form"] = self.VISITED[self.visited_form]
+        return d
 
 
 class Tuning(C.Structure):
@@ -94,6 +114,8 @@ SIGNATURES = {
     "coral_search_gpu_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                            C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "coral_search_query_counters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
+    "coral_search_row_counters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
+    "coral_search_plan_info": (C.c_int, [C.c_void_p, C.POINTER(PlanInfo)]),
     "coral_search": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(Stats)]),
     "coral_search_verify": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
@@ -249,6 +271,18 @@ class Index:
         out = np.empty((Q, 4), dtype=np.int32)
         _check(lib().coral_search_query_counters(self._h, _ptr(out), Q))
         return out
+
+    def row_counters(self, Q):
+        """int32 [Q][4] of the last search: rows measured on the smaller copy, fp32 rows read, words of beam state
+        moved in global memory, visited-state requests to global memory."""
+        out = np.empty((Q, 4), dtype=np.int32)
+        _check(lib().coral_search_row_counters(self._h, _ptr(out), Q))
+        return out
+
+    def plan_info(self):
+        p = PlanInfo()
+        _check(lib().coral_search_plan_info(self._h, C.byref(p)))
+        return p
 
     def bruteforce(self, queries, k, have_delete=False, want_dists=True):
         """Exact kNN of host queries among the index's vectors: (ids, dists, seconds)."""

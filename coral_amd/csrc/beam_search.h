@@ -17,7 +17,9 @@ struct SearchArgs {
     const float* queries;      // [Q][dim]
     int32_t* ids_out;          // [Q][k]
     float* dists_out;          // [Q][k] or nullptr
-    int32_t* counters;         // [Q][4]: hops, expansions, dist_evals, rounds
+    int32_t* counters;         // [2 Q][4]: per query hops, expansions, dist_evals, rounds; then, behind those of all Q
+                               // queries, what each read: rows measured on the smaller copy, fp32 rows, 32-bit words
+                               // of beam state moved in global memory, visited-state requests to global memory
     uint32_t* spill;           // [workgroups][spill_words] zeroed bitmaps
     int* next_qid;             // work counter, zero at launch
     int* spill_count;          // queries that left LDS, zero at launch
@@ -155,14 +157,14 @@ hipError_t launch_search(const SearchArgs& a, bool big, int workgroups, int thre
                          hipStream_t stream);
 
 // A fixed block of device memory inside the library's code object (no allocation call ever made for it): the
-// scratch of the entry point that must not allocate.  Layout: 256 bytes of scalars, kStaticMaxQ x 4 per-query
+// scratch of the entry point that must not allocate.  Layout: 256 bytes of scalars, kStaticMaxQ x 8 per-query
 // counters, kStaticSpillWords words of per-workgroup overflow bitmaps.  static_scratch_init(device) looks the
 // block's address up once per device (that device must be current) and static_scratch(device) returns it, or
 // nullptr before that.
 constexpr int kStaticMaxQ = 16384;
 constexpr size_t kStaticSpillWords = (size_t)8 << 20;  // 32 MiB
 constexpr int64_t kStaticMaxN = (int64_t)1 << 22;      // leaves at least 64 workgroups a bitmap each
-constexpr size_t kStaticScratchBytes = 256 + (size_t)kStaticMaxQ * 16 + kStaticSpillWords * 4;
+constexpr size_t kStaticScratchBytes = 256 + (size_t)kStaticMaxQ * 32 + kStaticSpillWords * 4;
 hipError_t static_scratch_init(int device);
 void* static_scratch(int device);
 hipError_t launch_verify(const int32_t* res, const int32_t* gt, unsigned long long* hit, int Q, int k,

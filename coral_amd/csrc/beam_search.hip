@@ -30,6 +30,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "beam_search.h"
 #include "search_device.h"
 
@@ -169,6 +173,9 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
 
     __shared__ int s_qid, s_ntodo, s_ntodo2, s_ncand, s_nexp, s_cntf, s_cursor, s_nover;
     __shared__ int s_wcnt[16];
+    // what the query read, by class (thread 0 alone adds to these and writes them out): rows measured on the smaller
+    // copy, fp32 rows, words of a beam in global memory
+    __shared__ int s_rows_screened, s_rows_exact, s_beam_words;
     __shared__ float s_qq, s_qscale, s_qerr;  // of the query in integer codes: |q~|^2, its scale, |q - q~| rounded up
 
     VisitedSet vs;
@@ -196,6 +203,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         for (int i = tid; i < a.table_words; i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
         if (tid == 0) s_ncand = 0, s_cntf = 0, s_nover = 0, s_cursor = 0, s_ntodo2 = 0;
+        if (tid == 0) s_rows_screened = 0, s_rows_exact = 0, s_beam_words = 0;
         __syncthreads();
 
         float4 qreg[CPL];
@@ -230,8 +238,9 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         // Most ids a long search measures fail the round's frozen threshold.  Each row is first measured in its
         // half-precision copy (half the bytes; 512-byte rows that start on a cache line).  From that distance d16, the
         // norm of the row |x| (stored behind it) and the rounding bound of the format, |x - half(x)| <= 2^-11 |x|,
-        // the exact distance d lies in [(sqrt(d16) - r)^2, (sqrt(d16) + r)^2], r = 2^-11 |x| (taken a little larger,
-        // and both ends widened by 1e-4 to cover the fp32 rounding of either computation).  A row whose whole
+        // the exact distance d lies in [(sqrt(d16) - r)^2, (sqrt(d16) + r)^2], r = 2^-11 |x| + sqrt(dim) 2^-25 (the second
+        // term for components below the format's normal range; both taken a little larger, and both ends widened by
+        // 1e-4 to cover the fp32 rounding of either computation).  A row whose whole
         // interval lies beyond the frozen threshold is no candidate whatever its exact distance; one whose interval
         // lies below the threshold and beyond the beam's current worst entry is a candidate that is counted and
         // cannot enter the beam.  Only the rest -- possible beam entries and rows within 0.1 % of the threshold --
@@ -250,6 +259,10 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     qa[t][1] = c + 1 < chunks ? reinterpret_cast<const float4*>(qs)[c + 1] : make_float4(0, 0, 0, 0);
                 }
                 const float s_live = st.live == kKeyMax ? 3.402823466e+38f : key_s(st.live);
+                // |x - half(x)| <= 2^-11 |x| holds for components that are normal numbers in half precision; one
+                // below 6.1e-5 is rounded to a multiple of 2^-24, an absolute error of up to 2^-25: sqrt(dim) 2^-25
+                // over a row
+                const float r_abs = 1.0e-6f + 3.0e-8f * sqrtf((float)(chunksH * 8));
                 int cnt = 0;
                 for (int base = wave * RPIH; base < T; base += NW * RPIH) {
                     int vid[U];
@@ -313,7 +326,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     for (int u = 1; u < U; ++u)
                         if ((lane & (U - 1)) == u) mine = acc[u];
                     mine = mine + __shfl_xor(mine, 16, 64);
-                    const float root = sqrtf(mine), r = 5.0e-4f * nx + 1.0e-6f;
+                    const float root = sqrtf(mine), r = 5.0e-4f * nx + r_abs;
                     const float lo_root = fmaxf(root - r, 0.0f), hi_root = root + r;
                     const float lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
                     // (a row with a component beyond the half format has an infinite norm: lo = 0, hi = inf)
@@ -488,6 +501,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 st.cur ^= 1;
                 st.live = st.nb == L ? dst[L - 1] : kKeyMax;
                 if (tid == 0) s_ncand = 0;
+                if (BIG && tid == 0) s_beam_words += 2 * (nb + st.nb);  // one pass: nb keys read, st.nb written
                 ncand_u = 0;
                 __syncthreads();
                 return;
@@ -650,6 +664,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             st.cur ^= 1;
             st.live = st.nb == L ? dst[L - 1] : kKeyMax;
             if (tid == 0) s_ncand = 0;
+            if (BIG && tid == 0) s_beam_words += 2 * (nb + st.nb);  // one pass: nb keys read, st.nb written
             ncand_u = 0;
             __syncthreads();
         };
@@ -664,7 +679,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             PHASE_MARK(5);
             distance_phase(todo2, n2);
             __syncthreads();
-            if (tid == 0) s_ntodo2 = 0;
+            if (tid == 0) s_ntodo2 = 0, s_rows_exact += n2;
             ncand_u = s_ncand, ntodo2_u = 0;  // (the next additions to either lie behind the barrier below)
             __syncthreads();
             PHASE_MARK(4);
@@ -687,6 +702,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     screening_phase(todo + off, n);
                 __syncthreads();
                 ntodo2_u = s_ntodo2;
+                if (tid == 0) s_rows_screened += n;
                 PHASE_MARK(7);
                 off += n;
                 if (off < T) __syncthreads();  // every thread has the count before the next piece adds to it
@@ -705,7 +721,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         distance_phase(todo, M);
         merge();
         PHASE_MARK(1);
-        if (tid == 0) s_cntf = 0;
+        if (tid == 0) s_cntf = 0, s_rows_exact += M;
         nd = M, nvis = M;
         if (a.policy == 1) hops = M;
 
@@ -760,6 +776,8 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             }
             __syncthreads();
             const int nexp = s_nexp;
+            // (rounds: the scan read the beam's nb0 keys and flagged nexp of them; the expand list is written, then read)
+            if (BIG && tid == 0) s_beam_words += (a.policy == 0 ? 2 * nb0 : 128) + 4 * nexp;
             PHASE_MARK(2);
             if (nexp == 0) {
                 // a round that finds every entry expanded still counts: the candidates of the round that first
@@ -838,6 +856,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                 } else {
                     distance_phase(todo, T);
                     __syncthreads();
+                    if (tid == 0) s_rows_exact += T;
                     ncand_u = s_ncand;  // (the next chunk's additions lie behind the barrier at its start)
                 }
                 PHASE_MARK(4);
@@ -910,6 +929,11 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
             if (tid == 0) {
                 int32_t* c = a.counters + (size_t)qid * 4;
                 c[0] = hops, c[1] = ne, c[2] = nd, c[3] = rounds;
+                {
+                    int32_t* rc = a.counters + ((size_t)a.Q + qid) * 4;
+                    // (ids sent to the bitmap in global memory: one atomic each; the clean-up writes them once more)
+                    rc[0] = s_rows_screened, rc[1] = s_rows_exact, rc[2] = s_beam_words, rc[3] = 2 * s_nover;
+                }
                 if (s_nover > 0) atomicAdd(a.spill_count, 1);
             }
             // leave the global bitmap clean: word by word from the list, or all of it
@@ -992,9 +1016,23 @@ size_t search_beam_stride(int L) {
 hipError_t search_kernel_prepare(int dim, bool big, size_t lds_bytes, int threads, int* max_wg_per_cu) {
     kernel_fn fn = pick_kernel(dim, big);
     if (!fn) return hipErrorInvalidValue;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    // The limit on a kernel's dynamic LDS is only ever raised: a launch planned earlier (the entry point that
+    // allocates nothing keeps its plan) must stay valid after a later plan for a shorter beam.
+    static std::mutex mu;
+    static std::map<std::pair<const void*, int>, size_t> limit;
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
     if (e != hipSuccess) return e;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        size_t& have = limit[{reinterpret_cast<const void*>(fn), device}];
+        if (lds_bytes > have) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds_bytes);
+            if (e != hipSuccess) return e;
+            have = lds_bytes;
+        }
+    }
     int nb = 0;
     e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, reinterpret_cast<const void*>(fn), threads,
                                                      lds_bytes);

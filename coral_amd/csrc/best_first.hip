@@ -202,6 +202,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
         int nb = 0, cursor = 0;
         uint64_t live = kKeyMax;
         int hops = M, nd = M, ne = 0, rounds = 0;
+        int n_screened = 0, n_exact = 0, n_vreq = 0;  // rows measured on the smaller copy, fp32 rows, visited-state requests to HBM
 
         // todo[0..T) -> distances -> the beam
         auto measure_and_merge = [&](int T) {
@@ -286,7 +287,8 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                     for (int u = 1; u < UH; ++u)
                         if ((lane & (UH - 1)) == u) mine = acc[u];
                     mine = mine + __shfl_xor(mine, 16, 64);
-                    const float root = sqrtf(mine), r = 5.0e-4f * nx + 1.0e-6f;
+                    // (2^-11 |x| for components that are normal in half precision, 2^-25 each for smaller ones)
+                    const float root = sqrtf(mine), r = 5.0e-4f * nx + 1.0e-6f + 3.0e-8f * sqrtf((float)(chunksH * 8));
                     const float lo_root = fmaxf(root - r, 0.0f);
                     const float lo = lo_root * lo_root * (1.0f - 1.0e-4f);
                     const bool exact = valid && !(lo > s_live);
@@ -296,6 +298,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 }
                 wave_sync();
                 list = todo2;
+                n_screened += T;
                 T = n2;
             }
             if constexpr (SCREEN == 2 && G == 64 && CPL <= 2) {
@@ -325,9 +328,11 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                     }
                     wave_sync();
                     list = todo2;
+                    n_screened += T;
                     T = n2;
                 }
             }
+            n_exact += T;
             int nc = 0;
             for (int base = 0; base < T; base += RPI) {
                 int vid[U];
@@ -452,6 +457,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 todo[lane] = id;
             }
             any_over = any_over || __ballot(over) != 0ull;
+            n_vreq += __popcll(__ballot(over)) * (PACKED ? 2 : 1);
             wave_sync();
             measure_and_merge(T);
         }
@@ -490,7 +496,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             }
             // the table first; what it has no room for is settled against the state in HBM, which holds nothing
             // before the first id went there, and whose filter knows every id that did
-            bool isnew = false, over = false;
+            bool isnew = false, over = false, tested = false;
             if (v >= 0) {
                 if (tl) {
                     const int r = table_test_and_set((uint32_t)v);
@@ -498,12 +504,17 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
                 } else {
                     over = true;
                 }
-                if (over) isnew = !any_over || (bl && !bloom_may_hold((uint32_t)v)) || unvisited((uint32_t)v);
+                if (over) {
+                    const bool settled = !any_over || (bl && !bloom_may_hold((uint32_t)v));
+                    isnew = settled || unvisited((uint32_t)v);
+                    tested = !settled;
+                }
             }
             if (isnew && over) {
                 mark((uint32_t)v);
                 if (bl) bloom_add((uint32_t)v);
             }
+            n_vreq += __popcll(__ballot(tested)) + __popcll(__ballot(isnew && over)) * (PACKED ? 2 : 1);
             const uint64_t m = __ballot(isnew);
             any_over = any_over || __ballot(isnew && over) != 0ull;
             const int T = __popcll(m);
@@ -556,6 +567,10 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 
             if (lane == 0) {
                 int32_t* c = a.counters + (size_t)qid * 4;
                 c[0] = hops, c[1] = ne, c[2] = nd, c[3] = rounds;
+                {
+                    int32_t* rc = a.counters + ((size_t)a.Q + qid) * 4;
+                    rc[0] = n_screened, rc[1] = n_exact, rc[2] = 0, rc[3] = n_vreq;
+                }
             }
         }
         wave_sync();

@@ -144,12 +144,15 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
         uint64_t wkey = kKeyMax;  // (kKeyMax has its flag set: nothing to expand)
         uint64_t live = kKeyMax;
         int hops = M, nd = M, ne = 0, rounds = 0;
+        // rows measured on the smaller copy, fp32 rows, words of the long run moved, visited-state requests to HBM
+        int n_screened = 0, n_exact = 0, n_words = 0, n_vreq = 0;
 
         // ---- buf into g: one coalesced pass over g, buf's places found through the sample
         auto flush = [&]() {
             if (nbuf == 0) return;
             memory_sync();  // the flags stored into g since the last merge
             const int nn = ng + nbuf;  // <= L
+            n_words += 2 * (ng + nn);  // one pass: ng keys read, nn written
             const int ntb = nn > tcap ? nn - tcap : 0;
             const int ns = ng > 0 ? ((ng - 1) >> ss) + 1 : 0;
             const uint64_t b_lo = buf[0], b_hi = buf[nbuf - 1];
@@ -234,9 +237,11 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                     }
                     wave_sync();
                     list = todo2;
+                    n_screened += T;
                     T = n2;
                 }
             }
+            n_exact += T;
             int nc = 0;
             for (int base = 0; base < T; base += RPI) {
                 int vid[U];
@@ -369,6 +374,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
                 mark(id);
                 todo[lane] = id;
             }
+            n_vreq += T * (PACKED ? 2 : 1);
             wave_sync();
             measure_and_merge(T);
         }
@@ -437,6 +443,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             const int T = __popcll(m);
             if (isnew) todo[prefix_popc(m)] = (uint32_t)v;
             nd += T;
+            n_vreq += __popcll(__ballot(v >= 0)) + T * (PACKED ? 2 : 1);  // a test per listed id, a mark per first visit
             wave_sync();
             measure_and_merge(T);
             // the tags written in this step are read by later steps through other lanes (see best_first.hip)
@@ -482,6 +489,10 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
             if (lane == 0) {
                 int32_t* c = a.counters + (size_t)qid * 4;
                 c[0] = hops, c[1] = ne, c[2] = nd, c[3] = rounds;
+                {
+                    int32_t* rc = a.counters + ((size_t)a.Q + qid) * 4;
+                    rc[0] = n_screened, rc[1] = n_exact, rc[2] = n_words, rc[3] = n_vreq;
+                }
             }
         }
         wave_sync();

@@ -39,6 +39,7 @@ using coral::fail;
 
 constexpr int kMaxL = CORAL_MAX_BEAM;  // beams beyond CORAL_MAX_LDS_BEAM live in global memory
 constexpr int kMaxLdsBytes = 160 * 1024;
+constexpr int kStaticLds = 128;  // what the workgroup kernel declares outside its dynamic block (counts, per-wave sums)
 constexpr int kLongBeamFrom = 1280;  // best-first: beams longer than this take the long-beam kernel
 
 // bits of a mixed id that a cell of the wavefront kernel's table stores: what the bucket index (a quarter of the
@@ -71,6 +72,18 @@ int choose_bf_table(int L, int id_bits, int wanted, int* table_log2) {
 }
 
 }  // namespace
+
+// Before a buffer that a search kernel reads is freed or rewritten: wait for the index's own stream and, if the entry
+// point that returns without waiting has been used, for everything on the device (its launches run on streams of the
+// caller's choosing).
+static hipError_t quiesce(coral_index* idx) {
+    hipError_t e = idx->stream ? hipStreamSynchronize(idx->stream) : hipSuccess;
+    if (e == hipSuccess && idx->noalloc_in_flight) {
+        e = hipDeviceSynchronize();
+        idx->noalloc_in_flight = false;
+    }
+    return e;
+}
 
 extern "C" {
 
@@ -176,7 +189,7 @@ int coral_index_create(const coral_index_desc* d, coral_index** out) {
 void coral_index_destroy(coral_index* idx) {
     if (!idx) return;
     (void)hipSetDevice(idx->device);
-    if (idx->stream) (void)hipStreamSynchronize(idx->stream);
+    (void)quiesce(idx);
     (void)hipFree(idx->d_vec);
     (void)hipFree(idx->d_nbrs);
     (void)hipFree(idx->d_start);
@@ -211,7 +224,8 @@ int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const int32_t* 
     if (!idx->d_nbrs) return fail(CORAL_ERR_STATE, "the index holds vectors only (no graph was given)");
     if (int rc = validate_graph(nbrs, idx->n, idx->R, start_ids, n_start)) return rc;
     HIP_TRY(hipSetDevice(idx->device));
-    HIP_TRY(hipStreamSynchronize(idx->stream));
+    HIP_TRY(quiesce(idx));
+    idx->noalloc_L = 0;  // (a plan depends on the number of start ids)
     if (n_start != idx->M) {
         int32_t* p = nullptr;
         HIP_TRY(hipMalloc(&p, (size_t)n_start * sizeof(int32_t)));
@@ -231,7 +245,7 @@ int coral_index_set_graph(coral_index* idx, const int32_t* nbrs, const int32_t* 
 int coral_index_set_deleted(coral_index* idx, const uint32_t* host_mask) {
     if (!idx) return fail(CORAL_ERR_ARG, "null index");
     HIP_TRY(hipSetDevice(idx->device));
-    HIP_TRY(hipStreamSynchronize(idx->stream));
+    HIP_TRY(quiesce(idx));
     if (!host_mask) {
         (void)hipFree(idx->d_deleted);
         idx->d_deleted = nullptr;
@@ -300,10 +314,10 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     // a million nodes, which leaves a CU one workgroup.
     const int bitmap_words = (int)(((idx->n + 31) / 32 + 3) & ~(int64_t)3);
     auto lds_bitmap = [&](bool big, int cap) {
-        return coral::search_lds_bytes(L, idx->dim, bitmap_words, cap, cap, 4, big, screen) + 64;
+        return coral::search_lds_bytes(L, idx->dim, bitmap_words, cap, cap, 4, big, screen) + kStaticLds;
     };
     auto lds_table = [&](bool big, int lg, int cap) {
-        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, 256, big, screen) + 64;
+        return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, 256, big, screen) + kStaticLds;
     };
     const bool bitmap_possible = idx->n <= ((int64_t)1 << 21);
     int slots_log2 = t.visited_slots_log2;
@@ -359,7 +373,7 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     // hold; a launch that is alone on its CU anyway takes a candidate buffer of twice the size where there is room
     // (half as many merges of a long beam).  Best-first expands one row at a time and needs neither.
     auto lds_for = [&](int tc, int cc) {
-        return coral::search_lds_bytes(L, idx->dim, p.table_words, tc, cc, ocap, p.big, screen) + 64;
+        return coral::search_lds_bytes(L, idx->dim, p.table_words, tc, cc, ocap, p.big, screen) + kStaticLds;
     };
     if (lds_for(min_cap, min_cap) > lds_max)
         return fail(CORAL_ERR_ARG, "L=%d with %d words of visited state needs %zu bytes of LDS", L, p.table_words,
@@ -498,7 +512,8 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         HIP_TRY(hipMalloc(&idx->d_beam, need_beam * sizeof(uint64_t)));
         idx->beam_alloc_words = need_beam;
     }
-    const size_t need_counters = (size_t)Q * 4;
+    // per query: the four traversal counters, then (behind those of the whole batch) the four counts of what it read
+    const size_t need_counters = (size_t)Q * 8;
     if (need_counters > idx->counters_alloc) {
         (void)hipFree(idx->d_counters);
         if (idx->h_counters) (void)hipHostFree(idx->h_counters);
@@ -742,7 +757,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
         HIP_TRY(coral::launch_search(a, plan.big, wgs, plan.threads, plan.lds_bytes, stream));
     }
     HIP_TRY(hipEventRecord(evk, stream));
-    HIP_TRY(hipMemcpyAsync(idx->h_counters, idx->d_counters, (size_t)Q * 4 * sizeof(int32_t),
+    HIP_TRY(hipMemcpyAsync(idx->h_counters, idx->d_counters, (size_t)Q * 8 * sizeof(int32_t),
                            hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipEventRecord(ev1, stream));
     HIP_TRY(hipEventSynchronize(ev1));
@@ -787,6 +802,9 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
             const int32_t* c = idx->h_counters + (size_t)q * 4;
             stats->hops += c[0], stats->expansions += c[1];
             stats->dist_evals += c[2], stats->rounds += c[3];
+            const int32_t* r = idx->h_counters + (size_t)Q * 4 + (size_t)q * 4;
+            stats->screened_rows += r[0], stats->exact_rows += r[1];
+            stats->beam_words += r[2], stats->visited_requests += r[3];
         }
         stats->spills = scal[1];
     }
@@ -822,12 +840,19 @@ int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* 
     t.screening = rounds && idx->d_vec8 && idx->dim / 4 > 16                            ? 2
                   : rounds && idx->d_vec16 && idx->dim / 4 > 32 && idx->metric == CORAL_L2 ? 1
                                                                                            : -1;
-    coral_search_plan plan;
-    if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, /*no_screen*/ t.screening < 0, &plan)) return rc;
+    // the launch geometry (kernel attributes, an occupancy query) is worked out on the first call with these
+    // arguments and kept: later calls only fill two buffers and launch
+    if (idx->noalloc_Q != Q || idx->noalloc_L != L || idx->noalloc_policy != policy || idx->noalloc_screen != t.screening) {
+        idx->noalloc_L = 0;
+        if (int rc = plan_search(idx, Q, L, t, 0, /*lds_beam_only*/ true, /*no_screen*/ t.screening < 0, &idx->noalloc_plan))
+            return rc;
+        idx->noalloc_Q = Q, idx->noalloc_L = L, idx->noalloc_policy = policy, idx->noalloc_screen = t.screening;
+    }
+    const coral_search_plan& plan = idx->noalloc_plan;
     // the block: 256 bytes of scalars, the per-query counters, then one overflow bitmap per workgroup
     int* scal = reinterpret_cast<int*>(base);
     int32_t* counters = reinterpret_cast<int32_t*>(base + 256);
-    uint32_t* spill = reinterpret_cast<uint32_t*>(base + 256 + (size_t)coral::kStaticMaxQ * 16);
+    uint32_t* spill = reinterpret_cast<uint32_t*>(base + 256 + (size_t)coral::kStaticMaxQ * 32);
     int wgs = std::min(plan.workgroups, (int)Q);
     if (plan.spill_words)  // (none when the visited set is a bitmap of all ids in LDS)
         wgs = (int)std::min<size_t>((size_t)wgs, coral::kStaticSpillWords / plan.spill_words);
@@ -838,6 +863,7 @@ int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries, int32_t* 
     coral::SearchArgs a = search_args(idx, plan, d_queries, d_ids, d_dists, Q, k, policy, have_delete);
     a.counters = counters, a.spill = spill, a.beam_scratch = nullptr;
     a.next_qid = scal, a.spill_count = scal + 1;
+    idx->noalloc_in_flight = true;
     HIP_TRY(coral::launch_search(a, false, wgs, plan.threads, plan.lds_bytes, stream));
     return CORAL_OK;
 }
@@ -846,6 +872,51 @@ int coral_search_query_counters(coral_index* idx, int32_t* host_out, int32_t Q) 
     if (!idx || !host_out) return fail(CORAL_ERR_ARG, "null argument");
     if (Q <= 0 || Q > idx->last_Q) return fail(CORAL_ERR_ARG, "no counters for %d queries", Q);
     std::memcpy(host_out, idx->h_counters, (size_t)Q * 4 * sizeof(int32_t));
+    return CORAL_OK;
+}
+
+int coral_search_row_counters(coral_index* idx, int32_t* host_out, int32_t Q) {
+    if (!idx || !host_out) return fail(CORAL_ERR_ARG, "null argument");
+    if (Q <= 0 || Q > idx->last_Q) return fail(CORAL_ERR_ARG, "no counters for %d queries", Q);
+    std::memcpy(host_out, idx->h_counters + (size_t)idx->last_Q * 4, (size_t)Q * 4 * sizeof(int32_t));
+    return CORAL_OK;
+}
+
+int coral_search_plan_info(const coral_index* idx, coral_plan_info* out) {
+    if (!idx || !out) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->prepared) return fail(CORAL_ERR_STATE, "coral_search_prepare has not been called");
+    std::memset(out, 0, sizeof *out);
+    const coral_search_plan& p = idx->plan;
+    const bool wave = idx->prepared_policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready;
+    if (wave) {
+        out->kernel = idx->bf_long ? 2 : 1;
+        out->threads = 256;
+        out->query_slots = std::min(idx->bf_slots, idx->Q);
+        out->workgroups = (out->query_slots + 3) / 4;
+        const size_t per_wave =
+            idx->bf_long
+                ? coral::best_first_long_lds_bytes(idx->bf_bcap, idx->bf_scap,
+                                                   idx->bf_screen == 2 ? coral::best_first_long_coded_bytes(idx->dim) : 0)
+                : coral::best_first_wave_lds_bytes(idx->L, idx->bf_bloom_log2, idx->bf_table_log2,
+                                                   idx->bf_screen == 2 ? coral::coded_query_bytes(idx->dim) : 0);
+        out->lds_bytes = (int32_t)(per_wave * 4);
+        out->screening = idx->bf_screen;
+        out->visited_form = !idx->bf_long && idx->bf_table_log2 ? 4 : idx->bf_packed ? 3 : 2;
+        out->visited_slots_log2 = idx->bf_long ? 0 : idx->bf_table_log2;
+        out->beam_in_hbm = idx->bf_long;
+    } else {
+        out->kernel = 0;
+        out->threads = p.threads, out->workgroups = p.workgroups, out->lds_bytes = (int32_t)p.lds_bytes;
+        out->screening = p.screen;
+        out->visited_form = p.direct ? 1 : 0;
+        out->visited_slots_log2 = p.direct ? 0 : p.slots_log2;
+        out->beam_in_hbm = p.big;
+        out->todo_cap = p.tcap, out->cand_cap = p.ccap;
+        out->query_slots = p.workgroups;
+    }
+    out->screen_row_bytes = out->screening == 2   ? (int32_t)coral::byte_row_stride(idx->dim)
+                            : out->screening == 1 ? (int32_t)coral::half_row_stride(idx->dim)
+                                                  : 0;
     return CORAL_OK;
 }
 

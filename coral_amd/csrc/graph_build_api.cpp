@@ -52,6 +52,7 @@ int set_start_ids(coral_index* idx, const int32_t* all_ids, int count) {
         idx->d_start = p;
         idx->M = M;
         idx->prepared = false;
+        idx->noalloc_L = 0;  // (launch plans depend on the number of start ids)
     }
     HIP_TRY(hipMemcpyAsync(idx->d_start, ids, (size_t)M * sizeof(int32_t), hipMemcpyHostToDevice, idx->stream));
     HIP_TRY(hipStreamSynchronize(idx->stream));

@@ -60,6 +60,11 @@ struct coral_index {
     unsigned long long* d_phase = nullptr;  // debug builds only
     int32_t* h_counters = nullptr;  // pinned, counters_alloc entries
     int last_Q = 0;
+    // the entry point that allocates nothing: its last plan (kernel attributes and occupancy are looked up once per
+    // (Q, L, policy, screening form)), and whether a launch of it may still be in flight on a stream of the caller's
+    coral_search_plan noalloc_plan;
+    int noalloc_Q = 0, noalloc_L = 0, noalloc_policy = -1, noalloc_screen = -2;
+    bool noalloc_in_flight = false;
     hipEvent_t ev[3] = {nullptr, nullptr, nullptr};  // start, kernel end, read-back end of a search
     // device staging of the host-buffer entry point (grow-only)
     float* d_io_q = nullptr;

@@ -87,6 +87,12 @@ typedef struct {
     int64_t dist_evals;  /* vector rows read (first visits + start ids) */
     int64_t rounds;      /* merge rounds (ROUNDS) or expansion steps (BEST_FIRST) */
     int64_t spills;      /* queries whose visited set outgrew LDS */
+    /* what the launch read, by class (the sums of coral_search_row_counters): */
+    int64_t screened_rows;  /* rows measured on the smaller copy of the vectors (codes or half precision) */
+    int64_t exact_rows;     /* fp32 vector rows read: dist_evals without screening, a fraction of them with it */
+    int64_t beam_words;     /* 32-bit words of beam state (keys, expand lists, long runs) read or written in global
+                               memory by passes over a beam that does not live in LDS */
+    int64_t visited_requests; /* tests and marks of the visited state that went to global memory */
 } coral_stats;
 
 /* Optional launch tuning; zero-initialise for defaults. */
@@ -186,7 +192,7 @@ CORAL_API int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t
  * harnesses that forbid hipMalloc).  No counterpart in the reference, whose search allocates on every call
  * (src/index_gpu.cpp:120-124, src/search_gpu.cu:846-852).  No coral_search_prepare is needed and none of its
  * scratch is used: the work counter, the per-query counters and the per-workgroup overflow bitmaps live in a fixed
- * 32.3 MiB block of device memory inside the library's code object (each GPU that loads the library holds its
+ * 32.5 MiB block of device memory inside the library's code object (each GPU that loads the library holds its
  * copy until the process ends).  The call makes no allocation of any kind, records only kernels on `stream`
  * (NULL = the index's own) and returns without waiting for them; both policies run on the workgroup-per-query
  * kernel, with the results of coral_search_gpu bit for bit.  Rows are screened on a smaller copy of the vectors
@@ -200,6 +206,32 @@ CORAL_API int coral_search_gpu_noalloc(coral_index* idx, const float* d_queries,
 /* Per-query counters of the last coral_search_gpu call, int32 [Q][4] on the
  * host: hops, expansions, dist_evals, rounds. */
 CORAL_API int coral_search_query_counters(coral_index* idx, int32_t* host_out, int32_t Q);
+
+/* What the last coral_search_gpu call read per query, by class, int32 [Q][4] on the host: rows measured on the
+ * smaller copy of the vectors, fp32 vector rows read, 32-bit words of beam state moved in global memory, visited-state
+ * requests to global memory.  Every distance evaluation reads one row of one or both kinds: screened_rows +
+ * exact_rows >= dist_evals >= exact_rows.  No counterpart in the reference (which reads the fp32 row for every
+ * evaluation, include/utils.cuh:254-275); these counts price the launch's memory traffic. */
+CORAL_API int coral_search_row_counters(coral_index* idx, int32_t* host_out, int32_t Q);
+
+/* The launch geometry the last coral_search_prepare chose (what a search call on this index runs with). */
+typedef struct {
+    int32_t kernel;          /* 0 beam_search_kernel (workgroup per query), 1 best_first_wave_kernel, 2 best_first_long_kernel */
+    int32_t threads;         /* per workgroup */
+    int32_t workgroups;      /* persistent workgroups (the wavefront kernels: query slots / 4) */
+    int32_t lds_bytes;       /* per workgroup */
+    int32_t screening;       /* 0 none, 1 half precision, 2 eight-bit codes */
+    int32_t screen_row_bytes;/* bytes of one row of the smaller copy (0 without screening) */
+    int32_t visited_form;    /* 0 table of 16-bit cells in LDS + bitmap in global memory, 1 bitmap of all ids in LDS,
+                                2 bytes per node and slot in global memory, 3 packed words in global memory,
+                                4 table of 16-bit cells in LDS in front of form 2 or 3 */
+    int32_t visited_slots_log2; /* cells of the LDS table (forms 0 and 4), else 0 */
+    int32_t beam_in_hbm;     /* the beam (or the long run) lives in global memory */
+    int32_t todo_cap, cand_cap; /* LDS list capacities of the workgroup kernel */
+    int32_t query_slots;     /* queries in flight */
+    int32_t reserved[4];
+} coral_plan_info;
+CORAL_API int coral_search_plan_info(const coral_index* idx, coral_plan_info* out);
 
 /* IndexGPU::Search (src/index_gpu.cpp:117-136): host buffers in and out; uploads
  * the queries, prepares for (Q, L), searches, downloads ids (and distances when

@@ -110,7 +110,32 @@ def test_exact_against_same_order_oracle(orc, case):
         assert st.hops == int(os_[:, 0].sum()) and st.dist_evals == int(os_[:, 2].sum())
         if slots == 11 and (policy == 0 or in_lds):
             assert st.spills > 0
+        check_row_counters(idx, st, cnt, M, policy)
     idx.close()
+
+
+def check_row_counters(idx, st, cnt, M, policy):
+    """What the kernels say they read, by class, against the traversal's own counters: every distance evaluation
+    reads its row on the smaller copy, in fp32, or both; without a screening all are fp32 rows; the rounds kernel
+    screens every row but the start ids'."""
+    Q = cnt.shape[0]
+    rc = idx.row_counters(Q)
+    plan = idx.plan_info()
+    assert (rc >= 0).all()
+    assert (rc[:, 1] <= cnt[:, 2]).all() and (rc[:, 0] + rc[:, 1] >= cnt[:, 2]).all()
+    if plan.screening == 0:
+        assert not rc[:, 0].any() and np.array_equal(rc[:, 1], cnt[:, 2])
+    elif policy == 0:
+        assert np.array_equal(rc[:, 0], cnt[:, 2] - M)
+    assert (rc[:, 0] <= cnt[:, 2] - M).all()
+    assert plan.screen_row_bytes % 128 == 0 and (plan.screen_row_bytes > 0) == (plan.screening > 0)
+    assert (st.screened_rows, st.exact_rows, st.beam_words, st.visited_requests) == tuple(int(x) for x in rc.sum(0))
+    if not plan.beam_in_hbm:
+        assert st.beam_words == 0
+    else:
+        assert st.beam_words > 0
+    if plan.kernel != 0 and plan.visited_form in (2, 3):  # every listed id is tested in HBM, every first visit marked
+        assert (rc[:, 3] >= cnt[:, 2]).all()
 
 
 BIG_CASES = [
@@ -189,6 +214,7 @@ def test_beams_in_global_memory_equal_the_oracle(orc, case):
         assert np.array_equal(cnt, os_), form
         if slots and not form.get("best_first_long"):
             assert st.spills > 0
+        check_row_counters(idx, st, cnt, M, policy)
         # the same call again on the used beam blocks and bitmaps
         ids2, dists2, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
         assert np.array_equal(ids2, oi) and dists2.tobytes() == od.tobytes(), form
@@ -201,7 +227,8 @@ def test_beams_in_global_memory_equal_the_oracle(orc, case):
 
 @pytest.mark.parametrize("kind", ["lattice", "large", "beyond_half", "tiny", "dim_not_a_multiple_of_8", "dim_200",
                                   "dim_264", "mixed_magnitudes", "outliers", "tiny_queries", "huge_rows", "ip_unit",
-                                  "ip_raw", "ip_lattice", "ip_mixed_magnitudes", "dim_128", "dim_72", "ip_dim_100"])
+                                  "ip_raw", "ip_lattice", "ip_mixed_magnitudes", "dim_128", "dim_72", "ip_dim_100",
+                                  "half_subnormal_dim_2048"])
 def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     """The rounds kernel measures every row in a smaller copy of the vectors first -- half precision, or eight-bit
     codes with a scale per row -- and reads the fp32 row only where bounds on the exact distance leave the row's fate
@@ -213,11 +240,14 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     in one base (a scale per row), rows with one component a hundred times the others (codes lose the rest), queries
     of 1e-20 (no scale: every row goes to the exact pass), rows of 1e18 (they take no part in the coded copy); and the
     inner-product metric, which is screened on codes only: unit vectors, raw Gaussian rows, a lattice, rows of very
-    different norms.  Ids, distance bits and counters equal the oracle's, with the screening and without."""
+    different norms; rows of 2048 components that sit half-way between two neighbours of the half format's subnormal
+    grid ((m + 1/2) 2^-24), where the rounding error of the copy is absolute, 2^-25 per component, and adds up to
+    sqrt(2048) 2^-25 = 1.35e-6 whatever the row's norm.  Ids, distance bits and counters equal the oracle's, with the screening and without."""
     n, dim, R, Q, L, k = 4000, 136, 24, 100, 200, 50
     dim = {"dim_not_a_multiple_of_8": 140, "dim_200": 200, "dim_264": 264, "ip_raw": 200, "dim_128": 128, "dim_72": 72,
-           "ip_dim_100": 100}.get(kind, dim)
+           "ip_dim_100": 100, "half_subnormal_dim_2048": 2048}.get(kind, dim)
     narrow = dim <= 128  # the rounds kernel screens such rows on codes; half precision and best-first do not
+    wide = dim > 512     # no copy in eight-bit codes for such rows
     ip = kind.startswith("ip_")
     m, mname = (capi.IP, "ip") if ip else (capi.L2, "l2")
     rng = np.random.RandomState(77)
@@ -225,9 +255,12 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
         base = rng.randint(0, 4, (n, dim)).astype(np.float32)
         q = (rng.randint(0, 8, (Q, dim)) * 0.5).astype(np.float32)
     else:
-        scale = {"large": 1.0e4, "beyond_half": 1.0e5, "tiny": 1.0e-6}.get(kind, 1.0)
+        scale = {"large": 1.0e4, "beyond_half": 1.0e5, "tiny": 1.0e-6, "half_subnormal_dim_2048": 2.0e-7}.get(kind, 1.0)
         base = (synth.gaussian_matrix(88, n, dim) * np.float32(scale)).astype(np.float32)
         q = (make_queries(Q, dim, 89) * np.float32(scale)).astype(np.float32)
+        if kind == "half_subnormal_dim_2048":
+            grid = np.float32(2.0 ** -24)
+            base = ((rng.randint(0, 4, (n, dim)) + 0.5) * rng.choice([-1.0, 1.0], (n, dim))).astype(np.float32) * grid
         if kind == "beyond_half":
             base[::7] *= np.float32(1e-3)  # a share of the rows fits the format, the rest does not
         if kind in ("mixed_magnitudes", "ip_mixed_magnitudes"):
@@ -248,7 +281,8 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     for form in (dict(screening=-1), dict(screening=1), dict(screening=1, beam_in_hbm=True),
                  dict(screening=1, visited_slots_log2=12, threads=256), dict(screening=2),
                  dict(screening=2, beam_in_hbm=True), dict(screening=2, visited_slots_log2=12, threads=256), dict()):
-        if (ip or narrow) and form.get("screening") == 1:  # half precision: L2 and more than 128 floats only
+        # half precision: L2 and more than 128 floats only; codes: up to 512 floats
+        if ((ip or narrow) and form.get("screening") == 1) or (wide and form.get("screening") == 2):
             with pytest.raises(capi.CoralError):
                 idx.prepare(Q, L, **form)
             continue
@@ -264,7 +298,8 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
                  dict(screening=2, best_first_packed=True, best_first_table_log2=-1), dict(best_first_table_log2=-1),
                  dict(best_first_long=1), dict(best_first_long=1, screening=-1),
                  dict(best_first_long=1, best_first_buffer=64, best_first_packed=True, screening=2)):
-        if (ip and form.get("screening") == 1) or (narrow and form.get("screening", 0) > 0):
+        if (ip and form.get("screening") == 1) or (narrow and form.get("screening", 0) > 0) or \
+                (wide and form.get("screening") == 2):
             continue
         idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, **form)
         ids, dists, _ = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)

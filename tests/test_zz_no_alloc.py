@@ -1,7 +1,9 @@
 """The entry point that allocates nothing (coral_search_gpu_noalloc: scratch in a fixed block of device memory
 inside the library) against coral_search_gpu on the same inputs: ids and distance bits equal, on two calls in a
 row, the second with a smaller input, for both traversal policies, with tombstones, and on a second index that
-shares the same block; sizes beyond the block are turned away."""
+shares the same block; sizes beyond the block are turned away.  The device's free memory is read around every such
+call: it must not move (the first launch of a kernel in a process aside, where the runtime may set up its own
+per-queue memory)."""
 import numpy as np
 import pytest
 
@@ -20,13 +22,18 @@ def _reference(idx, d_q, Q, k, L, policy, have_delete, torch):
     return ids.cpu().numpy(), dists.cpu().numpy()
 
 
+FREE_MEMORY_MOVED = []  # per coral_search_gpu_noalloc call of this file: free device memory before - after, bytes
+
+
 def _noalloc(idx, d_q, Q, k, L, policy, have_delete, torch):
     ids = torch.full((Q, k), -7, dtype=torch.int32, device="cuda")
     dists = torch.full((Q, k), -7.0, dtype=torch.float32, device="cuda")
     torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
     idx.search_device_noalloc(d_q.data_ptr(), ids.data_ptr(), dists.data_ptr(), Q, k, L, policy=policy,
                               have_delete=have_delete)
     torch.cuda.synchronize()  # the call does not wait for its kernels; the index's stream is a blocking stream
+    FREE_MEMORY_MOVED.append(free_before - torch.cuda.mem_get_info()[0])
     return ids.cpu().numpy(), dists.cpu().numpy()
 
 
@@ -81,9 +88,17 @@ def test_no_alloc_entry_point_equals_the_allocating_one():
     nbrs2 = workloads.exact_knn_graph(base2, 16)
     idx2 = capi.Index(base2, nbrs2, np.array([3, 999], np.int32))
     d_q2 = torch.from_numpy(make_queries(50, dim2, 902)).cuda()
-    got = _noalloc(idx2, d_q2, 50, 20, 100, capi.POLICY_ROUNDS, False, torch)
+    got = _noalloc(idx2, d_q2, 50, 20, 100, capi.POLICY_ROUNDS, False, torch)  # (the first call on a fresh index)
     want = _reference(idx2, d_q2, 50, 20, 100, capi.POLICY_ROUNDS, False, torch)
     assert np.array_equal(got[0], want[0]) and got[1].tobytes() == want[1].tobytes()
+    # no call took device memory: the same call again (its launch plan is kept: nothing but two fills and the launch)
+    # and all the calls above, the first launches of each kernel form in this process reported apart
+    for _ in range(3):
+        again = _noalloc(idx2, d_q2, 50, 20, 100, capi.POLICY_ROUNDS, False, torch)
+        assert np.array_equal(again[0], want[0]) and again[1].tobytes() == want[1].tobytes()
+    print("free device memory moved per call (bytes):", FREE_MEMORY_MOVED, flush=True)
+    assert all(d == 0 for d in FREE_MEMORY_MOVED[-3:])
+    assert sum(1 for d in FREE_MEMORY_MOVED if d != 0) <= 3, FREE_MEMORY_MOVED  # (three kernel forms: dim 200, 8, 64)
     # beyond the block: clear errors, nothing launched
     d_q = torch.from_numpy(q_all[:8]).cuda()
     out = torch.empty((8, 10), dtype=torch.int32, device="cuda")

@@ -40,29 +40,34 @@ def digest(*arrays):
 
 
 def near_tie_equal(ids_a, d_a, ids_b, d_b, rel=1e-6):
-    """True when two result lists are identical except for swaps or substitutions
-    among entries whose distances differ by less than rel * |d|."""
+    """True when two result lists (closest first, same length) are identical except for permutations or substitutions
+    among entries whose distances differ by less than rel * |d|:
+      * where the lists hold different ids at a rank, the two distances at that rank are within rel of each other
+        (the ids that swapped or replaced one another are a near-tie);
+      * an id that both lists hold has the same distance in both up to the summation order (1e-5);
+      * an id that only one list holds is within rel of the other list's last entry (a near-tie decided membership)."""
     if np.array_equal(ids_a, ids_b):
         return True
     k = len(ids_a)
-    if not np.allclose(d_a, d_b, rtol=1e-5, atol=0):
-        return False
-    sa, sb = set(ids_a.tolist()), set(ids_b.tolist())
+
+    def close(x, y, r):
+        return abs(float(x) - float(y)) <= r * max(abs(float(x)), abs(float(y)), 1e-30)
+
     for i in range(k):
         if ids_a[i] == ids_b[i]:
+            if not close(d_a[i], d_b[i], 1e-5):
+                return False
             continue
-        # the entry of a must appear in b at a position of (nearly) the same distance,
-        # or sit at the tail where a near-tie decided membership
-        for x, other_ids, other_d, mine_d in ((ids_a[i], ids_b, d_b, d_a[i]), (ids_b[i], ids_a, d_a, d_b[i])):
+        if not close(d_a[i], d_b[i], rel):
+            return False
+        for x, mine_d, other_ids, other_d in ((ids_a[i], d_a[i], ids_b, d_b), (ids_b[i], d_b[i], ids_a, d_a)):
             pos = np.where(other_ids == x)[0]
             if pos.size:
-                if abs(other_d[pos[0]] - mine_d) > rel * max(abs(mine_d), 1e-30) * 4:
+                if not close(other_d[pos[0]], mine_d, 1e-5):
                     return False
-            else:
-                # membership differs: only acceptable against the last entry's distance
-                if abs(other_d[k - 1] - mine_d) > rel * max(abs(mine_d), 1e-30) * 4:
-                    return False
-    return len(sa ^ sb) <= 2 * k
+            elif not close(other_d[k - 1], mine_d, rel):
+                return False
+    return True
 
 
 def rounds_hand_case():
