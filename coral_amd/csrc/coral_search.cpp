@@ -331,6 +331,10 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         // that overflowed (see coral_search_gpu)
         int want = 12;
         while ((1 << want) < 112 * L && want < 20) ++want;
+        // A 16-bit cell of a 2^s table keeps id_bits - s bits of the id and has the rest for the displacement: beyond
+        // 2^24 ids a table sized for the load alone carries displacements of 14 or fewer, and a few ids of every
+        // query would leave LDS for the bitmap in global memory.  Such launches take the table that carries 30.
+        while (want < 16 && id_bits - want > 11) ++want;
         want += bump_log2;
         const bool table_holds = !p.big && want <= 16 && lds_table(false, want, min_cap) <= lds_max;
         const bool table_alone_on_cu = table_holds && lds_table(false, want, min_cap) > lds_max / 2;
@@ -349,6 +353,7 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         } else {
             slots_log2 = 12;
             while ((1 << slots_log2) < 48 * L && slots_log2 < 16) ++slots_log2;
+            while (slots_log2 < 16 && id_bits - slots_log2 > 11) ++slots_log2;  // (displacements up to 30, as above)
             slots_log2 = std::min(16, slots_log2 + bump_log2);
             while (slots_log2 > 12 && lds_table(p.big, slots_log2, min_cap) > lds_max) --slots_log2;
         }

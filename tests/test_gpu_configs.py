@@ -157,6 +157,8 @@ def test_config2_headline_workload(orc):
 
 # the same for the graph of the reference's shipped config.json ("top_hit_num": 5000000): totals over the 10 000 queries
 SHIPPED_GRAPH_COUNTERS = {  # L: (expansions, distance evaluations)
+    512: (13294172, 244437655),
+    22528: (426698680, 2746117307),
 }
 SHIPPED_GRAPH_RECALL_BEAM = 22528  # the smallest multiple of 512 with recall@100 >= 0.90 on that graph (bench.py's leg)
 
@@ -292,6 +294,9 @@ def big_case(orc, n, dim, Qs, L, k, tomb_seed=None, built=False):
         B = st.expansions * 128 + st.dist_evals * dim * 4 + Q * (dim * 4 + k * 8)
         print("n=%d Q=%d: %.0f QPS, %.0f GB/s algorithmic, %d spills" %
               (n, Q, Q / st.kernel_s, B / st.kernel_s / 1e9, st.spills), flush=True)
+        # beyond 2^24 ids too the visited set of nearly every query stays in LDS: the library sizes the table of
+        # 16-bit cells for the displacement a cell has to carry, not for the load alone
+        assert st.spills * 20 <= Q or n <= (1 << 24)
     # a query's answer does not depend on the batch it travels in
     small = min(Qs)
     for Q in Qs:
