@@ -49,8 +49,11 @@ __device__ __forceinline__ void wave_sync() {
 // byte per node: a sixth of the memory, the same one line per test.
 // SCREEN: rows are first measured in a smaller copy of the vectors (rows of more than 128 floats): 1 the half-precision
 // copy (b.vec16), 2 the copy in eight-bit codes (b.vec8; rows of up to 512 floats).
-template <int G, int CPL, int RIF, bool PACKED, int SCREEN>
-__global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 32 ? 2 : RIF >= 16 ? 4 : 5)) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
+// WGS: workgroups a CU is to hold, which sets the registers a lane may use: what the rows in flight allow (two for a
+// whole step's rows at once, four for 16, five for 8), or three where the beam leaves LDS for no more than three anyway
+// (L beyond about 1000: +14 % at L = 1280 against squeezing into the registers of four).
+template <int G, int CPL, int RIF, bool PACKED, int SCREEN, int WGS>
+__global__ __launch_bounds__(kWavesPerWg * 64, WGS) void best_first_wave_kernel(const SearchArgs a, const BestFirstArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = blockIdx.x * kWavesPerWg + wave;
@@ -598,32 +601,39 @@ using bf_kernel_fn = void (*)(const SearchArgs, const BestFirstArgs);
 // RIF float4 registers of row data per lane are requested before any is added up: 16 halves the number of
 // dependent memory waits of a step against 8 and needs 128 registers; 32 (a whole step at once, 212 registers) is
 // for launches whose LDS holds a CU to eight wavefronts anyway (+2..3 %)
-template <int RIF, bool PACKED, int SCREEN>
+template <int RIF, bool PACKED, int SCREEN, int WGS>
 bf_kernel_fn pick_bf_kernel_rif(int chunks) {
     constexpr int WIDE = SCREEN == 2 ? 1 : SCREEN;  // rows of more than 512 floats have no copy in eight-bit codes
-    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED, 0>;
-    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, 0>;
-    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED, SCREEN>;
-    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED, SCREEN>;
-    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED, WIDE>;
-    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED, WIDE>;
+    if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED, 0, WGS>;
+    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, 0, WGS>;
+    if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED, SCREEN, WGS>;
+    if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED, SCREEN, WGS>;
+    if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED, WIDE, WGS>;
+    if (chunks <= 512) return best_first_wave_kernel<64, 8, RIF, PACKED, WIDE, WGS>;
     return nullptr;
 }
 
 template <int SCREEN>
-bf_kernel_fn pick_bf_kernel_screen(int dim, int rif, bool packed) {
+bf_kernel_fn pick_bf_kernel_screen(int dim, int rif, bool packed, bool three) {
     // 32: for launches that hold eight wavefronts per CU or fewer (256 registers per lane); rows of 17..64 chunks
     if (rif >= 32 && dim / 4 > 16 && dim / 4 <= 64)
-        return packed ? pick_bf_kernel_rif<32, true, SCREEN>(dim / 4) : pick_bf_kernel_rif<32, false, SCREEN>(dim / 4);
+        return packed ? pick_bf_kernel_rif<32, true, SCREEN, 2>(dim / 4) : pick_bf_kernel_rif<32, false, SCREEN, 2>(dim / 4);
+    if (three) {
+        if (packed)
+            return rif >= 16 ? pick_bf_kernel_rif<16, true, SCREEN, 3>(dim / 4) : pick_bf_kernel_rif<8, true, SCREEN, 3>(dim / 4);
+        return rif >= 16 ? pick_bf_kernel_rif<16, false, SCREEN, 3>(dim / 4) : pick_bf_kernel_rif<8, false, SCREEN, 3>(dim / 4);
+    }
     if (packed)
-        return rif >= 16 ? pick_bf_kernel_rif<16, true, SCREEN>(dim / 4) : pick_bf_kernel_rif<8, true, SCREEN>(dim / 4);
-    return rif >= 16 ? pick_bf_kernel_rif<16, false, SCREEN>(dim / 4) : pick_bf_kernel_rif<8, false, SCREEN>(dim / 4);
+        return rif >= 16 ? pick_bf_kernel_rif<16, true, SCREEN, 4>(dim / 4) : pick_bf_kernel_rif<8, true, SCREEN, 5>(dim / 4);
+    return rif >= 16 ? pick_bf_kernel_rif<16, false, SCREEN, 4>(dim / 4) : pick_bf_kernel_rif<8, false, SCREEN, 5>(dim / 4);
 }
 
-bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed, int screen) {
-    return screen == 2   ? pick_bf_kernel_screen<2>(dim, rif, packed)
-           : screen == 1 ? pick_bf_kernel_screen<1>(dim, rif, packed)
-                         : pick_bf_kernel_screen<0>(dim, rif, packed);
+// lds: bytes of one workgroup; a CU that has room for three workgroups at most runs the form compiled for three
+bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed, int screen, size_t lds) {
+    const bool three = lds * 4 > (size_t)160 * 1024;
+    return screen == 2   ? pick_bf_kernel_screen<2>(dim, rif, packed, three)
+           : screen == 1 ? pick_bf_kernel_screen<1>(dim, rif, packed, three)
+                         : pick_bf_kernel_screen<0>(dim, rif, packed, three);
 }
 
 }  // namespace
@@ -631,9 +641,9 @@ bf_kernel_fn pick_bf_kernel(int dim, int rif, bool packed, int screen) {
 hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, int screen, int bloom_log2,
                               int table_log2, int* max_wg_per_cu) {
     if (screen == 2 && dim > kMaxByteRowDim) return hipErrorInvalidValue;
-    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed, screen);
-    if (!fn) return hipErrorInvalidValue;
     const size_t lds = best_first_wave_lds_bytes(L, bloom_log2, table_log2, screen == 2 ? coded_query_bytes(dim) : 0) * kWavesPerWg;
+    bf_kernel_fn fn = pick_bf_kernel(dim, rows_in_flight, packed, screen, lds);
+    if (!fn) return hipErrorInvalidValue;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -647,11 +657,11 @@ hipError_t best_first_prepare(int dim, int L, int rows_in_flight, bool packed, i
 hipError_t launch_best_first(const SearchArgs& a, const BestFirstArgs& b, hipStream_t stream) {
     const int screen = b.vec8 != nullptr ? 2 : b.vec16 != nullptr ? 1 : 0;
     if (screen == 2 && (a.dim > kMaxByteRowDim || b.coded_bytes != coded_query_bytes(a.dim))) return hipErrorInvalidValue;
-    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0, screen);
+    const size_t lds = best_first_wave_lds_bytes(a.L, b.bloom_log2, b.table_log2, b.coded_bytes) * kWavesPerWg;
+    bf_kernel_fn fn = pick_bf_kernel(a.dim, b.rows_in_flight, b.packed != 0, screen, lds);
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
-    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64),
-                       best_first_wave_lds_bytes(a.L, b.bloom_log2, b.table_log2, b.coded_bytes) * kWavesPerWg, stream, a, b);
+    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), lds, stream, a, b);
     return hipGetLastError();
 }
 

@@ -55,9 +55,12 @@ __device__ __forceinline__ void memory_sync() {
 
 // SCREEN: once the queue is full, rows are first measured in the copy in eight-bit codes (b.vec8; rows of 132 .. 512
 // floats) and only those that may enter the queue are read in fp32 (search_device.h).
-template <int G, int CPL, int RIF, bool PACKED, bool SCREEN>
-__global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_first_long_kernel(const SearchArgs a,
-                                                                                                   const BestFirstLongArgs b) {
+// WGS: workgroups a CU is to hold.  The insert buffer decides how many fit its LDS (three at 512 keys); the registers
+// a lane may use follow from that number, and a launch that LDS holds to three workgroups per CU need not squeeze into
+// the 128 registers that four would leave.
+template <int G, int CPL, int RIF, bool PACKED, bool SCREEN, int WGS>
+__global__ __launch_bounds__(kWavesPerWg * 64, WGS) void best_first_long_kernel(const SearchArgs a,
+                                                                                   const BestFirstLongArgs b) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = blockIdx.x * kWavesPerWg + wave;
@@ -502,37 +505,45 @@ __global__ __launch_bounds__(kWavesPerWg * 64, (RIF >= 16 ? 4 : 5)) void best_fi
 
 using bfl_kernel_fn = void (*)(const SearchArgs, const BestFirstLongArgs);
 
-template <int RIF, bool PACKED, bool SCREEN>
+template <int RIF, bool PACKED, bool SCREEN, int WGS>
 bfl_kernel_fn pick_rif(int chunks) {
-    if (chunks <= 16) return best_first_long_kernel<16, 1, RIF, PACKED, false>;
-    if (chunks <= 32) return best_first_long_kernel<32, 1, RIF, PACKED, false>;
-    if (chunks <= 64) return best_first_long_kernel<64, 1, RIF, PACKED, SCREEN>;
-    if (chunks <= 128) return best_first_long_kernel<64, 2, RIF, PACKED, SCREEN>;
-    if (chunks <= 256) return best_first_long_kernel<64, 4, RIF, PACKED, false>;
-    if (chunks <= 512) return best_first_long_kernel<64, 8, RIF, PACKED, false>;
+    if (chunks <= 16) return best_first_long_kernel<16, 1, RIF, PACKED, false, WGS>;
+    if (chunks <= 32) return best_first_long_kernel<32, 1, RIF, PACKED, false, WGS>;
+    if (chunks <= 64) return best_first_long_kernel<64, 1, RIF, PACKED, SCREEN, WGS>;
+    if (chunks <= 128) return best_first_long_kernel<64, 2, RIF, PACKED, SCREEN, WGS>;
+    if (chunks <= 256) return best_first_long_kernel<64, 4, RIF, PACKED, false, WGS>;
+    if (chunks <= 512) return best_first_long_kernel<64, 8, RIF, PACKED, false, WGS>;
     return nullptr;
 }
 
-template <bool SCREEN>
+template <bool SCREEN, int WGS>
 bfl_kernel_fn pick_screen(int dim, bool packed) {
     const int chunks = dim / 4;
-    // 16 rows requested per wavefront before any is added up where that fits 128 registers, else 8
+    // 16 rows requested per wavefront before any is added up where that fits the registers, else 8
     const bool wide = chunks > 16 && chunks <= 256;
-    if (packed) return wide ? pick_rif<16, true, SCREEN>(chunks) : pick_rif<8, true, SCREEN>(chunks);
-    return wide ? pick_rif<16, false, SCREEN>(chunks) : pick_rif<8, false, SCREEN>(chunks);
+    if (packed) return wide ? pick_rif<16, true, SCREEN, WGS>(chunks) : pick_rif<8, true, SCREEN, WGS>(chunks);
+    return wide ? pick_rif<16, false, SCREEN, WGS>(chunks) : pick_rif<8, false, SCREEN, WGS>(chunks);
 }
 
-bfl_kernel_fn pick(int dim, bool packed, bool screen) {
-    return screen ? pick_screen<true>(dim, packed) : pick_screen<false>(dim, packed);
+// workgroups per CU that LDS leaves room for, in the steps the kernel is compiled for: 2, 3 or 4 and more
+int wgs_class(size_t lds_per_wg) {
+    const size_t fit = (size_t)160 * 1024 / lds_per_wg;
+    return fit >= 4 ? 4 : fit >= 3 ? 3 : 2;
+}
+
+bfl_kernel_fn pick(int dim, bool packed, bool screen, int wgs) {
+    if (wgs >= 4) return screen ? pick_screen<true, 4>(dim, packed) : pick_screen<false, 4>(dim, packed);
+    if (wgs == 3) return screen ? pick_screen<true, 3>(dim, packed) : pick_screen<false, 3>(dim, packed);
+    return screen ? pick_screen<true, 2>(dim, packed) : pick_screen<false, 2>(dim, packed);
 }
 
 }  // namespace
 
 hipError_t best_first_long_prepare(int dim, bool packed, bool screen, int bcap, int scap, int* max_wg_per_cu) {
     if (screen && (dim > kMaxByteRowDim || dim / 4 <= 32)) return hipErrorInvalidValue;
-    bfl_kernel_fn fn = pick(dim, packed, screen);
-    if (!fn) return hipErrorInvalidValue;
     const size_t lds = best_first_long_lds_bytes(bcap, scap, screen ? best_first_long_coded_bytes(dim) : 0) * kWavesPerWg;
+    bfl_kernel_fn fn = pick(dim, packed, screen, wgs_class(lds));
+    if (!fn) return hipErrorInvalidValue;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -547,11 +558,11 @@ hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& 
     const bool screen = b.vec8 != nullptr;
     if (screen && (a.dim > kMaxByteRowDim || a.dim / 4 <= 32 || b.coded_bytes != best_first_long_coded_bytes(a.dim)))
         return hipErrorInvalidValue;
-    bfl_kernel_fn fn = pick(a.dim, b.packed != 0, screen);
+    const size_t lds = best_first_long_lds_bytes(b.bcap, b.scap, b.coded_bytes) * kWavesPerWg;
+    bfl_kernel_fn fn = pick(a.dim, b.packed != 0, screen, wgs_class(lds));
     if (!fn) return hipErrorInvalidValue;
     const int wgs = (b.slots + kWavesPerWg - 1) / kWavesPerWg;
-    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64),
-                       best_first_long_lds_bytes(b.bcap, b.scap, b.coded_bytes) * kWavesPerWg, stream, a, b);
+    hipLaunchKernelGGL(fn, dim3(wgs), dim3(kWavesPerWg * 64), lds, stream, a, b);
     return hipGetLastError();
 }
 

@@ -535,11 +535,10 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // without the LDS table: L > 409): +12 % at L = 512 and 1024.  With the table (eight wavefronts per CU) the extra
     // wait per step costs more than the bytes it spares (L = 256 / 320: -27 %), so those launches go without unless
     // the caller asks for it by name.
-    if (long_form && idx->dim / 4 > 32 && idx->dim <= coral::kMaxByteRowDim &&
-        (t.screening == 2 || (t.screening == 0 && L <= 8192))) {
-        // the kernel of long beams screens on eight-bit codes only, and by itself only up to L = 8192: the longer
-        // the queue, the larger the share of rows that enter it and need their fp32 row after all (measured at a
-        // million nodes: +8 % at L = 1536, +2 % at 4096, nothing at 8192, -5 % at 19 456)
+    if (long_form && idx->dim / 4 > 32 && idx->dim <= coral::kMaxByteRowDim && (t.screening == 2 || t.screening == 0)) {
+        // the kernel of long beams screens on eight-bit codes only.  (The longer the queue, the larger the share of
+        // rows that enter it and need their fp32 row after all: a quarter at L = 19 456 on a million isotropic
+        // vectors, where the screening still spares a third of the launch's bytes.)
         const hipError_t e = ensure_vec8();
         if (e == hipSuccess) {
             idx->bf_screen = 2;
