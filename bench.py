@@ -221,7 +221,8 @@ def cpu_reference(w, gt, L, k, budget_s=20.0, stride_first=False):
         times.append(t)
     t = sorted(times)[len(times) // 2]
     hits = oracle.recall_hits(ids, gt[:n], k)
-    return {"value": n / t, "unit": "queries/s", "cores": threads, "kind": "reference" if use_ref else "port",
+    return {"_ids": ids,  # (dropped before the line is printed)
+            "value": n / t, "unit": "queries/s", "cores": threads, "kind": "reference" if use_ref else "port",
             "sample": "first %d of %d queries, L=%d, k=%d, M=%d start ids, policy best-first; median of %d passes" %
                       (n, q.shape[0], L, k, w["starts"].size, len(times)),
             "L": L, "recall": hits / float(n * k), "time_s": t, "passes_s": [round(x, 4) for x in times],
@@ -498,8 +499,7 @@ def main():
     recall_met = recall_met and head["recall"] >= RECALL_TARGET
     log("headline L=%d: %.0f q/s, recall %.4f" % (L_head, head["qps"], head["recall"]))
 
-    head_kernel = "beam_search_kernel" if args.policy == "rounds" else \
-        "best_first_long_kernel" if head["L"] > 1280 else "best_first_wave_kernel"
+    head_kernel = head["plan"]["kernel"]
     traffic = measured_traffic(head_kernel, head["L"], args.policy) if args.n == 1000000 and \
         args.queries == 10000 else None
     out = {
@@ -608,12 +608,20 @@ def main():
             def same_policy():
                 # the CPU path's traversal on the GPU at the CPU's beam, the whole batch
                 r = b.measure(cpu["L"], 2, 1, capi.POLICY_BEST_FIRST)
-                r["kernel"] = "best_first_long_kernel" if cpu["L"] > 1280 else "best_first_wave_kernel"
+                r["kernel"] = r["plan"]["kernel"]
+                # the same queries, the same traversal, the same beam on both sides: how many id lists are identical
+                # (the two differ in summation order only), and the GPU's recall on the CPU's sample
+                ci = cpu["_ids"]
+                gi = b.d_ids[:ci.shape[0]].cpu().numpy()
+                import oracle
+                r["id_lists_equal_to_cpu"] = float((gi == ci).all(1).mean())
+                r["recall_on_cpu_sample"] = oracle.recall_hits(gi, b.gt[:ci.shape[0]], k) / float(ci.size)
                 return r
             bf = optional(same_policy)
             if bf and "qps" in bf:
                 out["best_first"] = slim(bf)
-                out["best_first"]["kernel"] = bf["kernel"]
+                for key in ("kernel", "id_lists_equal_to_cpu", "recall_on_cpu_sample"):
+                    out["best_first"][key] = bf[key]
                 tr = measured_traffic(bf["kernel"], bf["L"], "best_first")
                 out["best_first"]["traffic"] = tr["bytes"] if tr else None
                 out["gpu_over_cpu_same_policy"] = bf["qps"] / cpu["value"]
@@ -641,7 +649,14 @@ def main():
         out["configs"] = {"1": optional(config1_leg, not args.no_cpu), "3": optional(config3_leg),
                           "4": optional(config4_leg), "5": optional(config5_leg)}
     out["wall_s"] = time.time() - T0
-    print(json.dumps(out), flush=True)
+
+    def scrub(o):  # arrays kept for cross-checks between legs are no part of the line
+        if isinstance(o, dict):
+            return {k2: scrub(v) for k2, v in o.items() if not k2.startswith("_")}
+        if isinstance(o, list):
+            return [scrub(v) for v in o]
+        return o
+    print(json.dumps(scrub(out)), flush=True)
     return 0
 
 

@@ -145,10 +145,12 @@ constexpr int search_exact_list_cap(int tcap) { return tcap < 1024 ? tcap : 1024
 size_t search_lds_bytes(int L, int dim, int table_words, int tcap, int ccap, int ocap, bool big, bool screening);
 // the half-precision copy of the vectors that the screening phase reads: bytes per row, and its construction
 size_t half_row_stride(int dim);
-// the copy in eight-bit codes (dim <= 512: a row's chunks of sixteen codes are read by sixteen lanes, two each at most)
+// the copy in eight-bit codes (a row's chunks of sixteen codes are read by sixteen lanes: up to two each for rows of
+// up to 512 floats, four or eight for longer ones)
 size_t byte_row_stride(int dim);
 hipError_t launch_byte_rows(const float* vec, int64_t n, int dim, unsigned char* out, hipStream_t stream);
-constexpr int kMaxByteRowDim = 512;
+constexpr int kMaxByteRowDim = 512;         // ... in the wavefront-per-query best-first kernels
+constexpr int kMaxByteRowDimRounds = 2048;  // ... in the workgroup-per-query kernel (rounds policy)
 hipError_t launch_half_rows(const float* vec, int64_t n, int dim, unsigned char* out, hipStream_t stream);
 // 64-bit words of global scratch one workgroup of a BIG launch needs for a beam of capacity L
 size_t search_beam_stride(int L);

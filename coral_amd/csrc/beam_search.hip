@@ -350,12 +350,13 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
         // classes from a quarter of the bytes.  Sixteen lanes per row (a 256-byte row at dim 200: two cache lines),
         // eight rows in flight per group, four groups per wavefront.
         auto screening_phase8 = [&](const uint32_t* list, int T) {
-            if constexpr (G >= 32 && CPL <= 2) {  // 64 < dim <= 512: a row's code chunks are CPL per lane of its sixteen
+            if constexpr (G >= 32) {  // dim > 64: a row's code chunks are CPL per lane of its sixteen
                 constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
+                constexpr bool WIDE8 = CPL8 > 2;  // rows of more than 512 codes: the coded query stays in LDS
                 const int gl8 = lane & 15, grp8 = lane >> 4;
                 const int nck = (dim + 15) >> 4;  // chunks of sixteen codes; the row's three figures are chunk nck
-                CodedQuery<CPL8> cq;
-                load_coded_query<CPL8>(qh8, ql8, nck, gl8, cq);
+                CodedQuery<WIDE8 ? 1 : CPL8> cq;
+                if constexpr (!WIDE8) load_coded_query<CPL8>(qh8, ql8, nck, gl8, cq);
                 const float qq = s_qq, sq = s_qscale, eq = s_qerr;
                 const float s_live = st.live == kKeyMax ? 3.402823466e+38f : key_s(st.live);
                 const uint32_t st8 = (uint32_t)a.stride8;
@@ -373,7 +374,10 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     if (gl8 >= U8 || mi >= T) myid = -1;
                     const bool valid = myid >= 0;
                     float lo, hi;
-                    coded_rows_bounds<CPL8, U8>(a.vec8, st8, nck, gl8, vid, myid, cq, qq, sq, eq, a.metric, lo, hi);
+                    if constexpr (WIDE8)
+                        coded_rows_bounds_wide<CPL8, U8>(a.vec8, st8, nck, gl8, vid, myid, qh8, ql8, qq, sq, eq, a.metric, lo, hi);
+                    else
+                        coded_rows_bounds<CPL8, U8>(a.vec8, st8, nck, gl8, vid, myid, cq, qq, sq, eq, a.metric, lo, hi);
                     const bool gone = valid && lo > thr;
                     const bool counted = valid && !gone && hi < thr && lo > s_live;
                     const bool exact = valid && !gone && !counted;

@@ -47,8 +47,8 @@ __device__ __forceinline__ void wave_sync() {
 
 // PACKED: the visited state of a slot is one 32-bit word per 24 nodes (8 bits of epoch, 24 flags) instead of one
 // byte per node: a sixth of the memory, the same one line per test.
-// SCREEN: rows are first measured in a smaller copy of the vectors (rows of more than 128 floats): 1 the half-precision
-// copy (b.vec16), 2 the copy in eight-bit codes (b.vec8; rows of up to 512 floats).
+// SCREEN: rows are first measured in a smaller copy of the vectors: 1 the half-precision copy (b.vec16; rows of more
+// than 128 floats), 2 the copy in eight-bit codes (b.vec8; rows of 68 .. 512 floats).
 // WGS: workgroups a CU is to hold, which sets the registers a lane may use: what the rows in flight allow (two for a
 // whole step's rows at once, four for 16, five for 8), or three where the beam leaves LDS for no more than three anyway
 // (L beyond about 1000: +14 % at L = 1280 against squeezing into the registers of four).
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, WGS) void best_first_wave_kernel(
                 n_screened += T;
                 T = n2;
             }
-            if constexpr (SCREEN == 2 && G == 64 && CPL <= 2) {
+            if constexpr (SCREEN == 2 && G >= 32 && CPL <= 2) {
                 if (nb == L) {
                     // the same on eight-bit codes: sixteen lanes per row, all 32 rows of a step in one round of requests
                     constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
@@ -605,7 +605,7 @@ template <int RIF, bool PACKED, int SCREEN, int WGS>
 bf_kernel_fn pick_bf_kernel_rif(int chunks) {
     constexpr int WIDE = SCREEN == 2 ? 1 : SCREEN;  // rows of more than 512 floats have no copy in eight-bit codes
     if (chunks <= 16) return best_first_wave_kernel<16, 1, RIF, PACKED, 0, WGS>;
-    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, 0, WGS>;
+    if (chunks <= 32) return best_first_wave_kernel<32, 1, RIF, PACKED, (SCREEN == 2 ? 2 : 0), WGS>;  // (codes only)
     if (chunks <= 64) return best_first_wave_kernel<64, 1, RIF, PACKED, SCREEN, WGS>;
     if (chunks <= 128) return best_first_wave_kernel<64, 2, RIF, PACKED, SCREEN, WGS>;
     if (chunks <= 256) return best_first_wave_kernel<64, 4, RIF, PACKED, WIDE, WGS>;

@@ -53,7 +53,7 @@ __device__ __forceinline__ void memory_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// SCREEN: once the queue is full, rows are first measured in the copy in eight-bit codes (b.vec8; rows of 132 .. 512
+// SCREEN: once the queue is full, rows are first measured in the copy in eight-bit codes (b.vec8; rows of 68 .. 512
 // floats) and only those that may enter the queue are read in fp32 (search_device.h).
 // WGS: workgroups a CU is to hold.  The insert buffer decides how many fit its LDS (three at 512 keys); the registers
 // a lane may use follow from that number, and a launch that LDS holds to three workgroups per CU need not squeeze into
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(kWavesPerWg * 64, WGS) void best_first_long_kernel(
         // todo[0..T) -> distances -> the queue
         auto measure_and_merge = [&](int T) {
             const uint32_t* list = todo;
-            if constexpr (SCREEN && G == 64 && CPL <= 2) {
+            if constexpr (SCREEN && G >= 32 && CPL <= 2) {
                 if (live != kKeyMax) {
                     // a row whose exact distance is certainly beyond the queue's worst entry is dropped on its codes
                     constexpr int CPL8 = CPL, U8 = 8 / CPL8, RPI8 = 4 * U8;
@@ -508,7 +508,7 @@ using bfl_kernel_fn = void (*)(const SearchArgs, const BestFirstLongArgs);
 template <int RIF, bool PACKED, bool SCREEN, int WGS>
 bfl_kernel_fn pick_rif(int chunks) {
     if (chunks <= 16) return best_first_long_kernel<16, 1, RIF, PACKED, false, WGS>;
-    if (chunks <= 32) return best_first_long_kernel<32, 1, RIF, PACKED, false, WGS>;
+    if (chunks <= 32) return best_first_long_kernel<32, 1, RIF, PACKED, SCREEN, WGS>;
     if (chunks <= 64) return best_first_long_kernel<64, 1, RIF, PACKED, SCREEN, WGS>;
     if (chunks <= 128) return best_first_long_kernel<64, 2, RIF, PACKED, SCREEN, WGS>;
     if (chunks <= 256) return best_first_long_kernel<64, 4, RIF, PACKED, false, WGS>;
@@ -540,7 +540,7 @@ bfl_kernel_fn pick(int dim, bool packed, bool screen, int wgs) {
 }  // namespace
 
 hipError_t best_first_long_prepare(int dim, bool packed, bool screen, int bcap, int scap, int* max_wg_per_cu) {
-    if (screen && (dim > kMaxByteRowDim || dim / 4 <= 32)) return hipErrorInvalidValue;
+    if (screen && (dim > kMaxByteRowDim || dim / 4 <= 16)) return hipErrorInvalidValue;
     const size_t lds = best_first_long_lds_bytes(bcap, scap, screen ? best_first_long_coded_bytes(dim) : 0) * kWavesPerWg;
     bfl_kernel_fn fn = pick(dim, packed, screen, wgs_class(lds));
     if (!fn) return hipErrorInvalidValue;
@@ -556,7 +556,7 @@ hipError_t best_first_long_prepare(int dim, bool packed, bool screen, int bcap, 
 
 hipError_t launch_best_first_long(const SearchArgs& a, const BestFirstLongArgs& b, hipStream_t stream) {
     const bool screen = b.vec8 != nullptr;
-    if (screen && (a.dim > kMaxByteRowDim || a.dim / 4 <= 32 || b.coded_bytes != best_first_long_coded_bytes(a.dim)))
+    if (screen && (a.dim > kMaxByteRowDim || a.dim / 4 <= 16 || b.coded_bytes != best_first_long_coded_bytes(a.dim)))
         return hipErrorInvalidValue;
     const size_t lds = best_first_long_lds_bytes(b.bcap, b.scap, b.coded_bytes) * kWavesPerWg;
     bfl_kernel_fn fn = pick(a.dim, b.packed != 0, screen, wgs_class(lds));

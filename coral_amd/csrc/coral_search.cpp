@@ -292,22 +292,27 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
     // ---- screening on a smaller copy of the vectors (rounds policy, L2, rows of 132 .. 2048 floats): eight-bit codes
     // (tuning 2; the library's choice up to 512 floats) or half precision (tuning 1); see beam_search.hip
     // (best-first: the wavefront-per-query kernel with the beam in LDS screens too, see coral_search_prepare)
-    const bool codes_possible = idx->dim <= coral::kMaxByteRowDim;  // the inner product is screened on codes only
+    // (the inner product is screened on codes only)
+    const bool codes_possible = idx->dim <= (best_first ? coral::kMaxByteRowDim : coral::kMaxByteRowDimRounds);
     // (the rounds kernel takes codes for rows of more than 64 floats; half precision, and the best-first kernels,
     // need more than 128)
-    const bool wide = idx->dim / 4 > 32, codes_wide = idx->dim / 4 > 16 && !best_first;
+    const bool wide = idx->dim / 4 > 32, codes_wide = idx->dim / 4 > 16;
     const bool screen_possible = !best_first && ((wide && idx->metric == CORAL_L2) || ((wide || codes_wide) && codes_possible));
     if (t.screening > 2 || t.screening < -1) return fail(CORAL_ERR_ARG, "screening must be -1, 0, 1 or 2 (got %d)", t.screening);
     if (t.screening > 0 && !wide && !(t.screening == 2 && codes_wide))
-        return fail(CORAL_ERR_ARG, "screening needs more than 128 dimensions (on eight-bit codes, rounds policy: more than 64)");
+        return fail(CORAL_ERR_ARG, "screening needs more than 128 dimensions (on eight-bit codes: more than 64)");
     if (t.screening == 1 && idx->metric != CORAL_L2)
         return fail(CORAL_ERR_ARG, "screening in half precision needs the L2 metric");
     if (t.screening == 2 && !codes_possible)
-        return fail(CORAL_ERR_ARG, "screening on eight-bit codes takes rows of up to %d floats", coral::kMaxByteRowDim);
+        return fail(CORAL_ERR_ARG, "screening on eight-bit codes takes rows of up to %d floats",
+                    best_first ? coral::kMaxByteRowDim : coral::kMaxByteRowDimRounds);
     // (by itself the library screens rows of more than 128 floats only: at 128 floats and the short beam of the
     // configuration that has such rows, the codes cost 9 %)
     const bool screen = screen_possible && (t.screening > 0 || (t.screening == 0 && !no_screen && wide));
-    p.screen = !screen ? 0 : t.screening > 0 ? t.screening : (codes_possible ? 2 : 1);
+    // (the library's own choice: codes, except for L2 rows of more than 1024 floats, where the kernel form that keeps
+    // eight chunks of codes per lane is no faster than half precision: 103 k against 106 k QPS at 2048 floats, after
+    // 382 k against 291 k at 1024)
+    p.screen = !screen ? 0 : t.screening > 0 ? t.screening : (codes_possible && (idx->dim <= 1024 || idx->metric != CORAL_L2) ? 2 : 1);
     // ---- the visited structure.  Three forms: a table of 2^s 16-bit cells with an overflow bitmap in global memory
     // (visited_slots_log2 = s, or the library's choice), or a plain bitmap of all n ids in LDS (visited_slots_log2 =
     // -1, or the library's choice): one LDS atomic per test and nothing ever overflows, at n / 8 bytes -- 125 KB for
@@ -497,9 +502,12 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
                            (t.best_first_long > 0 || (t.best_first_long == 0 && L > kLongBeamFrom));
     const bool wave_form = best_first && !t.best_first_in_lds && !long_form && !plan.big &&
                            coral::best_first_wave_lds_bytes(L, 0, 0) * 4 <= (size_t)kMaxLdsBytes;
+    // rows of 68 .. 128 floats are screened (on codes) only when the caller asks for it by name; the coded query then
+    // takes the LDS a table of visited ids would fill
+    const bool narrow_codes = best_first && t.screening == 2 && idx->dim / 4 > 16 && idx->dim / 4 <= 32;
     int table_log2 = 0;
     if (wave_form)
-        if (int rc = choose_bf_table(L, id_bits, t.best_first_table_log2, &table_log2)) return rc;
+        if (int rc = choose_bf_table(L, id_bits, narrow_codes ? -1 : t.best_first_table_log2, &table_log2)) return rc;
     // from here on buffers are replaced: a failure part-way leaves the index unprepared, not half-prepared
     idx->prepared = false;
     const size_t need_words = plan.spill_words * (size_t)workgroups;
@@ -535,7 +543,8 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // without the LDS table: L > 409): +12 % at L = 512 and 1024.  With the table (eight wavefronts per CU) the extra
     // wait per step costs more than the bytes it spares (L = 256 / 320: -27 %), so those launches go without unless
     // the caller asks for it by name.
-    if (long_form && idx->dim / 4 > 32 && idx->dim <= coral::kMaxByteRowDim && (t.screening == 2 || t.screening == 0)) {
+    if (long_form && (idx->dim / 4 > 32 || narrow_codes) && idx->dim <= coral::kMaxByteRowDim &&
+        (t.screening == 2 || t.screening == 0)) {
         // the kernel of long beams screens on eight-bit codes only.  (The longer the queue, the larger the share of
         // rows that enter it and need their fp32 row after all: a quarter at L = 19 456 on a million isotropic
         // vectors, where the screening still spares a third of the launch's bytes.)
@@ -551,8 +560,10 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
     // eight-bit codes where they apply; launches with the LDS table (whose size was chosen to fill LDS) and rows of
     // more than 512 floats screen in half precision, which only the L2 metric has
     const int form = t.screening == 1 || idx->dim > coral::kMaxByteRowDim || table_log2 != 0 ? 1 : 2;
-    if (wave_form && idx->dim / 4 > 32 && (form == 2 || idx->metric == CORAL_L2) &&
-        (t.screening > 0 || (t.screening == 0 && table_log2 == 0))) {
+    // (rows of more than 512 floats, which this kernel can only screen in half precision, go without unless asked by
+    // name: 156 k against 211 k QPS at 1024 floats and L = 512, 51 k against 111 k at 2048)
+    if (wave_form && (idx->dim / 4 > 32 || narrow_codes) && (form == 2 || idx->metric == CORAL_L2) &&
+        (t.screening > 0 || (t.screening == 0 && table_log2 == 0 && idx->dim <= coral::kMaxByteRowDim))) {
         const hipError_t e = form == 2 ? ensure_vec8() : ensure_vec16();
         if (e == hipSuccess) {
             idx->bf_screen = form;

@@ -105,7 +105,8 @@ __device__ __forceinline__ void load_coded_query(const signed char* qh8, const s
 //
 // Inner product (metric 1; the signed distance is -q.x): q.x = q~.x~ + q~.(x - x~) + (q - q~).x, so
 // |q.x - q~.x~| <= |q~| e + eq (|x~| + e); the bound is widened by 2e-4 (|q~| + eq)(|x~| + e) for the fp32 rounding of
-// the exact inner product and of the computed q~.x~ (each at most dim 2^-24 |q| |x|, dim <= 512).
+// the exact inner product and of the computed q~.x~ (each at most dim 2^-24 |q| |x|; rows of up to 512 floats: 6e-5;
+// 6e-4 for rows of up to 2048).
 template <int CPL8, int U8>
 struct CodedRows {
     uint4 hb[U8][CPL8];
@@ -133,6 +134,7 @@ __device__ __forceinline__ void coded_rows_request(const unsigned char* vec8, ui
 
 template <int CPL8, int U8>
 __device__ __forceinline__ void coded_rows_dots(const CodedRows<CPL8, U8>& r, const CodedQuery<CPL8>& q, int (&acc)[U8]) {
+    static_assert(CPL8 <= 4, "the combined sum 128 dh + dl fits 32 bits for rows of up to 1024 codes");
 #pragma unroll
     for (int u = 0; u < U8; ++u) {
         int dh = 0, dl = 0;
@@ -145,13 +147,40 @@ __device__ __forceinline__ void coded_rows_dots(const CodedRows<CPL8, U8>& r, co
                 dl = __builtin_amdgcn_sdot4(w[j], q.l[t][j], dl, false);
             }
         }
-        acc[u] = 128 * dh + dl;  // below 2^31 for 512 dimensions: 512 * 127 * 16256
+        acc[u] = 128 * dh + dl;  // below 2^31 for 1024 dimensions: 1024 * 127 * 16256
     }
 }
 
+// The same for rows of more than 512 codes (CPL8 = 4 or 8 chunks per lane): the coded query would take 8 CPL8
+// registers, so its chunks are read from LDS as they are used; and beyond 1024 codes 128 dh + dl no longer fits 32
+// bits, so the two sums stay apart (each below 2^26) until they are floats.
+template <int CPL8, int U8>
+__device__ __forceinline__ void coded_rows_dots_wide(const CodedRows<CPL8, U8>& r, const signed char* qh8,
+                                                     const signed char* ql8, int nck, int gl8, int (&acch)[U8],
+                                                     int (&accl)[U8]) {
+#pragma unroll
+    for (int u = 0; u < U8; ++u) acch[u] = 0, accl[u] = 0;
+#pragma unroll
+    for (int t = 0; t < CPL8; ++t) {
+        const int c = gl8 + 16 * t;
+        int4 qh = make_int4(0, 0, 0, 0), ql = make_int4(0, 0, 0, 0);
+        if (c < nck) qh = reinterpret_cast<const int4*>(qh8)[c], ql = reinterpret_cast<const int4*>(ql8)[c];
+        const int hq[4] = {qh.x, qh.y, qh.z, qh.w}, lq[4] = {ql.x, ql.y, ql.z, ql.w};
+#pragma unroll
+        for (int u = 0; u < U8; ++u) {
+            const int w[4] = {(int)r.hb[u][t].x, (int)r.hb[u][t].y, (int)r.hb[u][t].z, (int)r.hb[u][t].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acch[u] = __builtin_amdgcn_sdot4(w[j], hq[j], acch[u], false);
+                accl[u] = __builtin_amdgcn_sdot4(w[j], lq[j], accl[u], false);
+            }
+        }
+    }
+}
+
+// the sum over the sixteen lanes of a row, for the lane that files it
 template <int U8>
-__device__ __forceinline__ void coded_rows_finish(int (&acc)[U8], int gl8, const float4& fig, float qq, float sq, float eq,
-                                                  int metric, float& lo, float& hi) {
+__device__ __forceinline__ int coded_rows_reduce(int (&acc)[U8], int gl8) {
 #pragma unroll
     for (int u = 0; u < U8; ++u) {
         acc[u] = acc[u] + dpp_mov_i<0xB1>(acc[u]);   // quad_perm [1,0,3,2]
@@ -163,9 +192,17 @@ __device__ __forceinline__ void coded_rows_finish(int (&acc)[U8], int gl8, const
 #pragma unroll
     for (int u = 1; u < U8; ++u)
         if (gl8 == u) mine = acc[u];
+    return mine;
+}
+
+// bounds from the integer sum as a float; WIDE: rows of more than 512 codes (two more roundings on the way to the
+// sum, and a longer exact inner product to allow for)
+template <bool WIDE>
+__device__ __forceinline__ void coded_bounds(float isum, const float4& fig, float qq, float sq, float eq, int metric,
+                                             float& lo, float& hi) {
     if (metric == 0) {
         const float both = qq + fig.y;
-        const float d8 = both - (2.0f * sq * fig.x) * (float)mine, delta = 16.0f * 5.9604645e-8f * both, e = fig.z + eq;
+        const float d8 = both - (2.0f * sq * fig.x) * isum, delta = (WIDE ? 24.0f : 16.0f) * 5.9604645e-8f * both, e = fig.z + eq;
         // (the hardware's square root, good to one unit in the last place and only trusted on normal numbers: below
         // 1e-36 the lower end takes 0 and the upper end the root of 1e-36; the 1e-4 covers the last place)
         const float under = d8 - delta, over = fmaxf(d8 + delta, 1.0e-36f);
@@ -173,12 +210,19 @@ __device__ __forceinline__ void coded_rows_finish(int (&acc)[U8], int gl8, const
         const float hi_root = __builtin_amdgcn_sqrtf(over) + e;
         lo = lo_root * lo_root * (1.0f - 1.0e-4f), hi = hi_root * hi_root * (1.0f + 1.0e-4f);
     } else {
-        const float p = (sq * fig.x) * (float)mine;  // q~.x~
+        const float p = (sq * fig.x) * isum;  // q~.x~
         const float nq = sqrtf(qq) * (1.0f + 1.0e-6f), e = fig.z;
         const float nx = __builtin_amdgcn_sqrtf(fmaxf(fig.y, 1.0e-36f)) * (1.0f + 1.0e-6f);
-        const float bound = (nq * e + eq * (nx + e) + 2.0e-4f * (nq + eq) * (nx + e)) * (1.0f + 1.0e-5f);
+        const float bound = (nq * e + eq * (nx + e) + (WIDE ? 6.0e-4f : 2.0e-4f) * (nq + eq) * (nx + e)) * (1.0f + 1.0e-5f);
         lo = (0.0f - p) - bound, hi = (0.0f - p) + bound;  // e = inf or eq = inf: lo = -inf, hi = inf (or NaN)
     }
+}
+
+template <int U8>
+__device__ __forceinline__ void coded_rows_finish(int (&acc)[U8], int gl8, const float4& fig, float qq, float sq, float eq,
+                                                  int metric, float& lo, float& hi) {
+    const int mine = coded_rows_reduce<U8>(acc, gl8);
+    coded_bounds<false>((float)mine, fig, qq, sq, eq, metric, lo, hi);
 }
 
 // the three steps in one go
@@ -191,6 +235,20 @@ __device__ __forceinline__ void coded_rows_bounds(const unsigned char* vec8, uin
     int acc[U8];
     coded_rows_dots<CPL8, U8>(r, q, acc);
     coded_rows_finish<U8>(acc, gl8, r.fig, qq, sq, eq, metric, lo, hi);
+}
+
+// rows of more than 512 codes: the query's codes come from LDS (qh8, ql8)
+template <int CPL8, int U8>
+__device__ __forceinline__ void coded_rows_bounds_wide(const unsigned char* vec8, uint32_t st8, int nck, int gl8,
+                                                       const int (&vid)[U8], int myid, const signed char* qh8,
+                                                       const signed char* ql8, float qq, float sq, float eq, int metric,
+                                                       float& lo, float& hi) {
+    CodedRows<CPL8, U8> r;
+    coded_rows_request<CPL8, U8>(vec8, st8, nck, gl8, vid, myid, r);
+    int acch[U8], accl[U8];
+    coded_rows_dots_wide<CPL8, U8>(r, qh8, ql8, nck, gl8, acch, accl);
+    const int mh = coded_rows_reduce<U8>(acch, gl8), ml = coded_rows_reduce<U8>(accl, gl8);
+    coded_bounds<true>(128.0f * (float)mh + (float)ml, r.fig, qq, sq, eq, metric, lo, hi);
 }
 
 // inclusive prefix sum over the 64 lanes: four steps inside the rows of 16 lanes, then the totals of the rows

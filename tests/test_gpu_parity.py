@@ -54,6 +54,9 @@ CASES = [
     (12000, 256, 24, "ip", 0, 96, 32, 8, 5, 0, 0),
     (6000, 1024, 16, "l2", 0, 64, 10, 4, None, 0, 0),
     (6000, 2048, 8, "l2", 0, 32, 8, 2, None, 0, 0),
+    (6000, 1024, 16, "ip", 0, 64, 10, 4, None, 0, 0),       # the inner product on rows of more than 512 floats
+    (6000, 2048, 8, "ip", 0, 200, 50, 2, None, 0, 0),
+    (6000, 1028, 16, "l2", 0, 200, 50, 4, None, 0, 0),      # a last chunk of codes that is part padding
     (20000, 200, 32, "l2", 0, 256, 100, 16, None, 11, 0),   # visited set forced out of LDS
     (20000, 200, 32, "l2", 0, 256, 100, 16, 3, 12, 512),
     (20000, 200, 32, "l2", 1, 64, 10, 16, None, 0, 0),      # best-first policy
@@ -97,8 +100,7 @@ def test_exact_against_same_order_oracle(orc, case):
         forms = (dict(screening=-1),)
         if metric == "l2":
             forms += (dict(screening=1), dict(screening=1, beam_in_hbm=True))
-        if dim <= 512:  # what the copy in eight-bit codes takes
-            forms += (dict(screening=2), dict(screening=2, beam_in_hbm=True))
+        forms += (dict(screening=2), dict(screening=2, beam_in_hbm=True))  # codes: rows of up to 2048 floats
     for form in forms:
         in_lds = form.get("best_first_in_lds", False)
         idx.prepare(q.shape[0], L, visited_slots_log2=slots, threads=threads, policy=policy, **form)
@@ -246,8 +248,8 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     n, dim, R, Q, L, k = 4000, 136, 24, 100, 200, 50
     dim = {"dim_not_a_multiple_of_8": 140, "dim_200": 200, "dim_264": 264, "ip_raw": 200, "dim_128": 128, "dim_72": 72,
            "ip_dim_100": 100, "half_subnormal_dim_2048": 2048}.get(kind, dim)
-    narrow = dim <= 128  # the rounds kernel screens such rows on codes; half precision and best-first do not
-    wide = dim > 512     # no copy in eight-bit codes for such rows
+    narrow = dim <= 128  # such rows are screened on codes only
+    wide = dim > 512     # the best-first kernels have no screening on codes for such rows
     ip = kind.startswith("ip_")
     m, mname = (capi.IP, "ip") if ip else (capi.L2, "l2")
     rng = np.random.RandomState(77)
@@ -281,8 +283,8 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
     for form in (dict(screening=-1), dict(screening=1), dict(screening=1, beam_in_hbm=True),
                  dict(screening=1, visited_slots_log2=12, threads=256), dict(screening=2),
                  dict(screening=2, beam_in_hbm=True), dict(screening=2, visited_slots_log2=12, threads=256), dict()):
-        # half precision: L2 and more than 128 floats only; codes: up to 512 floats
-        if ((ip or narrow) and form.get("screening") == 1) or (wide and form.get("screening") == 2):
+        # half precision: L2 and more than 128 floats only
+        if (ip or narrow) and form.get("screening") == 1:
             with pytest.raises(capi.CoralError):
                 idx.prepare(Q, L, **form)
             continue
@@ -298,8 +300,8 @@ def test_screening_on_a_smaller_copy_changes_nothing(orc, kind):
                  dict(screening=2, best_first_packed=True, best_first_table_log2=-1), dict(best_first_table_log2=-1),
                  dict(best_first_long=1), dict(best_first_long=1, screening=-1),
                  dict(best_first_long=1, best_first_buffer=64, best_first_packed=True, screening=2)):
-        if (ip and form.get("screening") == 1) or (narrow and form.get("screening", 0) > 0) or \
-                (wide and form.get("screening") == 2):
+        # (half precision: L2 and more than 128 floats; codes: 68 .. 512 floats)
+        if ((ip or narrow) and form.get("screening") == 1) or (wide and form.get("screening") == 2):
             continue
         idx.prepare(Q, L, policy=capi.POLICY_BEST_FIRST, **form)
         ids, dists, _ = idx.search(q, k, L, policy=capi.POLICY_BEST_FIRST)
