@@ -35,7 +35,7 @@ class Stats(C.Structure):
     _fields_ = [("time_s", C.c_double), ("kernel_s", C.c_double), ("hops", C.c_int64), ("expansions", C.c_int64),
                 ("dist_evals", C.c_int64), ("rounds", C.c_int64), ("spills", C.c_int64),
                 ("screened_rows", C.c_int64), ("exact_rows", C.c_int64), ("beam_words", C.c_int64),
-                ("visited_requests", C.c_int64)]
+                ("visited_requests", C.c_int64), ("visited_dedupes", C.c_int64)]
 
     def as_dict(self):
         return {f: getattr(self, f) for f, _ in self._fields_}
@@ -49,7 +49,8 @@ class PlanInfo(C.Structure):
 
     KERNELS = ("beam_search_kernel", "best_first_wave_kernel", "best_first_long_kernel")
     SCREENING = ("none", "fp16", "int8")
-    VISITED = ("lds_table16+hbm_bitmap", "lds_bitmap", "hbm_bytes", "hbm_packed_words", "lds_table16+hbm_state")
+    VISITED = ("lds_table16+hbm_bitmap", "lds_bitmap", "hbm_bytes", "hbm_packed_words", "lds_table16+hbm_state",
+               "lds_buckets16x3+hbm_bitmap")
 
     def as_dict(self):
         d = {f: getattr(self, f) for f, _ in self._fields_ if f != "reserved"}
@@ -64,7 +65,7 @@ class Tuning(C.Structure):
                 ("policy", C.c_int32), ("best_first_in_lds", C.c_int32), ("best_first_packed", C.c_int32),
                 ("best_first_table_log2", C.c_int32), ("beam_in_hbm", C.c_int32), ("prefetch_rows", C.c_int32),
                 ("cand_cap", C.c_int32), ("best_first_long", C.c_int32), ("best_first_buffer", C.c_int32),
-                ("screening", C.c_int32)]
+                ("screening", C.c_int32), ("visited_choices", C.c_int32)]
 
 
 class BuildParams(C.Structure):
@@ -235,10 +236,10 @@ class Index:
 
     def prepare(self, Q, L, visited_slots_log2=0, workgroups=0, threads=0, policy=POLICY_ROUNDS, best_first_in_lds=False,
                 best_first_packed=False, best_first_table_log2=0, beam_in_hbm=False, prefetch_rows=0, cand_cap=0,
-                best_first_long=0, best_first_buffer=0, screening=0):
+                best_first_long=0, best_first_buffer=0, screening=0, visited_choices=0):
         t = Tuning(visited_slots_log2, workgroups, threads, policy, int(bool(best_first_in_lds)),
                    int(bool(best_first_packed)), best_first_table_log2, int(bool(beam_in_hbm)), prefetch_rows,
-                   cand_cap, best_first_long, best_first_buffer, screening)
+                   cand_cap, best_first_long, best_first_buffer, screening, visited_choices)
         _check(lib().coral_search_prepare(self._h, Q, L, C.byref(t)))
 
     def search(self, queries, k, L, policy=POLICY_ROUNDS, have_delete=False, want_dists=True):

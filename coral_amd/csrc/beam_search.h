@@ -22,7 +22,7 @@ struct SearchArgs {
                                // of beam state moved in global memory, visited-state requests to global memory
     uint32_t* spill;           // [workgroups][spill_words] zeroed bitmaps
     int* next_qid;             // work counter, zero at launch
-    int* spill_count;          // queries that left LDS, zero at launch
+    int* spill_count;          // [0] queries that left LDS, [1] lists of new ids searched for repeats; zero at launch
     unsigned long long* phase_ticks;  // debug builds: 8 per-phase tick sums, else nullptr
     size_t spill_words;        // ceil(n/32)
     int64_t n;
@@ -55,6 +55,10 @@ struct SearchArgs {
     int32_t scap;              // BIG form: keys of the LDS sample of the beam that the merge searches first
     int32_t prefetch_rows;     // request a chunk's graph rows one chunk ahead (launches with one workgroup per CU)
     int32_t table_words;       // 32-bit words of LDS the visited structure takes (cells / 2, or ceil(n / 32) rounded up to 4)
+    // the table of 16-bit cells in its bucket form (0 or 3): buckets of four cells, three candidate buckets per id;
+    // rem_bits is then id_bits - (slots_log2 - 2), at most 14, and dmax is unused.  4: the same with the bucket picked
+    // by the inserting wavefront's number instead of by load (for tests of what follows concurrent inserts of one id)
+    int32_t bucket_choices;
 };
 
 // What the wavefront-per-query best-first kernel (best_first.hip) needs beyond SearchArgs.

@@ -85,6 +85,68 @@ struct VisitedSet {
     uint32_t smask, bmask, rmask;
     int rb, xs, dmax, ocap;
     bool direct;       // words is a bitmap of all ids (launches over few enough nodes that have LDS to spare)
+    // Third form of the first level, for ids too wide for the displacement a 16-bit cell can carry beside them
+    // (beyond 2^24 ids): the cells form buckets of four, an id may sit in any of three buckets -- its home, picked by
+    // the high bits of the mixed id, and two more that follow from the home and the remaining bits -- and a cell
+    // stores those remaining bits and which of the three it is in: cell = 1 + (choice << rb | remainder).  (bucket,
+    // cell) give the mixed id back, so the table is exact; a new id goes to the emptiest of its buckets, which keeps
+    // the load so even that a table two thirds full turns practically no id away (linear probing at that load needs
+    // displacements far beyond the 14 that 2^27 ids leave room for in 2^15 cells).  The price is that the place of
+    // an id depends on what a thread saw of the three buckets: two threads that insert the same id at the same time
+    // can each find it absent and put it into different buckets.  Every thread therefore looks at the other two
+    // buckets again after its insert; of two such threads at least the later one sees the other's cell, and raises
+    // *dupflag: the list of new ids is then searched for repeats before it is used (see the kernel).
+    bool buckets;
+    uint32_t bkmask;   // buckets - 1
+    int* dupflag;      // LDS
+    int skew;          // -1; or (a form for tests) the inserting wavefront's number, which then picks the bucket in
+                       // place of the load, so that concurrent inserts of one id part as often as they can
+
+    // the three buckets of a mixed id and what its cells would hold
+    __device__ __forceinline__ void places(uint32_t h, uint32_t (&bk)[3], uint32_t (&want)[3]) const {
+        const uint32_t rem = h & rmask, b0 = (h >> rb) & bkmask;
+        // two nonzero offsets that differ, from the remainder alone (so that bucket ^ offset gives the home back)
+        uint32_t o1 = ((rem * 0x9E3779B1u + 0x7F4A7C15u) >> 7) & bkmask, o2 = ((rem * 0x85EBCA6Bu + 0x165667B1u) >> 9) & bkmask;
+        if (o1 == 0u) o1 = 1u & bkmask;
+        if (o2 == 0u || o2 == o1) o2 = (o1 ^ 2u) & bkmask ? (o1 ^ 2u) & bkmask : (o1 + 1u) & bkmask;
+        bk[0] = b0, bk[1] = b0 ^ o1, bk[2] = b0 ^ o2;
+        want[0] = 1u + rem, want[1] = 1u + ((1u << rb) | rem), want[2] = 1u + ((2u << rb) | rem);
+    }
+
+    __device__ __forceinline__ static bool holds(const uint2 w, uint32_t want) {
+        return (w.x & 0xffffu) == want || (w.x >> 16) == want || (w.y & 0xffffu) == want || (w.y >> 16) == want;
+    }
+    __device__ __forceinline__ static int empties(const uint2 w) {
+        return ((w.x & 0xffffu) == 0u) + ((w.x >> 16) == 0u) + ((w.y & 0xffffu) == 0u) + ((w.y >> 16) == 0u);
+    }
+
+    // 1: id was not in the table and now is; 0: it was; 2: it is not and no bucket has room
+    __device__ __forceinline__ int bucket_test_and_set(uint32_t id) {
+        uint32_t bk[3], want[3];
+        places(mix(id), bk, want);
+        const uint2* bks = reinterpret_cast<const uint2*>(words);
+        for (;;) {
+            const uint2 w0 = bks[bk[0]], w1 = bks[bk[1]], w2 = bks[bk[2]];
+            if (holds(w0, want[0]) || holds(w1, want[1]) || holds(w2, want[2])) return 0;
+            const int e0 = empties(w0), e1 = empties(w1), e2 = empties(w2);
+            if (e0 + e1 + e2 == 0) return 2;
+            int c = (e0 >= e1 && e0 >= e2) ? 0 : (e1 >= e2 ? 1 : 2);
+            if (skew >= 0) {
+                const int cs = skew % 3;
+                if ((cs == 0 ? e0 : cs == 1 ? e1 : e2) > 0) c = cs;
+            }
+            const uint2 w = c == 0 ? w0 : c == 1 ? w1 : w2;
+            // the first empty cell of that bucket
+            const int cell = (w.x & 0xffffu) == 0u ? 0 : (w.x >> 16) == 0u ? 1 : (w.y & 0xffffu) == 0u ? 2 : 3;
+            const uint32_t oldw = cell < 2 ? w.x : w.y;
+            uint32_t* word = words + bk[c] * 2u + (uint32_t)(cell >> 1);
+            if (atomicCAS(word, oldw, oldw | (want[c] << ((cell & 1) * 16))) != oldw) continue;  // another thread took a cell of that word: look again
+            // the same id in another of its buckets: somebody inserted it at the same time
+            const int c1 = c == 0 ? 1 : 0, c2 = c == 2 ? 1 : 2;
+            if (holds(bks[bk[c1]], want[c1]) || holds(bks[bk[c2]], want[c2])) *dupflag = 1;
+            return 1;
+        }
+    }
 
     __device__ __forceinline__ uint32_t mix(uint32_t id) const {
         uint32_t h = (id * 0x9E3779B1u) & bmask;
@@ -99,6 +161,23 @@ struct VisitedSet {
         if (direct) {
             const uint32_t b = 1u << (id & 31);
             return (atomicOr(&words[id >> 5], b) & b) == 0u;
+        }
+        if (buckets) {
+            if (!frozen) {
+                const int r = bucket_test_and_set(id);
+                if (r != 2) return r;
+            } else {
+                uint32_t bk[3], want[3];
+                places(mix(id), bk, want);
+                const uint2* bks = reinterpret_cast<const uint2*>(words);
+                if (holds(bks[bk[0]], want[0]) || holds(bks[bk[1]], want[1]) || holds(bks[bk[2]], want[2])) return 0;
+            }
+            const uint32_t bit = 1u << (id & 31);
+            const uint32_t old = atomicOr(&bitmap[id >> 5], bit);
+            if (old & bit) return 0;
+            const int p = atomicAdd(ocount, 1);
+            if (p < ocap) olist[p] = id;
+            return 1;
         }
         const uint32_t h = mix(id);
         const uint32_t home = h >> rb, rem = h & rmask;
@@ -171,7 +250,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     }
     float* qs = (float*)(olist + a.ocap);
 
-    __shared__ int s_qid, s_ntodo, s_ntodo2, s_ncand, s_nexp, s_cntf, s_cursor, s_nover;
+    __shared__ int s_qid, s_ntodo, s_ntodo2, s_ncand, s_nexp, s_cntf, s_cursor, s_nover, s_dup;
     __shared__ int s_wcnt[16];
     // what the query read, by class (thread 0 alone adds to these and writes them out): rows measured on the smaller
     // copy, fp32 rows, words of a beam in global memory
@@ -185,6 +264,8 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
     vs.rb = a.rem_bits, vs.rmask = (1u << a.rem_bits) - 1u;
     vs.xs = a.id_bits > 1 ? a.id_bits / 2 : 1, vs.dmax = a.dmax, vs.ocap = a.ocap;
     vs.direct = a.direct_bitmap != 0;
+    vs.buckets = a.bucket_choices != 0, vs.bkmask = ((uint32_t)slots >> 2) - 1u, vs.dupflag = &s_dup;
+    vs.skew = a.bucket_choices == 4 ? wave : -1;
     (void)slots;
 
     constexpr int GPW = 64 / G;                    // row groups per wave
@@ -202,7 +283,7 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
 
         for (int i = tid; i < a.table_words; i += NT) table[i] = 0u;
         for (int i = tid; i < dim; i += NT) qs[i] = a.queries[(size_t)qid * dim + i];
-        if (tid == 0) s_ncand = 0, s_cntf = 0, s_nover = 0, s_cursor = 0, s_ntodo2 = 0;
+        if (tid == 0) s_ncand = 0, s_cntf = 0, s_nover = 0, s_cursor = 0, s_ntodo2 = 0, s_dup = 0;
         if (tid == 0) s_rows_screened = 0, s_rows_exact = 0, s_beam_words = 0;
         __syncthreads();
 
@@ -835,7 +916,37 @@ __global__ __launch_bounds__(1024) void beam_search_kernel(const SearchArgs a) {
                     }
                 }
                 __syncthreads();
-                const int tall = s_ntodo, T = tall - tprev;
+                int tall = s_ntodo;
+                if (vs.buckets) {
+                    // (read by every thread behind the barrier above; the next chunk's inserts lie behind the barrier
+                    // at its start)
+                    if (s_dup != 0) {
+                        // Two threads may have inserted the same id at the same time (see VisitedSet): an id of this
+                        // chunk that stands in the list before is struck out, and the list closed up.  An id's first
+                        // entry is never struck, so the later ones find it whatever else is struck meanwhile.
+                        for (int i = tprev + tid; i < tall; i += NT) {
+                            const uint32_t id = todo[i];
+                            bool rep = false;
+                            for (int j = tprev; j < i && !rep; ++j) rep = todo[j] == id;
+                            if (rep) todo[i] = 0xffffffffu;
+                        }
+                        __syncthreads();
+                        if (wave == 0) {
+                            int out = tprev;
+                            for (int i0 = tprev; i0 < tall; i0 += 64) {
+                                const int i = i0 + lane;
+                                const uint32_t id = i < tall ? todo[i] : 0xffffffffu;
+                                const uint64_t m = __ballot(id != 0xffffffffu);
+                                if (id != 0xffffffffu) todo[out + prefix_popc(m)] = id;  // (out + rank <= i: the chunk was read whole before)
+                                out += __popcll(m);
+                            }
+                            if (lane == 0) s_ntodo = out, s_dup = 0, atomicAdd(a.spill_count + 1, 1);
+                        }
+                        __syncthreads();
+                        tall = s_ntodo;
+                    }
+                }
+                const int T = tall - tprev;
                 nd += T;
                 PHASE_MARK(3);
                 if (!screening && ncand_u + T > CCAP) merge();  // merge() starts and ends with a barrier

@@ -268,6 +268,25 @@ int coral_index_info(const coral_index* idx, int64_t* n, int32_t* dim, int32_t* 
     return CORAL_OK;
 }
 
+// Size (log2 of the cells) of the visited table for ids that leave a 16-bit cell little room: see plan_search.
+// want: the size the load asks for; choices: the caller's coral_tuning.visited_choices.
+static int size_for_wide_ids(int want, int id_bits, int choices, bool* three) {
+    *three = false;
+    if (choices != 1) {
+        // the bucket form wherever its cells have room for the ids at the size the load asks for (it is the faster
+        // form at any load: three reads side by side against a probe sequence: +7 % at L = 256 on a million nodes);
+        // at a larger size only for ids that would leave linear probing short displacements, or when asked for
+        int w3 = want;
+        while (w3 < 16 && id_bits - (w3 - 2) > 14) ++w3;
+        if (id_bits - (w3 - 2) <= 14 && (w3 == want || choices == 3 || id_bits - want > 11)) {
+            *three = true;
+            return w3;
+        }
+    }
+    while (want < 16 && id_bits - want > 11) ++want;
+    return want;
+}
+
 // Launch geometry of the workgroup-per-query kernel for a beam of capacity L: arithmetic, the kernel's LDS
 // attribute and an occupancy query; nothing is allocated.  bump_log2 raises the library's own choice of table size.
 static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral_tuning& t, int bump_log2,
@@ -325,6 +344,10 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         return coral::search_lds_bytes(L, idx->dim, (1 << lg) >> 1, cap, cap, 256, big, screen) + kStaticLds;
     };
     const bool bitmap_possible = idx->n <= ((int64_t)1 << 21);
+    if (t.visited_choices != 0 && t.visited_choices != 1 && t.visited_choices != 3 && t.visited_choices != 4)
+        return fail(CORAL_ERR_ARG, "visited_choices must be 0, 1, 3 or 4 (got %d)", t.visited_choices);
+    const int choices = t.visited_choices == 4 ? 3 : t.visited_choices;  // (4: the bucket form as tests want it)
+    bool three = false;  // the table of cells in its bucket form
     int slots_log2 = t.visited_slots_log2;
     if (slots_log2 == -1) {
         if (!bitmap_possible || lds_bitmap(p.big, min_cap) > lds_max)
@@ -338,8 +361,10 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         while ((1 << want) < 112 * L && want < 20) ++want;
         // A 16-bit cell of a 2^s table keeps id_bits - s bits of the id and has the rest for the displacement: beyond
         // 2^24 ids a table sized for the load alone carries displacements of 14 or fewer, and a few ids of every
-        // query would leave LDS for the bitmap in global memory.  Such launches take the table that carries 30.
-        while (want < 16 && id_bits - want > 11) ++want;
+        // query would leave LDS for the bitmap in global memory.  Such launches take the table in its bucket form
+        // (three candidate buckets of four cells per id: no displacement to carry, 14 bits of the id per cell), at the
+        // size the load asks for where the cells have room for the ids; or else the table that carries 30.
+        want = size_for_wide_ids(want, id_bits, choices, &three);
         want += bump_log2;
         const bool table_holds = !p.big && want <= 16 && lds_table(false, want, min_cap) <= lds_max;
         const bool table_alone_on_cu = table_holds && lds_table(false, want, min_cap) > lds_max / 2;
@@ -358,7 +383,7 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         } else {
             slots_log2 = 12;
             while ((1 << slots_log2) < 48 * L && slots_log2 < 16) ++slots_log2;
-            while (slots_log2 < 16 && id_bits - slots_log2 > 11) ++slots_log2;  // (displacements up to 30, as above)
+            slots_log2 = size_for_wide_ids(slots_log2, id_bits, choices, &three);  // (as above)
             slots_log2 = std::min(16, slots_log2 + bump_log2);
             while (slots_log2 > 12 && lds_table(p.big, slots_log2, min_cap) > lds_max) --slots_log2;
         }
@@ -373,6 +398,17 @@ static int plan_search(const coral_index* idx, int32_t Q, int32_t L, const coral
         // a cell is 1 + ((d << rem_bits) | remainder) in 16 bits
         p.dmax = p.rem_bits >= 16 ? -1 : std::min(63, (65535 >> p.rem_bits) - 1);
         p.vis_limit = p.dmax < 0 ? 0 : slots - slots / 4;
+        // the bucket form: a cell is 1 + ((choice << rem_bits) | remainder), the remainder what the bucket index (a
+        // quarter of the cells) does not imply; a lookup costs the same whatever the load, so nothing is frozen
+        const int rem3 = std::max(0, id_bits - (slots_log2 - 2));
+        if (choices == 3 && t.visited_slots_log2 > 0) three = true;
+        if (three && rem3 > 14) {
+            if (choices == 3)
+                return fail(CORAL_ERR_ARG, "ids of %d bits do not fit the cells of a 2^%d table in its bucket form", id_bits,
+                            slots_log2);
+            three = false;  // (LDS had no room for the size that was asked for)
+        }
+        if (three) p.choices = t.visited_choices == 4 ? 4 : 3, p.rem_bits = rem3, p.dmax = 0, p.vis_limit = 0x7fffffff;
         p.spill_words = ((size_t)idx->n + 31) / 32;
     } else {
         p.table_words = bitmap_words, ocap = 4;
@@ -693,6 +729,7 @@ static coral::SearchArgs search_args(const coral_index* idx, const coral_search_
     a.id_bits = p.id_bits, a.rem_bits = p.rem_bits, a.dmax = p.dmax, a.ocap = p.ocap;
     a.beam_stride = p.beam_stride, a.direct_bitmap = p.direct, a.table_words = p.table_words;
     a.prefetch_rows = p.prefetch;
+    a.bucket_choices = p.choices;
     a.vec16 = p.screen == 1 ? idx->d_vec16 : nullptr, a.stride16 = coral::half_row_stride(idx->dim);
     a.vec8 = p.screen == 2 ? idx->d_vec8 : nullptr, a.stride8 = coral::byte_row_stride(idx->dim);
     a.tcap2 = p.screen ? coral::search_exact_list_cap(p.tcap) : 0;
@@ -779,7 +816,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     float ms = 0.f, ms_kernel = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
     HIP_TRY(hipEventElapsedTime(&ms_kernel, ev0, evk));
-    int scal[2] = {0, 0};
+    int scal[3] = {0, 0, 0};
     HIP_TRY(hipMemcpyAsync(scal, idx->d_scalars, sizeof scal, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
 #ifdef CORAL_PHASE_TIMERS
@@ -795,11 +832,31 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
     }
 #endif
     idx->last_Q = Q;
+    coral_stats sum;
+    std::memset(&sum, 0, sizeof sum);
+    sum.time_s = ms / 1000.0, sum.kernel_s = ms_kernel / 1000.0;
+    for (int q = 0; q < Q; ++q) {
+        const int32_t* c = idx->h_counters + (size_t)q * 4;
+        sum.hops += c[0], sum.expansions += c[1], sum.dist_evals += c[2], sum.rounds += c[3];
+        const int32_t* r = idx->h_counters + (size_t)Q * 4 + (size_t)q * 4;
+        sum.screened_rows += r[0], sum.exact_rows += r[1], sum.beam_words += r[2], sum.visited_requests += r[3];
+    }
+    sum.spills = scal[1], sum.visited_dedupes = scal[2];
     // The table size the library picks assumes about 75 first visits per beam entry.  Data on which a query visits
     // more sends queries to the global bitmap (same results, slower): when more than a twentieth of a batch went
-    // there, the next launches get a table twice the size.
+    // there, the next launches get a table twice the size.  (The bucket form turns away only the ids that find their
+    // three buckets full, a handful per query at a load where linear probing freezes the table: it takes the larger
+    // table only when more than a fiftieth of all first visits went to the bitmap.)
     const bool lds_table = !(policy == CORAL_POLICY_BEST_FIRST && idx->bf_ready) && !plan.big;
-    if (lds_table && idx->tuning.visited_slots_log2 == 0 && (int64_t)scal[1] * 20 > Q && plan.slots_log2 < 16) {
+    bool grow = lds_table && idx->tuning.visited_slots_log2 == 0 && (int64_t)scal[1] * 20 > Q && plan.slots_log2 < 16;
+    if (grow && plan.choices != 0 && sum.visited_requests / 2 * 50 <= sum.dist_evals) {
+        // few ids left LDS: the larger table is worth taking only if it costs the CU no workgroup
+        coral_search_plan peek;
+        const int next = (idx->bump_L == idx->L ? idx->bump_log2 : 0) + 1;
+        grow = plan_search(idx, idx->Q, idx->L, idx->tuning, next, false, plan.screen == 0, &peek) == CORAL_OK &&
+               !peek.direct && peek.workgroups >= plan.workgroups;
+    }
+    if (grow) {
         const int had = plan.slots_log2;
         idx->bump_log2 = idx->bump_L == idx->L ? idx->bump_log2 + 1 : 1;
         idx->bump_L = idx->L;
@@ -809,20 +866,7 @@ int coral_search_gpu(coral_index* idx, const float* d_queries, int32_t* d_ids, f
             if (!idx->prepared) return fail(CORAL_ERR_DEVICE, "could not restore the search scratch");
         }
     }
-    if (stats) {
-        std::memset(stats, 0, sizeof *stats);
-        stats->time_s = ms / 1000.0;
-        stats->kernel_s = ms_kernel / 1000.0;
-        for (int q = 0; q < Q; ++q) {
-            const int32_t* c = idx->h_counters + (size_t)q * 4;
-            stats->hops += c[0], stats->expansions += c[1];
-            stats->dist_evals += c[2], stats->rounds += c[3];
-            const int32_t* r = idx->h_counters + (size_t)Q * 4 + (size_t)q * 4;
-            stats->screened_rows += r[0], stats->exact_rows += r[1];
-            stats->beam_words += r[2], stats->visited_requests += r[3];
-        }
-        stats->spills = scal[1];
-    }
+    if (stats) *stats = sum;
     return CORAL_OK;
 }
 
@@ -923,7 +967,7 @@ int coral_search_plan_info(const coral_index* idx, coral_plan_info* out) {
         out->kernel = 0;
         out->threads = p.threads, out->workgroups = p.workgroups, out->lds_bytes = (int32_t)p.lds_bytes;
         out->screening = p.screen;
-        out->visited_form = p.direct ? 1 : 0;
+        out->visited_form = p.direct ? 1 : p.choices != 0 ? 5 : 0;
         out->visited_slots_log2 = p.direct ? 0 : p.slots_log2;
         out->beam_in_hbm = p.big;
         out->todo_cap = p.tcap, out->cand_cap = p.ccap;

@@ -27,6 +27,7 @@ struct coral_search_plan {
     int screen = 0;           // rows are screened before their fp32 row is read: 1 in half precision, 2 in eight-bit codes
     int slots_log2 = 0, table_words = 0, vis_limit = 0, tcap = 0, ccap = 0, threads = 512, workgroups = 0;
     int id_bits = 0, rem_bits = 0, dmax = 0, ocap = 0;
+    int choices = 0;          // 3: the table of cells in its bucket form (three candidate buckets per id)
     size_t lds_bytes = 0;
     size_t spill_words = 0;   // words of one workgroup's overflow bitmap in global memory (0: never used)
     size_t beam_stride = 0;   // 64-bit words of one workgroup's beam block in global memory (0 unless big)

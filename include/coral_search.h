@@ -93,6 +93,8 @@ typedef struct {
     int64_t beam_words;     /* 32-bit words of beam state (keys, expand lists, long runs) read or written in global
                                memory by passes over a beam that does not live in LDS */
     int64_t visited_requests; /* tests and marks of the visited state that went to global memory */
+    int64_t visited_dedupes;  /* lists of new ids that the bucket form of the visited table had searched for repeats
+                                 (two threads inserted the same id at the same time) */
 } coral_stats;
 
 /* Optional launch tuning; zero-initialise for defaults. */
@@ -129,16 +131,24 @@ typedef struct {
                                    runs of L keys per query slot): 1 = that form whatever L is, -1 = never (beams
                                    beyond CORAL_MAX_LDS_BEAM then run on the workgroup-per-query kernel), 0 = by L */
     int32_t best_first_buffer;  /* keys of that insert buffer, a multiple of 64 in 64..4096; 0 = 512 */
-    int32_t screening;          /* rows of more than 128 floats (rounds policy on codes: more than 64): every row is
-                                   first measured in a smaller copy of the vectors (made on first use) and its fp32
-                                   row is read only if rigorous bounds on the exact distance leave open whether it
+    int32_t screening;          /* every row is first measured in a smaller copy of the vectors (made on first use) and its
+                                   fp32 row is read only if rigorous bounds on the exact distance leave open whether it
                                    is a candidate or a beam entry; results and counters are the same bit for bit.
-                                   2 = a copy in eight-bit codes (256 bytes per row at dim 200; rows of up to 512
-                                   floats), 1 = a half-precision copy (512 bytes per row at dim 200; L2 only),
-                                   -1 = off, 0 = the eight-bit copy where it applies, else the half-precision one,
-                                   where the memory for it is there.  Best-first: beams of 410 .. 1280 entries screen
-                                   on codes (in half precision under 1, or for rows beyond 512 floats), longer ones
-                                   on codes up to L = 8192 (under 2: whatever L). */
+                                   2 = a copy in eight-bit codes (256 bytes per row at dim 200): rows of 68 .. 2048
+                                   floats under the rounds policy, 68 .. 512 under best-first; 1 = a half-precision
+                                   copy (512 bytes per row at dim 200): L2 only, rows of more than 128 floats;
+                                   -1 = off; 0 = the library's choice where the memory for the copy is there: rows of
+                                   more than 128 floats on codes (L2 rows of more than 1024 floats in half precision)
+                                   under the rounds policy; under best-first rows of 132 .. 512 floats on codes for
+                                   beams of 410 entries and more. */
+    int32_t visited_choices;    /* form of the table of 16-bit cells: 1 = open addressing with linear probing (a cell
+                                   carries its displacement), 3 = buckets of four cells, three candidate buckets per
+                                   id (a cell carries which of the three: 14 bits of the id per cell whatever the
+                                   load; ids of up to 12 bits more than the table has cells); 0 = linear probing
+                                   unless the ids are so wide that a cell could carry displacements below 30
+                                   (beyond 2^24 ids); 4 = form 3 with the bucket picked by the inserting wavefront's
+                                   number instead of by the load: same results, for tests of the path that two
+                                   threads take when they insert one id at the same time */
 } coral_tuning;
 
 CORAL_API const char* coral_last_error(void);
@@ -224,7 +234,8 @@ typedef struct {
     int32_t screen_row_bytes;/* bytes of one row of the smaller copy (0 without screening) */
     int32_t visited_form;    /* 0 table of 16-bit cells in LDS + bitmap in global memory, 1 bitmap of all ids in LDS,
                                 2 bytes per node and slot in global memory, 3 packed words in global memory,
-                                4 table of 16-bit cells in LDS in front of form 2 or 3 */
+                                4 table of 16-bit cells in LDS in front of form 2 or 3, 5 form 0 with the table in
+                                its bucket form (three candidate buckets of four cells per id) */
     int32_t visited_slots_log2; /* cells of the LDS table (forms 0 and 4), else 0 */
     int32_t beam_in_hbm;     /* the beam (or the long run) lives in global memory */
     int32_t todo_cap, cand_cap; /* LDS list capacities of the workgroup kernel */

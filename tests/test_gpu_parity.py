@@ -113,6 +113,70 @@ def test_exact_against_same_order_oracle(orc, case):
         if slots == 11 and (policy == 0 or in_lds):
             assert st.spills > 0
         check_row_counters(idx, st, cnt, M, policy)
+    # the table of 16-bit cells in its bucket form (three candidate buckets of four cells per id; what the library
+    # takes by itself only beyond 2^24 ids): at the library's size, at the case's own, and one so small that most
+    # ids find their three buckets full and go to the bitmap in global memory
+    for s3 in sorted({0, slots, 10}):
+        idx.prepare(q.shape[0], L, visited_slots_log2=s3, visited_choices=3, threads=threads, policy=policy,
+                    best_first_in_lds=policy == 1)
+        # (where the library sizes the visited set itself it may still prefer a bitmap of all ids)
+        assert idx.plan_info().visited_form == 5 or (s3 == 0 and idx.plan_info().visited_form == 1)
+        ids, dists, st = idx.search(q, k, L, policy=policy)
+        assert np.array_equal(ids, oi), s3
+        assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), s3
+        assert np.array_equal(idx.query_counters(q.shape[0]), os_), s3
+        if s3 == 10 and L >= 128 and policy == 0 and R == 32:
+            assert st.spills > 0
+    idx.close()
+
+
+def test_bucket_table_when_many_threads_insert_the_same_id(orc):
+    """The bucket form of the visited table puts a new id into the emptiest of its three buckets, as the inserting
+    thread sees them: two threads that meet the same unvisited id at the same time can put it into different buckets
+    and both call it new.  The kernel notices (each looks at the other buckets after its insert) and strikes the
+    repeats from the list of new ids.  A graph made for it: most of a row's neighbours come from a pool of a few
+    hundred popular nodes, so the 32 rows of a chunk list the same unvisited ids many times over.  Ids, distance bits
+    and counters equal the oracle's, whatever the table size and the workgroup's width; the number of lists that had
+    to be searched for repeats is printed."""
+    n, dim, R, Q, L, k = 30000, 64, 32, 200, 256, 50
+    base = synth.gaussian_matrix(5, n, dim)
+    near = gpu_graph(base, 8)
+    rng = np.random.RandomState(6)
+    pool = rng.choice(n, 600, replace=False).astype(np.int32)
+    nbrs = np.empty((n, R), np.int32)
+    for i0 in range(0, n, 4096):  # 24 distinct popular nodes per row, then the row's 8 nearest
+        m = min(4096, n - i0)
+        pick = np.argsort(rng.rand(m, pool.size), axis=1)[:, :R - 8]
+        nbrs[i0:i0 + m, :R - 8] = pool[pick]
+        nbrs[i0:i0 + m, R - 8:] = near[i0:i0 + m]
+    for i in range(n):  # a row lists an id once (and never its own node)
+        row = nbrs[i]
+        keep = [v for j, v in enumerate(row) if v != i and v not in row[:j]]
+        nbrs[i] = -1
+        nbrs[i, :len(keep)] = keep
+    starts = rng.choice(n, 16, replace=False).astype(np.int32)
+    q = make_queries(Q, dim, 71)
+    prob = orc.Problem(base, nbrs, starts)
+    oi, od, os_, _ = orc.search_B(prob, q, k, L, start_order=WAVE64, nbr_order=WAVE64)
+    idx = capi.Index(base, nbrs, starts)
+    dedupes = {3: 0, 4: 0}
+    for choices in (3, 4):  # 4: the bucket is picked by the inserting wavefront's number, so concurrent inserts part
+        for slots in (0, 12, 14):
+            for threads in (256, 512, 1024):
+                idx.prepare(Q, L, visited_slots_log2=slots, visited_choices=choices, threads=threads)
+                for _ in range(3):
+                    ids, dists, st = idx.search(q, k, L)
+                    assert np.array_equal(ids, oi), (choices, slots, threads)
+                    assert dists.view(np.uint32).tolist() == od.view(np.uint32).tolist(), (choices, slots, threads)
+                    assert np.array_equal(idx.query_counters(Q), os_), (choices, slots, threads)
+                    dedupes[choices] += st.visited_dedupes
+    print("lists of new ids searched for repeats: %s" % dedupes, flush=True)
+    assert dedupes[4] > 0  # the path was taken
+    # best-first on the workgroup kernel goes through the same table
+    oi, od, os_, _ = orc.search_A(prob, q, k, L, order=WAVE64)
+    idx.prepare(Q, L, policy=1, best_first_in_lds=True, visited_slots_log2=13, visited_choices=4)
+    ids, dists, st = idx.search(q, k, L, policy=1)
+    assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes() and np.array_equal(idx.query_counters(Q), os_)
     idx.close()
 
 
