@@ -544,8 +544,13 @@ def main():
                                            "distance evaluation, a 128-byte graph row per expansion; the screening "
                                            "reads fewer, so this can exceed the peak"}},
     }
+    # the same two figures under the names a bounded "scheme" roofline goes by: every byte the launch's scheme moves,
+    # its own beam passes and visited-state requests included
+    out["roofline"]["scheme_bytes"] = head["bytes_per_launch"] + head["scratch_bytes_per_launch"]
+    out["roofline"]["frac_scheme"] = head["frac_with_scratch"]
     if traffic:
         out["roofline"]["traffic_over_bytes"] = traffic["bytes"] / head["bytes_per_launch"]
+        out["roofline"]["traffic_over_scheme_bytes"] = traffic["bytes"] / out["roofline"]["scheme_bytes"]
     if also:
         out["also"] = also
 
