@@ -72,7 +72,42 @@ class BuildParams(C.Structure):
     _fields_ = [("R", C.c_int32), ("k_b", C.c_int32), ("batch", C.c_int32), ("need_discard", C.c_int32),
                 ("connect_enhance", C.c_int32), ("enhance_search_batch", C.c_int32), ("enhance_nap_batch", C.c_int32),
                 ("enhance_L", C.c_int32), ("n_start", C.c_int32), ("first_start_id", C.c_int32),
-                ("top_hit_num", C.c_int32), ("reserved", C.c_int32 * 5)]
+                ("top_hit_num", C.c_int32), ("test_search_frequency", C.c_int32), ("monitor", C.c_void_p),
+                ("reserved", C.c_int32 * 2)]
+
+
+MONITOR_BATCHES, MONITOR_ISOLATED, MONITOR_TOP, MONITOR_DONE = 0, 1, 2, 3
+BUILD_REPORT_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.POINTER(Stats), C.c_int64)
+
+
+class BuildMonitor(C.Structure):
+    _fields_ = [("h_queries", C.c_void_p), ("h_gt", C.c_void_p), ("Q", C.c_int32), ("k", C.c_int32), ("L", C.c_int32),
+                ("reserved", C.c_int32), ("report", BUILD_REPORT_FN), ("user", C.c_void_p)]
+
+
+class Monitor:
+    """GPUFuncs::test_search during a build: `queries` [Q][dim] searched with beam L and compared with their true
+    neighbours `gt` [Q][k] at the points where the reference does it.  Attach to build parameters with `attach`;
+    `reports` then collects (phase, done, total, hits, hops, kernel seconds) per search.  Keep the object alive
+    while the build runs."""
+
+    def __init__(self, queries, gt, L):
+        self.queries = np.ascontiguousarray(queries, dtype=np.float32)
+        self.gt = np.ascontiguousarray(gt, dtype=np.int32)
+        self.reports = []
+
+        def report(_user, phase, done, total, st, hits):
+            self.reports.append((phase, done, total, hits, st.contents.hops, st.contents.kernel_s))
+
+        self._fn = BUILD_REPORT_FN(report)
+        self.c = BuildMonitor(self.queries.ctypes.data, self.gt.ctypes.data, self.queries.shape[0], self.gt.shape[1], L,
+                              0, self._fn, None)
+
+    def attach(self, params, every_batches=None):
+        params.monitor = C.addressof(self.c)
+        if every_batches is not None:
+            params.test_search_frequency = every_batches
+        return params
 
 
 class BuildStats(C.Structure):
@@ -133,6 +168,7 @@ SIGNATURES = {
                                                 C.c_void_p, C.c_void_p]),
     "coral_build_resume": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_build_top_hit_ids": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
+    "coral_build_test_search": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64]),
     "coral_build_connect_enhance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "coral_build_graph": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "coral_build_graph_from_clusters": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
@@ -383,6 +419,10 @@ class Index:
         self.R = params.R
         self._refresh_n_start()
         return st
+
+    def build_test_search(self, params, phase=MONITOR_DONE, done=0, total=0):
+        """GPUFuncs::test_search on the graph as it stands, reported to the monitor attached to `params`."""
+        _check(lib().coral_build_test_search(self._h, C.byref(params), phase, done, total))
 
     def build_graph_from_clusters(self, clusters, params):
         """The construction from precomputed clusters, int32 [A][k_b] (the reference's --train_gt_file)."""

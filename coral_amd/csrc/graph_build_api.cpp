@@ -5,6 +5,7 @@
 //   coral_build_enhance_batch    GPUFuncs::enhance_neibor_aware_gpu src/enhance.cu:660-689
 //   coral_build_enhance_top_batch  its five-argument form      src/enhance.cu:632-658 (most-hit nodes, :819-856)
 //   coral_build_resume           Graph ctor in Mode::CE        include/graph.cuh:252-256 (rows of a saved build)
+//   coral_build_test_search      GPUFuncs::test_search         include/gpufuncs.cuh:688-702 (and its calls during a build)
 #include <algorithm>
 #include <chrono>
 #include <climits>
@@ -81,6 +82,53 @@ int ensure_stage(coral_index* idx, size_t rows) {
     return CORAL_OK;
 }
 
+// GPUFuncs::test_search (include/gpufuncs.cuh:688-702) on the graph as it stands: prepare for (Q, L), one search from
+// the index's current start ids, the hit count against the true neighbours, and the caller's report.  With
+// fresh_starts (the calls between batches, when the index has no entry points yet) the start ids are sampled first,
+// as the enhancement does for its own searches; they are replaced again before the build ends.
+int monitor_search(coral_index* idx, const coral_build_params* prm, int32_t phase, int64_t done, int64_t total,
+                   bool fresh_starts) {
+    const coral_build_monitor* m = prm->monitor;
+    if (!m || !m->report) return CORAL_OK;
+    if (!m->h_queries || !m->h_gt || m->Q < 1 || m->k < 1 || m->k > m->L)
+        return fail(CORAL_ERR_ARG, "build monitor: queries, true neighbours, Q >= 1 and 1 <= k <= L are needed");
+    if (fresh_starts) {
+        std::vector<int32_t> deg((size_t)idx->n), starts((size_t)prm->n_start);
+        HIP_TRY(hipMemcpyAsync(deg.data(), idx->d_deg, (size_t)idx->n * sizeof(int32_t), hipMemcpyDeviceToHost, idx->stream));
+        HIP_TRY(hipStreamSynchronize(idx->stream));
+        int32_t first = prm->first_start_id;
+        if (first < 0 || first >= idx->n || deg[first] == 0) {
+            first = -1;
+            for (int64_t i = 0; i < idx->n && first < 0; ++i)
+                if (deg[i] > 0) first = (int32_t)i;
+        }
+        if (first < 0) return CORAL_OK;  // nothing to search from yet
+        if (int rc = coral_start_ids_fps(idx, first, prm->n_start, starts.data())) return rc;
+        if (int rc = set_start_ids(idx, starts.data(), prm->n_start)) return rc;
+    }
+    float* d_q = nullptr;
+    int32_t *d_gt = nullptr, *d_res = nullptr;
+    const size_t qb = (size_t)m->Q * idx->dim * sizeof(float), rb = (size_t)m->Q * m->k * sizeof(int32_t);
+    int rc = CORAL_OK;
+    if (hipMalloc(&d_q, qb) != hipSuccess || hipMalloc(&d_gt, rb) != hipSuccess || hipMalloc(&d_res, rb) != hipSuccess) {
+        (void)hipGetLastError();
+        rc = fail(CORAL_ERR_MEMORY, "build monitor: device allocation failed");
+    } else if (hipMemcpy(d_q, m->h_queries, qb, hipMemcpyHostToDevice) != hipSuccess ||
+               hipMemcpy(d_gt, m->h_gt, rb, hipMemcpyHostToDevice) != hipSuccess) {
+        rc = fail(CORAL_ERR_DEVICE, "build monitor: upload failed");
+    }
+    coral_stats st{};
+    int64_t hits = 0;
+    coral_tuning tun{};
+    tun.policy = CORAL_POLICY_ROUNDS;
+    if (rc == CORAL_OK) rc = coral_search_prepare(idx, m->Q, m->L, &tun);
+    if (rc == CORAL_OK) rc = coral_search_gpu(idx, d_q, d_res, nullptr, m->Q, m->k, CORAL_POLICY_ROUNDS, 0, nullptr, &st);
+    if (rc == CORAL_OK) rc = coral_search_verify(idx, d_res, d_gt, m->Q, m->k, &hits);
+    (void)hipFree(d_q), (void)hipFree(d_gt), (void)hipFree(d_res);
+    if (rc == CORAL_OK) m->report(m->user, phase, done, total, &st, hits);
+    return rc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -91,6 +139,7 @@ int coral_build_params_default(coral_build_params* p) {
     p->R = 32, p->k_b = 100, p->batch = 1024, p->need_discard = 1, p->connect_enhance = 1;
     p->enhance_search_batch = 524288, p->enhance_nap_batch = 4096, p->enhance_L = 256;
     p->n_start = 16, p->first_start_id = -1;
+    p->test_search_frequency = 100;
     return CORAL_OK;
 }
 
@@ -354,10 +403,12 @@ int coral_build_connect_enhance(coral_index* idx, const coral_build_params* prm,
                 if (stats && top) stats->top_reverse_edges += ins;
                 if (stats && !top) stats->reverse_edges += ins, stats->reverse_rejected += rej;
             }
+            if (rc == CORAL_OK && top) rc = monitor_search(idx, prm, CORAL_MONITOR_TOP, i + batch, count, false);
         }
         (void)hipFree(d_ids), (void)hipFree(d_res), (void)hipFree(d_vecs), (void)hipFree(d_res_d);
     };
     if (iso_num > 0) phase(iso, false);
+    if (rc == CORAL_OK && iso_num > 0) rc = monitor_search(idx, prm, CORAL_MONITOR_ISOLATED, iso_num, iso_num, false);
     // src/enhance.cu:819-856: the nodes most clusters contain, as many as top_hit_num exceeds the isolated ones
     int64_t top_n = rc == CORAL_OK && prm->top_hit_num > iso_num ? std::min<int64_t>(prm->top_hit_num - iso_num, n) : 0;
     if (top_n > 0) {
@@ -372,6 +423,13 @@ int coral_build_connect_enhance(coral_index* idx, const coral_build_params* prm,
         rc = set_start_ids(idx, starts.data(), prm->n_start);
     }
     return rc;
+}
+
+int coral_build_test_search(coral_index* idx, const coral_build_params* prm, int32_t phase, int64_t done, int64_t total) {
+    if (!idx || !prm) return fail(CORAL_ERR_ARG, "null argument");
+    if (!idx->d_nbrs || idx->M < 1) return fail(CORAL_ERR_STATE, "the index has no graph or no start ids to search from");
+    HIP_TRY(hipSetDevice(idx->device));
+    return monitor_search(idx, prm, phase, done, total, false);
 }
 
 // the construction from auxiliary queries (h_aux) or from their precomputed clusters (h_clusters)
@@ -418,7 +476,11 @@ static int build_impl(coral_index* idx, const float* h_aux, const int32_t* h_clu
         for (int64_t b0 = 0; b0 < cq; b0 += prm->batch) {
             const int b = (int)std::min<int64_t>(prm->batch, cq - b0);
             if ((rc = coral_build_nap_batch(idx, d_knn + (size_t)b0 * kb, b, kb, prm->need_discard))) break;
-            ++S->batches;
+            const int64_t batch_id = S->batches++;
+            if (prm->monitor && prm->test_search_frequency > 0 && batch_id > 0 &&
+                batch_id % prm->test_search_frequency == 0 &&
+                (rc = monitor_search(idx, prm, CORAL_MONITOR_BATCHES, a0 + b0 + b, A, true)))
+                break;
         }
         S->nap_s += now_s() - t1;
     }
@@ -442,6 +504,7 @@ static int build_impl(coral_index* idx, const float* h_aux, const int32_t* h_clu
         if ((rc = set_start_ids(idx, starts.data(), prm->n_start))) return rc;
     }
     S->enhance_s = now_s() - t2;
+    if (prm->connect_enhance && (rc = monitor_search(idx, prm, CORAL_MONITOR_DONE, A, A, false))) return rc;
     std::vector<int32_t> deg((size_t)idx->n);
     HIP_TRY(hipMemcpy(deg.data(), idx->d_deg, (size_t)idx->n * sizeof(int32_t), hipMemcpyDeviceToHost));
     for (int32_t d : deg) S->edges += d;

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cctype>
 #include <cstdlib>
 #include <cstring>
@@ -91,6 +92,8 @@ void IndexGPU::load_config(const std::string& config_file) {
     if (json_number(text, "enhance_nap_batch", &v)) pc.enhance_nap_batch = (int)v;
     if (json_number(text, "top_hit_num", &v)) pc.top_hit_num = (int)v;
     if (json_number(text, "enhance_search_batch", &v)) pc.enhance_search_batch = (int)v;
+    if (json_number(text, "test_search", &v)) pc.test_search = (int)v;
+    if (json_number(text, "test_search_frequency", &v)) pc.test_search_frequency = (int)v;
 }
 
 void IndexGPU::LoadSearchNeededData(const char* base_file, const char* sampled_query_file, DIST_METRIC m) {
@@ -190,6 +193,51 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
     p.enhance_search_batch = PC.enhance_search_batch, p.enhance_nap_batch = PC.enhance_nap_batch;
     p.top_hit_num = PC.top_hit_num;
     p.n_start = PC.search_start_nodes_num;
+    p.test_search_frequency = PC.test_search_frequency;
+    // the test queries of the searches during the build: the first TEST_SEARCH_QUERY_SIZE = "batch" of query_test_file
+    // (include/uni.h:63) with their true neighbours from gt_test_file
+    std::vector<float> test_queries;
+    std::vector<int32_t> test_gt;
+    coral_build_monitor monitor{};
+    struct Sink {
+        IndexGPU* self;
+        int Q, k;
+    } sink{this, 0, 0};
+    test_reports.clear();
+    const std::string qt = parameters.Get<std::string>("query_test_file", std::string("None"));
+    const std::string gt = parameters.Get<std::string>("gt_test_file", std::string("None"));
+    if (PC.test_search && qt != "None" && !qt.empty() && gt != "None" && !gt.empty()) {
+        int64_t nq = 0;
+        int32_t qdim = 0, gn = 0, gk = 0;
+        if (coral_fbin_read_meta(qt.c_str(), &nq, &qdim)) raise("query_test_file");
+        if ((size_t)((qdim + 3) / 4 * 4) != row_width_) throw std::runtime_error("BuildGPU: test queries of another dimension");
+        if (coral_gt_read_meta(gt.c_str(), &gn, &gk)) raise("gt_test_file");
+        const int Q = (int)std::min<int64_t>({nq, (int64_t)gn, (int64_t)PC.batch});
+        const int gtk = std::min(k_, (int)gk);
+        if (Q > 0 && gtk > 0) {
+            test_queries.resize((size_t)Q * row_width_);
+            if (coral_fbin_read(qt.c_str(), test_queries.data(), Q, qdim, (int32_t)row_width_)) raise("query_test_file");
+            if (dist_metric_ == DIST_METRIC::IP_) coral_normalize_l2(test_queries.data(), Q, (int32_t)row_width_);
+            std::vector<int32_t> rows((size_t)gn * gk);
+            if (coral_gt_read(gt.c_str(), rows.data(), gn, gk)) raise("gt_test_file");
+            test_gt.resize((size_t)Q * gtk);
+            for (int q = 0; q < Q; ++q) std::copy_n(rows.data() + (size_t)q * gk, gtk, test_gt.data() + (size_t)q * gtk);
+            sink.Q = Q, sink.k = gtk;
+            monitor.h_queries = test_queries.data(), monitor.h_gt = test_gt.data();
+            monitor.Q = Q, monitor.k = gtk, monitor.L = std::max(PC.test_beam_capacity, gtk);
+            monitor.user = &sink;
+            monitor.report = [](void* user, int32_t phase, int64_t done, int64_t total, const coral_stats* st, int64_t h) {
+                Sink* s = (Sink*)user;
+                Test_Result res((int)h, (size_t)st->hops, (float)st->time_s);
+                const float recall = res.calc_recall(s->Q * s->k), avg_hops = res.avg_hops(s->Q);
+                static const char* const kWhen[] = {"batches", "isolated nodes attached", "most-hit nodes", "graph complete"};
+                std::cout << "[" << kWhen[phase & 3] << " " << done << "/" << total << "] Testing recall-" << recall
+                          << "%, avg_hops-" << avg_hops << ", cost_time-" << res.get_time() << "s" << std::endl;
+                s->self->test_reports.push_back(TestReport{phase, (long long)done, (long long)total, res});
+            };
+            p.monitor = &monitor;
+        }
+    }
     std::vector<uint32_t> hits(nd_);
     if (CE == 2) {
         // enhancement only (src/index_gpu.cpp:332-333, 367-373): the rows, their distances and the hit counts of an
@@ -202,6 +250,7 @@ void IndexGPU::BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data
         if (coral_build_resume(index_, max_degree_, nbrs_.data(), saved.data(), hits.data())) raise("BuildGPU");
         p.connect_enhance = 1;
         if (coral_build_connect_enhance(index_, &p, &last_build)) raise("BuildGPU");
+        if (coral_build_test_search(index_, &p, CORAL_MONITOR_DONE, (int64_t)nd_, (int64_t)nd_)) raise("BuildGPU");
     } else {
         const std::string train_gt = parameters.Get<std::string>("train_gt_file", std::string("None"));
         if (train_gt != "None" && !train_gt.empty()) {

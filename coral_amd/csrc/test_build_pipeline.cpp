@@ -146,6 +146,9 @@ int main(int argc, char** argv) {
         parameters.Set<std::string>("dist", dist);
         parameters.Set<std::string>("dataset", dataset);
         parameters.Set<std::string>("train_gt_file", str("train_gt_file").empty() ? "None" : str("train_gt_file"));
+        // tests/test_build_pipeline.cpp:215-216: BuildGPU searches these while the graph grows (config.json "test_search")
+        parameters.Set<std::string>("query_test_file", str("query_test_file"));
+        parameters.Set<std::string>("gt_test_file", str("gt_test_file"));
 
         IndexGPU index((size_t)base_stride, (size_t)(base_num + sq_num), dist_metric, nullptr);
         const auto s = std::chrono::high_resolution_clock::now();

@@ -294,6 +294,29 @@ CORAL_API int coral_start_ids_fps(coral_index* idx, int32_t first_id, int32_t M,
  * connectivity enhancement does).  Two outcomes that the reference leaves to thread timing are fixed here:
  * equal distances keep the order in which the candidates were listed (cluster order, then the current row),
  * and a node that several clusters (or several isolated nodes) of one batch claim goes to the first of them. */
+/* The search the reference runs on a set of test queries while a graph grows, GPUFuncs::test_search
+ * (include/gpufuncs.cuh:688-702: search_prepare(TEST_SEARCH_QUERY_SIZE, test_beam_capacity), Search with the current
+ * start ids, search_verify against the test queries' true neighbours): called every test_search_frequency batches
+ * (src/index_gpu.cpp:525-570), after the isolated nodes were attached (src/enhance.cu:814), after every search batch
+ * of the most-hit nodes (src/enhance.cu:852) and on the finished graph (src/index_gpu.cpp:376-378).  It changes
+ * nothing in the graph.  `report` is called once per such search, from the thread that runs the build. */
+#define CORAL_MONITOR_BATCHES 0  /* done = auxiliary queries consumed so far, total = all of them */
+#define CORAL_MONITOR_ISOLATED 1 /* done = total = isolated nodes attached */
+#define CORAL_MONITOR_TOP 2      /* done = most-hit nodes gone over so far, total = all of them */
+#define CORAL_MONITOR_DONE 3     /* the finished graph (only with connect_enhance, as in the reference) */
+typedef void (*coral_build_report_fn)(void* user, int32_t phase, int64_t done, int64_t total, const coral_stats* search,
+                                      int64_t hits);
+typedef struct {
+    const float* h_queries; /* host [Q][dim]: test_query_data */
+    const int32_t* h_gt;    /* host [Q][k]: test_query_knns, the k true nearest of each */
+    int32_t Q;              /* TEST_SEARCH_QUERY_SIZE (the reference: config.json "batch") */
+    int32_t k;              /* gtk */
+    int32_t L;              /* config.json "test_beam_capacity" (512) */
+    int32_t reserved;
+    coral_build_report_fn report; /* search->hops / Q = Test_Result::avg_hops, 100 hits / (Q k) = calc_recall */
+    void* user;
+} coral_build_monitor;
+
 typedef struct {
     int32_t R;                    /* row width, <= 32: --M_pjbp, tests/test_build_pipeline.cpp:82 */
     int32_t k_b;                  /* nearest base points per auxiliary query, 2..128: config.json "k" */
@@ -309,7 +332,10 @@ typedef struct {
     int32_t top_hit_num;          /* config.json "top_hit_num": after the isolated nodes, the (top_hit_num - isolated)
                                      nodes that most clusters contain are searched for and rewired too; 0 (the code's
                                      default, src/index_gpu.cpp:78) = no such phase */
-    int32_t reserved[5];
+    int32_t test_search_frequency; /* config.json "test_search_frequency" (100): a monitor search after every batch
+                                      whose number (from 0) is a positive multiple of it; 0 = none during the batches */
+    const coral_build_monitor* monitor; /* NULL (the default) = no test searches */
+    int32_t reserved[2];
 } coral_build_params;
 
 typedef struct {
@@ -364,6 +390,13 @@ CORAL_API int coral_build_enhance_batch(coral_index* idx, const int32_t* d_iso_i
  * number of isolated nodes: the (top_hit_num - isolated) nodes of coral_build_top_hit_ids, capped at n (the reference
  * reads past its id array beyond that), go through the same search and coral_build_enhance_top_batch. */
 CORAL_API int coral_build_connect_enhance(coral_index* idx, const coral_build_params* params, coral_build_stats* stats);
+
+/* GPUFuncs::test_search by itself (include/gpufuncs.cuh:688-702): one search of params->monitor's queries from the
+ * index's current start ids on the graph as it stands, reported through params->monitor->report with the phase and
+ * progress given.  Does nothing without a monitor.  (IndexGPU::BuildGPU's closing call, src/index_gpu.cpp:376-378,
+ * where the enhancement ran on a saved build.) */
+CORAL_API int coral_build_test_search(coral_index* idx, const coral_build_params* params, int32_t phase, int64_t done,
+                                      int64_t total);
 
 /* The five-argument GPUFuncs::enhance_neibor_aware_gpu (src/enhance.cu:632-658, 58-129): d_top_ids [batch] nodes that
  * have rows, d_knn_ids / d_knn_dists [batch][k] what the search found for their vectors (the node itself included, as

@@ -50,6 +50,8 @@ struct ProConfig {
     int enhance_nap_batch = 4096;
     int enhance_search_batch = 524288;
     int top_hit_num = 0;  // include/uni.h:124; the shipped config.json sets 5000000
+    int test_search = 1;             // include/uni.h:109: search the test queries while the graph grows
+    int test_search_frequency = 100; // include/uni.h:122: ... every so many batches
 };
 CORAL_API ProConfig& GetProConfig();
 #define PC (::efanna2e::GetProConfig())
@@ -119,6 +121,16 @@ class CORAL_API IndexGPU : public Index {
     // size), dist, graph_file, train_gt_file (optional: the clusters, as a ground-truth file of the sampled queries with k
     // ids per row; sq_data is then unused).  Both arrays hold rows of GetRowWidth() floats.  The built index stays loaded, so
     // Search works right after.  The timings and counts of the run are in last_build.
+    // With query_test_file and gt_test_file among the parameters (tests/test_build_pipeline.cpp:215-216) and
+    // config.json's "test_search" not 0, the first "batch" test queries are searched with beam test_beam_capacity while
+    // the graph grows (GPUFuncs::test_search, include/gpufuncs.cuh:688-702, at the points where the reference calls it)
+    // and a line per search goes to stdout in the wording of src/enhance_disk.cu:468-469; test_reports keeps them.
+    struct TestReport {
+        int phase;  // CORAL_MONITOR_*
+        long long done, total;
+        Test_Result result;
+    };
+    std::vector<TestReport> test_reports;
     void BuildGPU(size_t n_sq, float* sq_data, size_t n_bp, float* bp_data, Parameters& parameters);
     coral_build_stats last_build{};
     // src/index_gpu.cpp:138-206 with upd_type 0: the ids are tombstoned on the device (del_node_mark,

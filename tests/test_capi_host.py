@@ -32,6 +32,45 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == bound
 
 
+LAYOUT_PROBE = r"""
+#include <stddef.h>
+#include <stdio.h>
+#include "coral_search.h"
+#define S(t) printf(#t " size %zu\n", sizeof(t))
+#define F(t, f) printf(#t " " #f " %zu\n", offsetof(t, f))
+int main(void) {
+    S(coral_stats); F(coral_stats, hops); F(coral_stats, screened_rows); F(coral_stats, visited_dedupes);
+    S(coral_tuning); F(coral_tuning, visited_choices);
+    S(coral_plan_info); F(coral_plan_info, query_slots);
+    S(coral_build_params); F(coral_build_params, top_hit_num); F(coral_build_params, test_search_frequency);
+    F(coral_build_params, monitor);
+    S(coral_build_monitor); F(coral_build_monitor, L); F(coral_build_monitor, report); F(coral_build_monitor, user);
+    S(coral_build_stats); F(coral_build_stats, top_reverse_edges);
+    return 0;
+}
+"""
+
+
+def test_ctypes_structures_have_the_layout_of_the_header(tmp_path):
+    """What a C compiler makes of include/coral_search.h (the header is plain C) against the ctypes mirror that the
+    tests and bench.py call through: sizes and the offsets of the fields added last."""
+    (tmp_path / "probe.c").write_text(LAYOUT_PROBE)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(tmp_path / "probe.c"),
+                    "-o", str(tmp_path / "probe")], check=True)
+    out = subprocess.run([str(tmp_path / "probe")], capture_output=True, text=True, check=True).stdout
+    mirror = {"coral_stats": capi.Stats, "coral_tuning": capi.Tuning, "coral_plan_info": capi.PlanInfo,
+              "coral_build_params": capi.BuildParams, "coral_build_monitor": capi.BuildMonitor,
+              "coral_build_stats": capi.BuildStats}
+    lines = out.splitlines()
+    assert len(lines) >= 17
+    for line in lines:
+        if not line:
+            continue
+        name, what, value = line.split()
+        cls = mirror[name]
+        assert (ctypes.sizeof(cls) if what == "size" else getattr(cls, what).offset) == int(value), line
+
+
 def test_cxx_class_symbols_are_exported():
     out = subprocess.run(["nm", "-DC", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
     for sym in ("efanna2e::IndexGPU::Search(float const*, int, int, int*, int)",

@@ -267,6 +267,68 @@ def test_enhancement_alone_on_a_resumed_build_equals_the_whole_construction():
     idx.close()
 
 
+def test_searches_during_a_build_report_and_change_nothing(orc):
+    """GPUFuncs::test_search at the reference's points of a construction (include/gpufuncs.cuh:688-702; every
+    test_search_frequency batches src/index_gpu.cpp:525, after the isolated nodes src/enhance.cu:814, after every search
+    batch of the most-hit nodes :852, on the finished graph src/index_gpu.cpp:376-378): the watched construction ends
+    in the state of the unwatched one, and each report is the search it says it is."""
+    import torch
+    n, dim, A, Q, k, L = 12000, 48, 900, 64, 10, 64
+    base = base_of(n, dim, 311, capi.L2)
+    aux = make_queries(A, dim, 411)
+    q = make_queries(Q, dim, 511)
+    gt, _ = orc.bruteforce(base, q, k)
+    kw = dict(R=16, k_b=24, batch=128, enhance_search_batch=2500, enhance_nap_batch=700, enhance_L=64, n_start=8,
+              top_hit_num=9000)
+    idx = capi.Index(base, None, None)
+    idx.build_graph(aux, capi.build_params(**kw))
+    want = idx.get_graph(with_build_state=True)
+    idx.close()
+    mon = capi.Monitor(q, gt, L)
+    p = mon.attach(capi.build_params(**kw), every_batches=3)
+    idx = capi.Index(base, None, None)
+    stats = idx.build_graph(aux, p)
+    got = idx.get_graph(with_build_state=True)
+    for g, w in zip(got, want):
+        assert g.tobytes() == w.tobytes()
+    phases = [r[0] for r in mon.reports]
+    top_n = 9000 - stats.isolated
+    assert stats.batches == 8 and phases[:2] == [capi.MONITOR_BATCHES] * 2  # after the batches numbered 3 and 6
+    assert [r[1:3] for r in mon.reports[:2]] == [(512, A), (896, A)]
+    assert phases[2] == capi.MONITOR_ISOLATED and mon.reports[2][1:3] == (stats.isolated, stats.isolated)
+    tops = [r for r in mon.reports if r[0] == capi.MONITOR_TOP]
+    assert [r[1] for r in tops] == list(range(2500, top_n, 2500)) + [top_n] and all(r[2] == top_n for r in tops)
+    assert phases[-1] == capi.MONITOR_DONE and len(phases) == 3 + len(tops) + 1
+    # the last report against a search of the finished graph by hand, and against the oracle on that graph
+    d_q = dev(q)
+    d_ids = torch.empty((Q, k), dtype=torch.int32, device="cuda")
+    idx.prepare(Q, L)
+    st = idx.search_device(d_q.data_ptr(), d_ids.data_ptr(), None, Q, k)
+    hits = idx.verify(d_ids.data_ptr(), dev(gt).data_ptr(), Q, k)
+    assert mon.reports[-1][3] == hits and mon.reports[-1][4] == st.hops
+    oi, _, os_, _ = orc.search_B(orc.Problem(base, got[0], got[3]), q, k, L, start_order=WAVE64, nbr_order=WAVE64)
+    assert hits == orc.recall_hits(oi, gt, k) and st.hops == os_[:, 0].sum()
+    assert mon.reports[0][3] < mon.reports[2][3] <= Q * k
+    # GPUFuncs::test_search by itself: the same search again, reported under the phase the caller names
+    idx.build_test_search(p, capi.MONITOR_TOP, 5, 7)
+    assert mon.reports[-1][:5] == (capi.MONITOR_TOP, 5, 7, hits, st.hops)
+    idx.build_test_search(capi.build_params(**kw))  # no monitor: nothing happens
+    assert len(mon.reports) == len(phases) + 1
+    # a monitor that cannot be searched for is turned away before the build starts changing rows
+    bad = capi.Monitor(q, gt, k - 1)
+    with pytest.raises(capi.CoralError) as e:
+        idx.build_test_search(bad.attach(capi.build_params(**kw)))
+    assert e.value.code == capi.ERR_ARG
+    idx.close()
+    # without the enhancement there is no closing search (src/index_gpu.cpp:376: CE && test_search)
+    mon2 = capi.Monitor(q, gt, L)
+    idx = capi.Index(base, None, None)
+    idx.build_graph(aux, mon2.attach(capi.build_params(connect_enhance=0, **kw), every_batches=3))
+    assert [r[0] for r in mon2.reports] == [capi.MONITOR_BATCHES] * 2
+    assert [r[3:5] for r in mon2.reports] == [r[3:5] for r in mon.reports[:2]]
+    idx.close()
+
+
 def test_builder_argument_errors():
     base = synth.gaussian_matrix(1, 100, 8)
     idx = capi.Index(base, None, None)
@@ -312,7 +374,7 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     gt, _ = orc.bruteforce(base, q, k)
     formats.gt_write(work / "gt.bin", gt)
     (work / "config.json").write_text('{"batch": 256, "enhance_nap_batch": 1000, "search_start_nodes_num": 8, '
-                                      '"top_hit_num": 20000}')
+                                      '"top_hit_num": 20000, "test_search_frequency": 2}')
     cli = os.path.join(root, "coral_amd", "lib", "test_build_pipeline")
     args = [cli, "--data_type", "float", "--dist", "l2", "--dataset", "syn", "--base_data_path", str(work / "base.fbin"),
             "--sampled_query_data_path", str(work / "aux.fbin"), "--M_pjbp", "16", "--k", "24", "--CE", "1",
@@ -341,6 +403,17 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
     line = [l for l in r.stdout.splitlines() if l.startswith("test search:")][0]
     o24, _, os24, _ = orc.search_B(orc.Problem(base, nbrs, starts), q, 24, 512, start_order=WAVE64, nbr_order=WAVE64)
     assert "L 512, recall@24 " in line
+    # the searches of the same test queries while the graph grew (config.json "test_search", on by default; five
+    # batches, one search after those numbered 2 and 4): they left the graph as the unwatched construction above
+    # made it, and the last of them, on the finished graph, says what the driver's own closing search says
+    watch = [l for l in r.stdout.splitlines() if "Testing recall-" in l]
+    assert len(watch) == 5 and watch[0].startswith("[batches 768/1100]") and watch[1].startswith("[batches 1100/1100]")
+    assert watch[4].startswith("[graph complete 1100/1100]")
+    assert watch[2].startswith("[isolated nodes attached ") and watch[3].startswith("[most-hit nodes ")
+    recalls = [float(l.split("Testing recall-")[1].split("%")[0]) for l in watch]
+    assert recalls[0] < recalls[-1] and recalls[1] < recalls[2]  # (isolated nodes cannot be found before they are attached)
+    assert abs(recalls[-1] - float(line.split("recall@24 ")[1].split(" %")[0])) < 1e-3
+    assert abs(float(watch[-1].split("avg_hops-")[1].split(",")[0]) - os24[:, 0].sum() / Q) < 1e-2
     assert abs(float(line.split("recall@24 ")[1].split(" %")[0]) - 100.0 * orc.recall_hits(o24, gt24, 24) / (Q * 24)) < 1e-3
     assert abs(float(line.split("avg hops ")[1].split(",")[0]) - os24[:, 0].sum() / Q) < 1e-2
     # and the search driver on that directory
@@ -376,6 +449,8 @@ def test_build_driver_writes_the_index_directory_the_search_driver_reads(orc, tm
         a = build_args[:ce_at] + [ce] + build_args[ce_at + 1:] + staged
         r = subprocess.run(a, cwd=work / "cwd", capture_output=True, text=True, timeout=120)
         assert r.returncode == 0, r.stderr + r.stdout
+        marks = [l.split("]")[0].split(" ")[0] for l in r.stdout.splitlines() if "Testing recall-" in l]
+        assert marks == (["[batches", "[batches"] if ce == "0" else ["[isolated", "[most-hit", "[graph"])
         if ce == "0":
             nbrs0, _ = formats.graph_dir_read(work / "staged", n, 16, want_dists=True)
             assert (nbrs0[:, 0] < 0).sum() > 1000 and not np.array_equal(nbrs0, nbrs)
