@@ -429,7 +429,9 @@ def test_randomised_search_problems_equal_the_oracle(orc):
     """Seeded random sizes, widths, degrees, beam lengths, k, start ids, batch sizes, table sizes, workgroup
     shapes, ragged rows, repeated ids, tombstones, both metrics, both traversals (best-first in its three kernel
     forms): ids, distance bits and per-query counters equal the oracle's in the kernel's summation order."""
-    for c in range(120):
+    # (CORAL_RANDOM_FIRST / CORAL_RANDOM_CASES: other stretches of the same sequence of cases, for longer runs by hand)
+    first = int(os.environ.get("CORAL_RANDOM_FIRST", 0))
+    for c in range(first, first + int(os.environ.get("CORAL_RANDOM_CASES", 120))):
         rng = np.random.RandomState(5000 + c)
         n = int(rng.choice([300, 700, 2000, 5000, 12000]))
         dim = int(rng.choice([4, 8, 12, 16, 20, 32, 48, 64, 100, 128, 200, 256, 384, 512, 768, 1024]))
@@ -454,10 +456,8 @@ def test_randomised_search_problems_equal_the_oracle(orc):
             slots = -1  # the visited set as a bitmap of all ids in LDS
         ahead = int(rng.choice([0, 1, -1]))  # graph rows requested a chunk ahead: the library's choice, yes, no
         screen = int(rng.choice([0, 1, 2, -1])) if (policy == 0 and dim > 128) else 0
-        if screen == 2 and dim > 512:
-            screen = 1
         if screen == 1 and metric != "l2":
-            screen = 2 if dim <= 512 else -1
+            screen = 2
         print("case", dict(c=c, n=n, dim=dim, R=R, metric=metric, policy=policy, L=L, k=k, M=M, Q=Q, slots=slots,
                            threads=threads, rg=rg, dele=dele, dup=dup, wgs=wgs, tbl=tbl, big=big, ahead=ahead,
                            screen=screen),
@@ -485,12 +485,15 @@ def test_randomised_search_problems_equal_the_oracle(orc):
         if dele:
             idx.set_deleted(mask)
         longb = int(rng.choice([64, 128, 512]))  # insert buffer of the long-beam form of best-first
+        # the table of cells probed linearly, in buckets, or in buckets that several threads fill with one id at once
+        choices = int(rng.choice([0, 1, 3, 4])) if slots > 0 else 0
+        print("     ", dict(longb=longb, choices=choices), flush=True)
         for in_lds, packed, long_ in (((False, False, 0), (False, True, 0), (True, False, 0), (False, False, 1),
                                        (False, True, 1)) if policy == 1 else ((False, False, 0),)):
             idx.prepare(Q, L, visited_slots_log2=slots, threads=threads, workgroups=wgs, policy=policy,
                         best_first_in_lds=in_lds, best_first_packed=packed, best_first_table_log2=tbl,
                         beam_in_hbm=big, prefetch_rows=ahead, best_first_long=long_, best_first_buffer=longb,
-                        screening=screen)
+                        screening=screen, visited_choices=choices)
             ids, dists, _ = idx.search(q, k, L, policy=policy, have_delete=dele)
             assert np.array_equal(ids, oi) and dists.tobytes() == od.tobytes()
             assert np.array_equal(idx.query_counters(Q), os_)
