@@ -86,12 +86,21 @@ int ensure_stage(coral_index* idx, size_t rows) {
 // the index's current start ids, the hit count against the true neighbours, and the caller's report.  With
 // fresh_starts (the calls between batches, when the index has no entry points yet) the start ids are sampled first,
 // as the enhancement does for its own searches; they are replaced again before the build ends.
+int check_monitor(const coral_build_params* prm) {
+    const coral_build_monitor* m = prm->monitor;
+    if (!m || !m->report) return CORAL_OK;
+    if (!m->h_queries || !m->h_gt || m->Q < 1 || m->k < 1 || m->k > m->L || m->L > CORAL_MAX_BEAM)
+        return fail(CORAL_ERR_ARG, "build monitor: queries, true neighbours, Q >= 1 and 1 <= k <= L <= %d are needed",
+                    CORAL_MAX_BEAM);
+    if (prm->test_search_frequency < 0) return fail(CORAL_ERR_ARG, "test_search_frequency must not be negative");
+    return CORAL_OK;
+}
+
 int monitor_search(coral_index* idx, const coral_build_params* prm, int32_t phase, int64_t done, int64_t total,
                    bool fresh_starts) {
     const coral_build_monitor* m = prm->monitor;
     if (!m || !m->report) return CORAL_OK;
-    if (!m->h_queries || !m->h_gt || m->Q < 1 || m->k < 1 || m->k > m->L)
-        return fail(CORAL_ERR_ARG, "build monitor: queries, true neighbours, Q >= 1 and 1 <= k <= L are needed");
+    if (int rc = check_monitor(prm)) return rc;
     if (fresh_starts) {
         std::vector<int32_t> deg((size_t)idx->n), starts((size_t)prm->n_start);
         HIP_TRY(hipMemcpyAsync(deg.data(), idx->d_deg, (size_t)idx->n * sizeof(int32_t), hipMemcpyDeviceToHost, idx->stream));
@@ -342,6 +351,7 @@ int coral_build_connect_enhance(coral_index* idx, const coral_build_params* prm,
     if (prm->k_b < 1 || prm->k_b > prm->enhance_L) return fail(CORAL_ERR_ARG, "k_b must be in 1..enhance_L");
     if (prm->n_start < 1 || prm->enhance_search_batch < 1 || prm->enhance_nap_batch < 1)
         return fail(CORAL_ERR_ARG, "n_start and the enhancement batch sizes must be positive");
+    if (int rc = check_monitor(prm)) return rc;
     HIP_TRY(hipSetDevice(idx->device));
     hipStream_t st = idx->stream;
     const int64_t n = idx->n;
@@ -439,6 +449,7 @@ static int build_impl(coral_index* idx, const float* h_aux, const int32_t* h_clu
     if (A <= 0) return fail(CORAL_ERR_ARG, "no auxiliary queries");
     if (prm->batch <= 0) return fail(CORAL_ERR_ARG, "batch must be positive");
     if (prm->k_b > idx->n) return fail(CORAL_ERR_ARG, "k_b exceeds the number of base vectors");
+    if (int rc = check_monitor(prm)) return rc;
     coral_build_stats local{};
     coral_build_stats* S = stats ? stats : &local;
     *S = coral_build_stats{};

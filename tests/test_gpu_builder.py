@@ -320,6 +320,13 @@ def test_searches_during_a_build_report_and_change_nothing(orc):
         idx.build_test_search(bad.attach(capi.build_params(**kw)))
     assert e.value.code == capi.ERR_ARG
     idx.close()
+    idx = capi.Index(base, None, None)
+    with pytest.raises(capi.CoralError) as e:
+        idx.build_graph(aux, bad.attach(capi.build_params(**kw)))
+    assert e.value.code == capi.ERR_ARG and not bad.reports
+    with pytest.raises(capi.CoralError):  # nothing was begun
+        idx.get_graph(with_build_state=True)
+    idx.close()
     # without the enhancement there is no closing search (src/index_gpu.cpp:376: CE && test_search)
     mon2 = capi.Monitor(q, gt, L)
     idx = capi.Index(base, None, None)
