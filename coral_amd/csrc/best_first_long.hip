@@ -519,8 +519,9 @@ bfl_kernel_fn pick_rif(int chunks) {
 template <bool SCREEN, int WGS>
 bfl_kernel_fn pick_screen(int dim, bool packed) {
     const int chunks = dim / 4;
-    // 16 rows requested per wavefront before any is added up where that fits the registers, else 8
-    const bool wide = chunks > 16 && chunks <= 256;
+    // 16 rows requested per wavefront before any is added up where that fits the registers, else 8; with the
+    // screening few rows of a step are left to read in fp32, and the registers are worth more to its own requests
+    const bool wide = chunks > 16 && chunks <= 256 && !SCREEN;
     if (packed) return wide ? pick_rif<16, true, SCREEN, WGS>(chunks) : pick_rif<8, true, SCREEN, WGS>(chunks);
     return wide ? pick_rif<16, false, SCREEN, WGS>(chunks) : pick_rif<8, false, SCREEN, WGS>(chunks);
 }

@@ -658,6 +658,7 @@ int coral_search_prepare(coral_index* idx, int32_t Q, int32_t L, const coral_tun
         // 16 rows requested per wavefront before any is added up where that fits 128 registers without spilling; a
         // launch whose LDS leaves a CU eight wavefronts may as well use 256 registers per lane: all 32 rows of a step
         int rif = (chunks > 16 && chunks <= 256) ? 16 : 8;
+        if (idx->bf_screen != 0 && table_log2 == 0) rif = 8;  // (the screening leaves few rows to read in fp32)
         if (table_log2 && coral::best_first_wave_lds_bytes(L, 0, table_log2) * 12 > (size_t)kMaxLdsBytes && chunks > 16 &&
             chunks <= 64)
             rif = 32;
